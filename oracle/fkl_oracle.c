@@ -1,0 +1,397 @@
+/*
+ * fkl_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE (see fkl_oracle.h).
+ *
+ * Plain-C restatement of FKL's fused data-parallel path on its CPU backend.
+ * Reference paths are relative to the reference root; FK/ = include/fused_kernel/.
+ */
+#include "fkl_oracle.h"
+
+#include <math.h>
+#include <string.h>
+
+/* One value travelling through the chain: either uchar or float channels. */
+typedef struct {
+    int elem; /* FKLO_U8 / FKLO_F32 */
+    int cn;
+    float f[4];
+    uint8_t u[4];
+} fklo_val;
+
+/* ---- scalar helpers ---------------------------------------------------- */
+
+/* cxp::round, FK/core/constexpr_libs/constexpr_cmath.h:354-385: half away from
+ * zero (std::round at run time). Used on the host for letterbox sizes. */
+float fklo_round_half_away(float s) {
+    if (s != s || isinf(s) || s == 0.0f) return s;
+    const float a = s < 0.0f ? -s : s;
+    if (a >= 8388608.0f) return s;
+    const float t = (float)(int)a;
+    const float r = (a - t) >= 0.5f ? t + 1.0f : t;
+    return s < 0.0f ? -r : r;
+}
+
+/* cxp::banker_round, FK/core/constexpr_libs/constexpr_saturate.h:28-66:
+ * truncate |u|, look at the exact remainder, push odd ties up. */
+float fklo_banker_round(float u) {
+    if (u != u) return u;
+    const int neg = u < 0.0f;
+    const float a = neg ? -u : u;
+    if (a >= 9007199254740992.0f) return u;
+    long long i = (long long)a;
+    const float diff = a - (float)i;
+    if (diff > 0.5f) {
+        i += 1;
+    } else if (diff >= 0.5f) {
+        if (i % 2 != 0) i += 1;
+    }
+    const float r = (float)i;
+    return neg ? -r : r;
+}
+
+/* cxp::saturate_cast<uchar>(float), FK/core/constexpr_libs/constexpr_saturate.h:91-113
+ * via SaturateCast<I,O>, FK/algorithms/image_processing/saturate.h:25-36. */
+uint8_t fklo_saturate_cast_u8(float s) {
+    if (s != s) return 0;
+    const float r = fklo_banker_round(s);
+    if (r >= 255.0f) return 255;
+    if (r <= 0.0f) return 0;
+    return (uint8_t)r;
+}
+
+/* computeMatrix<Full, bt709, YCbCr2RGB, p8bit>, FK/algorithms/image_processing/itu_color.h:185-265.
+ * All arithmetic in binary32, same expression order. */
+void fklo_yuv2rgb_709_full_matrix(float m[9]) {
+    const float Kr = 0.2126f, Kb = 0.0722f;
+    const float Kg = 1.0f - Kr - Kb;
+    m[0] = 1.0f; m[1] = 0.0f;                           m[2] = 2.0f * (1.0f - Kr);
+    m[3] = 1.0f; m[4] = -2.0f * Kb * (1.0f - Kb) / Kg;  m[5] = -2.0f * Kr * (1.0f - Kr) / Kg;
+    m[6] = 1.0f; m[7] = 2.0f * (1.0f - Kb);             m[8] = 0.0f;
+}
+
+/* ConvertYUVToRGB<p8bit,Full,bt709>::exec, FK/algorithms/image_processing/color_conversion.h:150-174,
+ * MxVFloat3<UnaryType>::exec, FK/algorithms/basic_ops/algebraic.h:50-55: per row three
+ * products then (a + b) + c; chroma offset 128 (itu_color.h:120-121); no clamp. */
+void fklo_yuv2rgb_709_full(const uint8_t yuv[3], float rgb[3]) {
+    float m[9];
+    fklo_yuv2rgb_709_full_matrix(m);
+    const float v0 = (float)yuv[0];
+    const float v1 = (float)yuv[1] - 128.0f;
+    const float v2 = (float)yuv[2] - 128.0f;
+    for (int r = 0; r < 3; ++r) {
+        const float a = v0 * m[3 * r + 0];
+        const float b = v1 * m[3 * r + 1];
+        const float c = v2 * m[3 * r + 2];
+        rgb[r] = (a + b) + c;
+    }
+}
+
+/* InterpolateComplete<INTER_LINEAR>::exec, FK/algorithms/image_processing/interpolation.h:70-104:
+ * weights from the UNCLAMPED x2,y2; each weight one product of two differences;
+ * the four terms summed left to right. */
+float fklo_bilinear(float p00, float p10, float p01, float p11, float sx, float sy) {
+    const int x1 = (int)floorf(sx), y1 = (int)floorf(sy);
+    const int x2 = x1 + 1, y2 = y1 + 1;
+    const float w00 = ((float)x2 - sx) * ((float)y2 - sy);
+    const float w10 = (sx - (float)x1) * ((float)y2 - sy);
+    const float w01 = ((float)x2 - sx) * (sy - (float)y1);
+    const float w11 = (sx - (float)x1) * (sy - (float)y1);
+    return ((p00 * w00 + p10 * w10) + p01 * w01) + p11 * w11;
+}
+
+/* Resize<...>::build(backIOp, dstSize, bg) and compute_target_size,
+ * FK/algorithms/image_processing/resize.h:164-233 (PRESERVE_AR) and :266-278 (IGNORE_AR).
+ * Factors are computed in double on the host and narrowed once. */
+void fklo_compute_resize_params(int32_t src_w, int32_t src_h, int32_t dst_w, int32_t dst_h,
+                                int32_t ar, fklo_resize_params *out) {
+    out->dst_w = dst_w;
+    out->dst_h = dst_h;
+    if (ar == FKLO_IGNORE_AR) {
+        const double cfx = (double)dst_w / (double)src_w;
+        const double cfy = (double)dst_h / (double)src_h;
+        out->fx = (float)(1.0 / cfx);
+        out->fy = (float)(1.0 / cfy);
+        out->x1 = 0; out->y1 = 0; out->x2 = dst_w - 1; out->y2 = dst_h - 1;
+        return;
+    }
+    const float scale = (float)dst_h / (float)src_h;
+    int tw = (int)fklo_round_half_away(scale * (float)src_w);
+    int th = dst_h;
+    if (tw > dst_w) {
+        const float scale2 = (float)dst_w / (float)src_w;
+        tw = dst_w;
+        th = (int)fklo_round_half_away(scale2 * (float)src_h);
+    }
+    const double cfx = (double)tw / (double)src_w;
+    const double cfy = (double)th / (double)src_h;
+    out->fx = (float)(1.0 / cfx);
+    out->fy = (float)(1.0 / cfy);
+    out->x1 = (dst_w - tw) / 2;
+    out->y1 = (dst_h - th) / 2;
+    out->x2 = out->x1 + tw - 1;
+    out->y2 = out->y1 + th - 1;
+}
+
+/* ---- ops on values ----------------------------------------------------- */
+
+static float chan_as_float(const fklo_val *v, int c) {
+    return v->elem == FKLO_F32 ? v->f[c] : (float)v->u[c];
+}
+
+/* Add/Sub/Mul/Div<I,P,O,BinaryType>::exec, FK/algorithms/basic_ops/arithmetic.h:26-124 with the
+ * channel-wise operators of FK/core/utils/vector_utils.h:508-563 (uchar op float -> float);
+ * VectorReorder, FK/algorithms/basic_ops/vector_ops.h:43-56; Cast, FK/algorithms/basic_ops/cast.h:22-33. */
+static int apply_op(const fklo_op *op, fklo_val *v) {
+    switch (op->code) {
+    case FKLO_MUL: case FKLO_ADD: case FKLO_SUB: case FKLO_DIV: {
+        for (int c = 0; c < v->cn; ++c) {
+            const float a = chan_as_float(v, c), p = op->p[c];
+            float r;
+            if (op->code == FKLO_MUL) r = a * p;
+            else if (op->code == FKLO_ADD) r = a + p;
+            else if (op->code == FKLO_SUB) r = a - p;
+            else r = a / p;
+            v->f[c] = r;
+        }
+        v->elem = FKLO_F32;
+        return FKLO_OK;
+    }
+    case FKLO_REORDER: {
+        fklo_val t = *v;
+        for (int c = 0; c < v->cn; ++c) {
+            const int s = op->idx[c];
+            if (s < 0 || s >= v->cn) return FKLO_EINVAL;
+            v->f[c] = t.f[s];
+            v->u[c] = t.u[s];
+        }
+        return FKLO_OK;
+    }
+    case FKLO_SATCAST_U8: {
+        if (v->elem != FKLO_F32) return FKLO_ETYPE;
+        for (int c = 0; c < v->cn; ++c) v->u[c] = fklo_saturate_cast_u8(v->f[c]);
+        v->elem = FKLO_U8;
+        return FKLO_OK;
+    }
+    case FKLO_CAST_F32: {
+        if (v->elem == FKLO_U8) {
+            for (int c = 0; c < v->cn; ++c) v->f[c] = (float)v->u[c];
+            v->elem = FKLO_F32;
+        }
+        return FKLO_OK;
+    }
+    case FKLO_YUV2RGB_709_FULL: {
+        if (v->elem != FKLO_U8 || v->cn != 3) return FKLO_ETYPE;
+        fklo_yuv2rgb_709_full(v->u, v->f);
+        v->elem = FKLO_F32;
+        return FKLO_OK;
+    }
+    default:
+        return FKLO_EINVAL;
+    }
+}
+
+/* ---- the read stack ---------------------------------------------------- */
+
+/* PerThreadRead<_2D,T>::exec + PtrAccessor<_2D>::cr_point, FK/algorithms/basic_ops/memory_operations.h:26-67,
+ * FK/core/data/rawptr.h:202-213: address = data + y*pitch + x*sizeof(T).
+ * ReadYUV<NV12>::exec, FK/algorithms/image_processing/color_conversion.h:219-238: Y at (x,y) of the
+ * luma plane; (U,V) at element x>>1 of chroma row y>>1, chroma base = data + pitch*height. */
+static void read_source(const fklo_read *r, int x, int y, fklo_val *out) {
+    const uint8_t *base = (const uint8_t *)r->data;
+    if (r->kind == FKLO_READ_NV12) {
+        out->elem = FKLO_U8;
+        out->cn = 3;
+        out->u[0] = base[(int64_t)y * r->pitch + x];
+        const uint8_t *chroma = base + (int64_t)r->pitch * r->height + (int64_t)(y >> 1) * r->pitch;
+        out->u[1] = chroma[2 * (x >> 1) + 0];
+        out->u[2] = chroma[2 * (x >> 1) + 1];
+        return;
+    }
+    out->elem = r->elem;
+    out->cn = r->cn;
+    const uint8_t *row = base + (int64_t)y * r->pitch;
+    if (r->elem == FKLO_U8) {
+        const uint8_t *p = row + (int64_t)x * r->cn;
+        for (int c = 0; c < r->cn; ++c) out->u[c] = p[c];
+    } else {
+        const float *p = (const float *)row + (int64_t)x * r->cn;
+        for (int c = 0; c < r->cn; ++c) out->f[c] = p[c];
+    }
+}
+
+/* Crop<BackIOp>::exec, FK/algorithms/image_processing/crop.h:36-39: shift by the rect origin, no clipping;
+ * then whatever compute ops were fused into the read (FusedOperation, iop_fuser.h:99-106). */
+static int read_tap(const fklo_read *r, int x, int y, fklo_val *out) {
+    if (r->has_crop) {
+        x += r->crop[0];
+        y += r->crop[1];
+    }
+    read_source(r, x, y, out);
+    for (int i = 0; i < r->n_tap_ops; ++i) {
+        const int rc = apply_op(&r->tap_ops[i], out);
+        if (rc) return rc;
+    }
+    return FKLO_OK;
+}
+
+static void read_extent(const fklo_read *r, int *w, int *h) {
+    if (r->has_crop) { *w = r->crop[2]; *h = r->crop[3]; }
+    else { *w = r->width; *h = r->height; }
+}
+
+/* ResizeComplete<AR,...>::exec / exec_resize, FK/algorithms/image_processing/resize.h:86-98,117-123 and
+ * InterpolateComplete<INTER_LINEAR>::exec, interpolation.h:70-104. */
+static int read_resized(const fklo_read *r, const fklo_resize_params *rp, int x, int y, fklo_val *out) {
+    if (r->ar != FKLO_IGNORE_AR) {
+        if (!(x >= rp->x1 && x <= rp->x2 && y >= rp->y1 && y <= rp->y2)) {
+            /* params.defaultValue: float_<cn> of the tap type (resize.h:74) */
+            out->elem = FKLO_F32;
+            out->cn = r->kind == FKLO_READ_NV12 ? 3 : r->cn;
+            for (int c = 0; c < out->cn; ++c) out->f[c] = r->bg[c];
+            return FKLO_OK;
+        }
+        x -= rp->x1;
+        y -= rp->y1;
+    }
+    const float sx = (float)x * rp->fx;
+    const float sy = (float)y * rp->fy;
+    const int x1 = (int)floorf(sx), y1 = (int)floorf(sy);
+    const int x2 = x1 + 1, y2 = y1 + 1;
+    int sw, sh;
+    read_extent(r, &sw, &sh);
+    const int x2r = x2 < sw - 1 ? x2 : sw - 1;
+    const int y2r = y2 < sh - 1 ? y2 : sh - 1;
+    fklo_val t00, t10, t01, t11;
+    int rc;
+    if ((rc = read_tap(r, x1, y1, &t00))) return rc;
+    if ((rc = read_tap(r, x2r, y1, &t10))) return rc;
+    if ((rc = read_tap(r, x1, y2r, &t01))) return rc;
+    if ((rc = read_tap(r, x2r, y2r, &t11))) return rc;
+    out->elem = FKLO_F32;
+    out->cn = t00.cn;
+    for (int c = 0; c < t00.cn; ++c) {
+        out->f[c] = fklo_bilinear(chan_as_float(&t00, c), chan_as_float(&t10, c),
+                                  chan_as_float(&t01, c), chan_as_float(&t11, c), sx, sy);
+    }
+    return FKLO_OK;
+}
+
+/* ---- writers ----------------------------------------------------------- */
+
+/* PerThreadWrite<_2D,T>, TensorWrite<T>, TensorSplit<T>: FK/algorithms/basic_ops/memory_operations.h:84-107,
+ * 159-179, 181-212; PtrAccessor<_3D>::point, FK/core/data/rawptr.h:215-226 (plane stride =
+ * plane_pitch*color_planes with plane_pitch = pitch*height). */
+static int write_value(const fklo_write *w, int x, int y, int z, const fklo_val *v) {
+    if (v->elem != w->elem || v->cn != w->cn) return FKLO_ETYPE;
+    uint8_t *base = (uint8_t *)w->data;
+    const int64_t esz = w->elem == FKLO_U8 ? 1 : 4;
+    if (w->kind == FKLO_WRITE_2D) {
+        uint8_t *p = base + (int64_t)y * w->pitch + (int64_t)x * esz * w->cn;
+        if (w->elem == FKLO_U8) memcpy(p, v->u, (size_t)w->cn);
+        else memcpy(p, v->f, (size_t)w->cn * 4);
+        return FKLO_OK;
+    }
+    const int64_t plane_pitch = (int64_t)w->pitch * w->height;
+    uint8_t *row = base + plane_pitch * w->color_planes * z + (int64_t)y * w->pitch;
+    if (w->kind == FKLO_TENSOR_WRITE) {
+        uint8_t *p = row + (int64_t)x * esz * w->cn;
+        if (w->elem == FKLO_U8) memcpy(p, v->u, (size_t)w->cn);
+        else memcpy(p, v->f, (size_t)w->cn * 4);
+        return FKLO_OK;
+    }
+    if (w->kind == FKLO_TENSOR_SPLIT) {
+        const int64_t plane_px = (int64_t)w->width * w->height;
+        for (int c = 0; c < w->cn; ++c) {
+            uint8_t *p = row + ((int64_t)x + c * plane_px) * esz;
+            if (w->elem == FKLO_U8) *p = v->u[c];
+            else memcpy(p, &v->f[c], 4);
+        }
+        return FKLO_OK;
+    }
+    return FKLO_EINVAL;
+}
+
+/* ---- the loop ---------------------------------------------------------- */
+
+/* TransformDPP<CPU>::exec, FK/core/execution_model/data_parallel_patterns.h:271-283: for z, y, x over the
+ * active threads of the (fused) read; BatchRead picks plane z (batch_operations.h:205-212) and
+ * activeThreads = (max W, max H, BATCH) (batch_operations.h:401-424). Planes whose own geometry is smaller
+ * than the maximum are rejected here: the reference runs them unchecked, which reads outside the crop. */
+int fklo_execute(int32_t n_planes, const fklo_read *reads,
+                 int32_t n_ops, const fklo_op *ops,
+                 int32_t n_writes, const fklo_write *writes) {
+    if (n_planes < 1 || !reads || !writes) return FKLO_EINVAL;
+    if (n_writes != 1 && n_writes != n_planes) return FKLO_EINVAL;
+    int act_w = 0, act_h = 0;
+    for (int z = 0; z < n_planes; ++z) {
+        int w, h;
+        if (reads[z].has_resize) { w = reads[z].dst_w; h = reads[z].dst_h; }
+        else read_extent(&reads[z], &w, &h);
+        if (z == 0) { act_w = w; act_h = h; }
+        else if (w != act_w || h != act_h) return FKLO_EGEOM;
+    }
+    for (int z = 0; z < n_planes; ++z) {
+        const fklo_read *r = &reads[z];
+        const fklo_write *w = n_writes == 1 ? &writes[0] : &writes[z];
+        const int wz = n_writes == 1 ? z : 0;
+        fklo_resize_params rp;
+        if (r->has_resize) {
+            int sw, sh;
+            read_extent(r, &sw, &sh);
+            fklo_compute_resize_params(sw, sh, r->dst_w, r->dst_h, r->ar, &rp);
+        }
+        for (int y = 0; y < act_h; ++y) {
+            for (int x = 0; x < act_w; ++x) {
+                fklo_val v;
+                int rc = r->has_resize ? read_resized(r, &rp, x, y, &v) : read_tap(r, x, y, &v);
+                if (rc) return rc;
+                for (int i = 0; i < n_ops; ++i) {
+                    if ((rc = apply_op(&ops[i], &v))) return rc;
+                }
+                if ((rc = write_value(w, x, y, wz, &v))) return rc;
+            }
+        }
+    }
+    return FKLO_OK;
+}
+
+/* ---- synthetic inputs: std::mt19937 ------------------------------------ */
+
+void fklo_mt_seed(fklo_mt19937 *g, uint32_t seed) {
+    g->mt[0] = seed;
+    for (int i = 1; i < 624; ++i)
+        g->mt[i] = 1812433253u * (g->mt[i - 1] ^ (g->mt[i - 1] >> 30)) + (uint32_t)i;
+    g->idx = 624;
+}
+
+uint32_t fklo_mt_next(fklo_mt19937 *g) {
+    if (g->idx >= 624) {
+        for (int i = 0; i < 624; ++i) {
+            const uint32_t y = (g->mt[i] & 0x80000000u) | (g->mt[(i + 1) % 624] & 0x7fffffffu);
+            g->mt[i] = g->mt[(i + 397) % 624] ^ (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
+        }
+        g->idx = 0;
+    }
+    uint32_t y = g->mt[g->idx++];
+    y ^= y >> 11;
+    y ^= (y << 7) & 0x9d2c5680u;
+    y ^= (y << 15) & 0xefc60000u;
+    y ^= y >> 18;
+    return y;
+}
+
+void fklo_mt_fill_bytes(fklo_mt19937 *g, uint8_t *dst, uint64_t n) {
+    for (uint64_t i = 0; i < n; ++i) dst[i] = (uint8_t)(fklo_mt_next(g) & 0xFFu);
+}
+
+void fklo_mt_fill_unit_floats(fklo_mt19937 *g, float *dst, uint64_t n) {
+    for (uint64_t i = 0; i < n; ++i) dst[i] = (float)(fklo_mt_next(g) >> 8) * (1.0f / 8388608.0f) - 1.0f;
+}
+
+void fklo_mt_fill_range_floats(fklo_mt19937 *g, float *dst, uint64_t n, float a, float b) {
+    for (uint64_t i = 0; i < n; ++i)
+        dst[i] = a + ((float)(fklo_mt_next(g) >> 8) * (1.0f / 16777216.0f)) * (b - a);
+}
+
+void fklo_mt_fill_u32(fklo_mt19937 *g, uint32_t *dst, uint64_t n) {
+    for (uint64_t i = 0; i < n; ++i) dst[i] = fklo_mt_next(g);
+}

@@ -1,0 +1,241 @@
+// ref_chains.cpp -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// A thin C-ABI harness around the REFERENCE library's own CPU backend.  It is compiled against the
+// reference's headers where they lie on disk (see oracle/Makefile: -I$(FKL_REFERENCE)), never copied,
+// and the resulting shared object goes to oracle/_ref/ (git-ignored).  Each entry point spells one fused
+// chain with the reference's public API, runs it with TransformDPP<ParArch::CPU> on caller-owned host
+// buffers and returns.  Tests use it to validate the plain-C restatement in fkl_oracle.c and the HIP
+// kernels; bench.py may time it as the CPU baseline.
+//
+// Build flags: -std=c++20 -O2 -ffp-contract=off (contraction off makes the floats compiler independent).
+#include <fused_kernel/algorithms/basic_ops/memory_operations.h>
+#include <fused_kernel/algorithms/basic_ops/arithmetic.h>
+#include <fused_kernel/algorithms/basic_ops/cast.h>
+#include <fused_kernel/algorithms/image_processing/crop.h>
+#include <fused_kernel/algorithms/image_processing/color_conversion.h>
+#include <fused_kernel/algorithms/image_processing/resize.h>
+#include <fused_kernel/algorithms/image_processing/saturate.h>
+#include <fused_kernel/algorithms/image_processing/image.h>
+#include <fused_kernel/fused_kernel.h>
+
+#include <array>
+#include <cstdint>
+#include <utility>
+
+using namespace fk;
+using CpuDPP = TransformDPP<ParArch::CPU>;
+using CpuDPPTF = TransformDPP<ParArch::CPU, TF::ENABLED>;
+using CpuStream = Stream_<ParArch::CPU>;
+
+namespace {
+
+template <typename T>
+Ptr2D<T> wrap2d(const void* data, int w, int h, int pitch) {
+    return Ptr2D<T>(reinterpret_cast<T*>(const_cast<void*>(data)), uint(w), uint(h), uint(pitch), MemType::Host, 0);
+}
+
+template <size_t B>
+std::array<Rect, B> rects_from(const int32_t* r) {
+    std::array<Rect, B> a{};
+    for (size_t i = 0; i < B; ++i) a[i] = Rect(r[4 * i + 0], r[4 * i + 1], r[4 * i + 2], r[4 * i + 3]);
+    return a;
+}
+
+// README chain (benchmark configuration 1): uchar3 source, B crops, bilinear resize with PRESERVE_AR and a
+// background, Mul, Sub, SaturateCast, TensorWrite<uchar3>.
+template <size_t B>
+int crop_resize_par_u8(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                       const float* bg, const float* mul, const float* sub, uint8_t* out) {
+    CpuStream stream;
+    const auto in = wrap2d<uchar3>(src, w, h, pitch);
+    Tensor<uchar3> o(reinterpret_cast<uchar3*>(out), uint(dw), uint(dh), uint(B), 1, MemType::Host, 0);
+    const auto crops = rects_from<B>(rects);
+    executeOperations<CpuDPP>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
+        Crop<>::build(crops),
+        Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(dw, dh), float3{bg[0], bg[1], bg[2]}),
+        Mul<float3>::build(make_<float3>(mul[0], mul[1], mul[2])),
+        Sub<float3>::build(make_<float3>(sub[0], sub[1], sub[2])),
+        SaturateCast<float3, uchar3>::build(),
+        TensorWrite<uchar3>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
+// Benchmark configuration 3: BGR uchar3 source, B crops, bilinear resize IGNORE_AR, BGR->RGB, Sub, Div,
+// TensorSplit to planar float B x 3 x dh x dw.
+template <size_t B>
+int crop_resize_norm_split(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                           const float* sub, const float* div, float* out) {
+    CpuStream stream;
+    const auto in = wrap2d<uchar3>(src, w, h, pitch);
+    Tensor<float> o(out, uint(dw), uint(dh), uint(B), 3, MemType::Host, 0);
+    const auto crops = rects_from<B>(rects);
+    executeOperations<CpuDPP>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
+        Crop<>::build(crops),
+        Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
+        ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, float3, float3>::build(),
+        Sub<float3>::build(make_<float3>(sub[0], sub[1], sub[2])),
+        Div<float3>::build(make_<float3>(div[0], div[1], div[2])),
+        TensorSplit<float3>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
+// Benchmark configuration 4: B independent uchar3 images, per-image Mul and Add fused into each plane's
+// read, SaturateCast, B separate outputs in one launch.
+template <size_t B>
+int batch_muladd_sat(const uint8_t* const* srcs, int w, int h, int pitch, const float* mul, const float* add,
+                     uint8_t* const* outs, int out_pitch) {
+    CpuStream stream;
+    using PlaneIOp = decltype(PerThreadRead<ND::_2D, uchar3>::build(std::declval<RawPtr<ND::_2D, uchar3>>())
+                                  .then(Mul<uchar3, float3, float3>::build(float3{}))
+                                  .then(Add<float3>::build(float3{})));
+    std::array<PlaneIOp, B> planes{};
+    std::array<Ptr2D<uchar3>, B> outPtrs{};
+    for (size_t i = 0; i < B; ++i) {
+        const auto in = wrap2d<uchar3>(srcs[i], w, h, pitch);
+        planes[i] = PerThreadRead<ND::_2D, uchar3>::build(in.ptr())
+                        .then(Mul<uchar3, float3, float3>::build(make_<float3>(mul[3 * i], mul[3 * i + 1], mul[3 * i + 2])))
+                        .then(Add<float3>::build(make_<float3>(add[3 * i], add[3 * i + 1], add[3 * i + 2])));
+        outPtrs[i] = wrap2d<uchar3>(outs[i], w, h, out_pitch);
+    }
+    executeOperations<CpuDPP>(stream,
+        BatchRead<PlanePolicy::PROCESS_ALL>::build(planes),
+        SaturateCast<float3, uchar3>::build(),
+        PerThreadWrite<ND::_2D, uchar3>::build(outPtrs));
+    stream.sync();
+    return 0;
+}
+
+// Benchmark configuration 2: N alternating Add(0.5f)/Mul(1.0001f) on a float image, starting with Add.
+template <typename DPP, size_t... Is>
+void add_mul_chain(CpuStream& stream, const Ptr2D<float>& in, const Ptr2D<float>& out, float addv, float mulv,
+                   std::index_sequence<Is...>) {
+    const auto pick = [&](auto idx) {
+        if constexpr (decltype(idx)::value % 2 == 0) return Add<float>::build(addv);
+        else return Mul<float>::build(mulv);
+    };
+    executeOperations<DPP>(stream, PerThreadRead<ND::_2D, float>::build(in.ptr()),
+                           pick(std::integral_constant<size_t, Is>{})...,
+                           PerThreadWrite<ND::_2D, float>::build(out.ptr()));
+}
+
+template <size_t N>
+int add_mul_n(const float* in, int w, int h, int pitch, float addv, float mulv, float* out, int out_pitch, int tf) {
+    CpuStream stream;
+    const auto i = wrap2d<float>(in, w, h, pitch);
+    const auto o = wrap2d<float>(out, w, h, out_pitch);
+    if (tf) add_mul_chain<CpuDPPTF>(stream, i, o, addv, mulv, std::make_index_sequence<N>{});
+    else add_mul_chain<CpuDPP>(stream, i, o, addv, mulv, std::make_index_sequence<N>{});
+    stream.sync();
+    return 0;
+}
+
+// Integer-only chain: uchar3 source, B crops of one size, BGR->RGB on uchar3, TensorWrite<uchar3>.
+template <size_t B>
+int crop_swap_u8(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
+    CpuStream stream;
+    const auto in = wrap2d<uchar3>(src, w, h, pitch);
+    Tensor<uchar3> o(reinterpret_cast<uchar3*>(out), uint(rects[2]), uint(rects[3]), uint(B), 1, MemType::Host, 0);
+    const auto crops = rects_from<B>(rects);
+    // A batched Crop is only fused backwards by executeOperations when a Resize follows it, so this chain
+    // fuses the read explicitly with then().
+    executeOperations<CpuDPP>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr()).then(Crop<>::build(crops)),
+        ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, uchar3, uchar3>::build(),
+        TensorWrite<uchar3>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int fklref_crop_resize_par_u8_b5(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                                 const float* bg, const float* mul, const float* sub, uint8_t* out) {
+    return crop_resize_par_u8<5>(src, w, h, pitch, rects, dw, dh, bg, mul, sub, out);
+}
+
+int fklref_crop_resize_norm_split_b8(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw,
+                                     int dh, const float* sub, const float* div, float* out) {
+    return crop_resize_norm_split<8>(src, w, h, pitch, rects, dw, dh, sub, div, out);
+}
+int fklref_crop_resize_norm_split_b64(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw,
+                                      int dh, const float* sub, const float* div, float* out) {
+    return crop_resize_norm_split<64>(src, w, h, pitch, rects, dw, dh, sub, div, out);
+}
+
+int fklref_batch_muladd_sat_b4(const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,
+                               const float* add, uint8_t* const* outs, int out_pitch) {
+    return batch_muladd_sat<4>(srcs, w, h, pitch, mul, add, outs, out_pitch);
+}
+int fklref_batch_muladd_sat_b100(const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,
+                                 const float* add, uint8_t* const* outs, int out_pitch) {
+    return batch_muladd_sat<100>(srcs, w, h, pitch, mul, add, outs, out_pitch);
+}
+
+int fklref_add_mul_chain(const float* in, int w, int h, int pitch, int n_ops, float addv, float mulv, float* out,
+                         int out_pitch, int tf) {
+    switch (n_ops) {
+    case 1: return add_mul_n<1>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 2: return add_mul_n<2>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 3: return add_mul_n<3>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 10: return add_mul_n<10>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 50: return add_mul_n<50>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 100: return add_mul_n<100>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    default: return 1;
+    }
+}
+
+// Benchmark configuration 5: NV12 frame -> RGB (BT.709 full range) -> bilinear resize -> Mul by a scalar ->
+// TensorSplit to planar float 3 x dh x dw.  `nv12` is w x (h*3/2) bytes with row pitch `pitch`.
+int fklref_nv12_rgb_resize_split(const uint8_t* nv12, int w, int h, int pitch, int dw, int dh, float scale,
+                                 float* out) {
+    CpuStream stream;
+    const Ptr2D<uchar> data(const_cast<uchar*>(nv12), uint(w), uint(h + h / 2), uint(pitch), MemType::Host, 0);
+    const Image<PixelFormat::NV12> img(data, uint(w), uint(h));
+    Tensor<float> o(out, uint(dw), uint(dh), 1, 3, MemType::Host, 0);
+    executeOperations<CpuDPP>(stream,
+        ReadYUV<PixelFormat::NV12>::build(img.ptr()),
+        ConvertYUVToRGB<ColorDepth::p8bit, ColorRange::Full, ColorPrimitives::bt709>::build(),
+        Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
+        Mul<float3, float>::build(scale),
+        TensorSplit<float3>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
+int fklref_crop_swap_u8_b4(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
+    return crop_swap_u8<4>(src, w, h, pitch, rects, out);
+}
+
+// SaturateCast<float, uchar> over an array, one element at a time.
+int fklref_saturate_cast_u8(const float* in, int n, uint8_t* out) {
+    for (int i = 0; i < n; ++i) out[i] = SaturateCast<float, uchar>::exec(in[i]);
+    return 0;
+}
+
+// The constexpr BT.709 full-range YCbCr->RGB matrix the reference computes, row major.
+int fklref_yuv2rgb_709_full_matrix(float* m9) {
+    constexpr M3x3Float m = ccMatrix<ColorRange::Full, ColorPrimitives::bt709, ColorConversionDir::YCbCr2RGB, ColorDepth::p8bit>;
+    m9[0] = m.x.x; m9[1] = m.x.y; m9[2] = m.x.z;
+    m9[3] = m.y.x; m9[4] = m.y.y; m9[5] = m.y.z;
+    m9[6] = m.z.x; m9[7] = m.z.y; m9[8] = m.z.z;
+    return 0;
+}
+
+// Letterbox geometry and factors the reference computes for one crop size (PRESERVE_AR), read back from the
+// built IOp: out = {x1, y1, x2, y2}, f = {fx, fy}.
+int fklref_resize_params_par(int sw, int sh, int dw, int dh, int32_t* out4, float* f2) {
+    constexpr RawPtr<ND::_2D, uchar3> dummy{nullptr, {1u << 14, 1u << 14, 3u << 14}};
+    const auto back = PerThreadRead<ND::_2D, uchar3>::build(dummy).then(Crop<>::build(Rect(0, 0, sw, sh)));
+    const auto r = back.then(Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(dw, dh), float3{0.f, 0.f, 0.f}));
+    out4[0] = r.params.x1; out4[1] = r.params.y1; out4[2] = r.params.x2; out4[3] = r.params.y2;
+    f2[0] = r.params.src_conv_factors.x; f2[1] = r.params.src_conv_factors.y;
+    return 0;
+}
+
+} // extern "C"

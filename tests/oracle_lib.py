@@ -1,0 +1,328 @@
+"""ctypes bindings for the test-only CPU oracle (oracle/libfkl_oracle.so) and, when it has been built, the
+reference library's own CPU backend behind a C ABI (oracle/_ref/libfkl_ref.so).
+
+Only tests, the smoke check and the CPU-baseline leg of bench.py may import this module.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_SO = os.path.join(ROOT, "oracle", "libfkl_oracle.so")
+REF_SO = os.path.join(ROOT, "oracle", "_ref", "libfkl_ref.so")
+
+U8, F32 = 0, 1
+READ_2D, READ_NV12 = 0, 1
+PRESERVE_AR, IGNORE_AR = 0, 1
+MUL, ADD, SUB, DIV, REORDER, SATCAST_U8, CAST_F32, YUV2RGB_709_FULL = 1, 2, 3, 4, 5, 6, 7, 8
+WRITE_2D, TENSOR_WRITE, TENSOR_SPLIT = 0, 1, 2
+
+
+class Op(C.Structure):
+    _fields_ = [("code", C.c_int32), ("p", C.c_float * 4), ("idx", C.c_int32 * 4)]
+
+
+class Read(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int32), ("elem", C.c_int32), ("cn", C.c_int32),
+        ("width", C.c_int32), ("height", C.c_int32), ("pitch", C.c_int32),
+        ("data", C.c_void_p),
+        ("has_crop", C.c_int32), ("crop", C.c_int32 * 4),
+        ("has_resize", C.c_int32), ("dst_w", C.c_int32), ("dst_h", C.c_int32),
+        ("ar", C.c_int32), ("bg", C.c_float * 4),
+        ("n_tap_ops", C.c_int32), ("tap_ops", C.POINTER(Op)),
+    ]
+
+
+class Write(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int32), ("elem", C.c_int32), ("cn", C.c_int32), ("data", C.c_void_p),
+        ("width", C.c_int32), ("height", C.c_int32), ("planes", C.c_int32), ("color_planes", C.c_int32),
+        ("pitch", C.c_int32),
+    ]
+
+
+class ResizeParams(C.Structure):
+    _fields_ = [("dst_w", C.c_int32), ("dst_h", C.c_int32), ("fx", C.c_float), ("fy", C.c_float),
+                ("x1", C.c_int32), ("y1", C.c_int32), ("x2", C.c_int32), ("y2", C.c_int32)]
+
+
+class MT(C.Structure):
+    _fields_ = [("mt", C.c_uint32 * 624), ("idx", C.c_int32)]
+
+
+_oracle = None
+_ref = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is None:
+        lib = C.CDLL(ORACLE_SO)
+        lib.fklo_execute.restype = C.c_int
+        lib.fklo_execute.argtypes = [C.c_int32, C.POINTER(Read), C.c_int32, C.POINTER(Op), C.c_int32, C.POINTER(Write)]
+        lib.fklo_compute_resize_params.restype = None
+        lib.fklo_compute_resize_params.argtypes = [C.c_int32] * 5 + [C.POINTER(ResizeParams)]
+        lib.fklo_saturate_cast_u8.restype = C.c_uint8
+        lib.fklo_saturate_cast_u8.argtypes = [C.c_float]
+        lib.fklo_banker_round.restype = C.c_float
+        lib.fklo_banker_round.argtypes = [C.c_float]
+        lib.fklo_round_half_away.restype = C.c_float
+        lib.fklo_round_half_away.argtypes = [C.c_float]
+        lib.fklo_yuv2rgb_709_full_matrix.restype = None
+        lib.fklo_yuv2rgb_709_full_matrix.argtypes = [C.POINTER(C.c_float)]
+        lib.fklo_yuv2rgb_709_full.restype = None
+        lib.fklo_yuv2rgb_709_full.argtypes = [C.POINTER(C.c_uint8), C.POINTER(C.c_float)]
+        lib.fklo_bilinear.restype = C.c_float
+        lib.fklo_bilinear.argtypes = [C.c_float] * 6
+        lib.fklo_mt_seed.restype = None
+        lib.fklo_mt_seed.argtypes = [C.POINTER(MT), C.c_uint32]
+        lib.fklo_mt_next.restype = C.c_uint32
+        lib.fklo_mt_next.argtypes = [C.POINTER(MT)]
+        lib.fklo_mt_fill_bytes.restype = None
+        lib.fklo_mt_fill_bytes.argtypes = [C.POINTER(MT), C.c_void_p, C.c_uint64]
+        lib.fklo_mt_fill_unit_floats.restype = None
+        lib.fklo_mt_fill_unit_floats.argtypes = [C.POINTER(MT), C.c_void_p, C.c_uint64]
+        lib.fklo_mt_fill_range_floats.restype = None
+        lib.fklo_mt_fill_range_floats.argtypes = [C.POINTER(MT), C.c_void_p, C.c_uint64, C.c_float, C.c_float]
+        lib.fklo_mt_fill_u32.restype = None
+        lib.fklo_mt_fill_u32.argtypes = [C.POINTER(MT), C.c_void_p, C.c_uint64]
+        _oracle = lib
+    return _oracle
+
+
+def have_ref() -> bool:
+    return os.path.exists(REF_SO)
+
+
+def ref():
+    global _ref
+    if _ref is None:
+        lib = C.CDLL(REF_SO)
+        for name in dir(lib):
+            pass
+        _ref = lib
+    return _ref
+
+
+# ---- helpers to describe chains to the oracle -----------------------------------------------------------
+
+def op(code, p=(0, 0, 0, 0), idx=(0, 0, 0, 0)) -> Op:
+    o = Op()
+    o.code = code
+    pv = list(np.asarray(p, dtype=np.float32).reshape(-1))
+    pv = (pv + [pv[-1]] * 4)[:4] if len(pv) == 1 else (pv + [0.0] * 4)[:4]
+    for i in range(4):
+        o.p[i] = float(pv[i])
+        o.idx[i] = int(idx[i])
+    return o
+
+
+def ops_array(ops):
+    arr = (Op * max(1, len(ops)))()
+    for i, o in enumerate(ops):
+        arr[i] = o
+    return arr
+
+
+def _ptr(a: np.ndarray) -> int:
+    return a.ctypes.data
+
+
+def read_2d(a: np.ndarray, cn: int, crop=None, resize=None, ar=IGNORE_AR, bg=(0, 0, 0, 0), tap_ops=None,
+            pitch=None, width=None) -> Read:
+    """`a` is (H, W, cn) uint8/float32 or (H, W) for cn == 1 (possibly a padded row buffer if pitch given)."""
+    r = Read()
+    r.kind = READ_2D
+    r.elem = U8 if a.dtype == np.uint8 else F32
+    r.cn = cn
+    r.height = a.shape[0]
+    r.width = int(width) if width is not None else a.shape[1]
+    r.pitch = int(pitch) if pitch is not None else a.strides[0]
+    r.data = _ptr(a)
+    _fill_common(r, crop, resize, ar, bg, tap_ops)
+    return r
+
+
+def read_nv12(buf: np.ndarray, width: int, height: int, resize=None, ar=IGNORE_AR, tap_ops=None) -> Read:
+    r = Read()
+    r.kind = READ_NV12
+    r.elem = U8
+    r.cn = 3
+    r.width, r.height = width, height
+    r.pitch = buf.strides[0]
+    r.data = _ptr(buf)
+    _fill_common(r, None, resize, ar, (0, 0, 0, 0), tap_ops)
+    return r
+
+
+def _fill_common(r, crop, resize, ar, bg, tap_ops):
+    if crop is not None:
+        r.has_crop = 1
+        for i in range(4):
+            r.crop[i] = int(crop[i])
+    if resize is not None:
+        r.has_resize = 1
+        r.dst_w, r.dst_h = int(resize[0]), int(resize[1])
+        r.ar = ar
+    for i in range(min(4, len(bg))):
+        r.bg[i] = float(bg[i])
+    if tap_ops:
+        arr = ops_array(tap_ops)
+        r._keep = arr  # keep alive
+        r.n_tap_ops = len(tap_ops)
+        r.tap_ops = C.cast(arr, C.POINTER(Op))
+
+
+def write(kind, a: np.ndarray, cn: int, width: int, height: int, planes: int = 1, color_planes: int = 1,
+          pitch=None) -> Write:
+    w = Write()
+    w.kind = kind
+    w.elem = U8 if a.dtype == np.uint8 else F32
+    w.cn = cn
+    w.data = _ptr(a)
+    w.width, w.height, w.planes, w.color_planes = width, height, planes, color_planes
+    esz = 1 if a.dtype == np.uint8 else 4
+    if pitch is None:
+        pitch = width * esz * (1 if kind == TENSOR_SPLIT else cn)
+    w.pitch = int(pitch)
+    return w
+
+
+def execute(reads, ops, writes) -> None:
+    ra = (Read * len(reads))(*reads)
+    wa = (Write * len(writes))(*writes)
+    oa = ops_array(ops)
+    rc = oracle().fklo_execute(len(reads), ra, len(ops), oa, len(writes), wa)
+    if rc != 0:
+        raise RuntimeError(f"fklo_execute failed with code {rc}")
+
+
+# ---- the five benchmark chains, through the oracle ------------------------------------------------------
+
+def oracle_crop_resize_par_u8(src, rects, dst, bg, mul, sub):
+    dw, dh = dst
+    b = len(rects)
+    out = np.zeros((b, dh, dw, 3), np.uint8)
+    reads = [read_2d(src, 3, crop=rects[i], resize=dst, ar=PRESERVE_AR, bg=bg) for i in range(b)]
+    execute(reads, [op(MUL, mul), op(SUB, sub), op(SATCAST_U8)], [write(TENSOR_WRITE, out, 3, dw, dh, b, 1)])
+    return out
+
+
+def oracle_crop_resize_norm_split(src, rects, dst, sub, div):
+    dw, dh = dst
+    b = len(rects)
+    out = np.zeros((b, 3, dh, dw), np.float32)
+    reads = [read_2d(src, 3, crop=rects[i], resize=dst, ar=IGNORE_AR) for i in range(b)]
+    execute(reads, [op(REORDER, idx=(2, 1, 0, 0)), op(SUB, sub), op(DIV, div)],
+            [write(TENSOR_SPLIT, out, 3, dw, dh, b, 3)])
+    return out
+
+
+def oracle_batch_muladd_sat(srcs, mul, add):
+    b = len(srcs)
+    h, w = srcs[0].shape[:2]
+    outs = [np.zeros((h, w, 3), np.uint8) for _ in range(b)]
+    reads = [read_2d(srcs[i], 3, tap_ops=[op(MUL, mul[i]), op(ADD, add[i])]) for i in range(b)]
+    execute(reads, [op(SATCAST_U8)], [write(WRITE_2D, outs[i], 3, w, h) for i in range(b)])
+    return outs
+
+
+def oracle_add_mul_chain(src, n_ops, addv, mulv):
+    h, w = src.shape
+    out = np.zeros((h, w), np.float32)
+    ops = [op(ADD, [addv]) if i % 2 == 0 else op(MUL, [mulv]) for i in range(n_ops)]
+    execute([read_2d(src, 1)], ops, [write(WRITE_2D, out, 1, w, h)])
+    return out
+
+
+def oracle_nv12_rgb_resize_split(nv12, width, height, dst, scale):
+    dw, dh = dst
+    out = np.zeros((3, dh, dw), np.float32)
+    execute([read_nv12(nv12, width, height, resize=dst, tap_ops=[op(YUV2RGB_709_FULL)])],
+            [op(MUL, [scale])], [write(TENSOR_SPLIT, out, 3, dw, dh, 1, 3)])
+    return out
+
+
+def oracle_crop_swap_u8(src, rects):
+    b = len(rects)
+    cw, ch = int(rects[0][2]), int(rects[0][3])
+    out = np.zeros((b, ch, cw, 3), np.uint8)
+    reads = [read_2d(src, 3, crop=rects[i]) for i in range(b)]
+    execute(reads, [op(REORDER, idx=(2, 1, 0, 0))], [write(TENSOR_WRITE, out, 3, cw, ch, b, 1)])
+    return out
+
+
+# ---- the same chains through the reference's CPU backend ------------------------------------------------
+
+def _f32p(a):
+    return np.ascontiguousarray(a, dtype=np.float32).ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _i32p(a):
+    return np.ascontiguousarray(a, dtype=np.int32).ctypes.data_as(C.POINTER(C.c_int32))
+
+
+def ref_crop_resize_par_u8(src, rects, dst, bg, mul, sub):
+    assert len(rects) == 5
+    dw, dh = dst
+    out = np.zeros((5, dh, dw, 3), np.uint8)
+    rc = ref().fklref_crop_resize_par_u8_b5(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0],
+                                            _i32p(rects), dw, dh, _f32p(bg), _f32p(mul), _f32p(sub),
+                                            C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
+def ref_crop_resize_norm_split(src, rects, dst, sub, div):
+    b = len(rects)
+    fn = {8: "fklref_crop_resize_norm_split_b8", 64: "fklref_crop_resize_norm_split_b64"}[b]
+    dw, dh = dst
+    out = np.zeros((b, 3, dh, dw), np.float32)
+    rc = getattr(ref(), fn)(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], _i32p(rects), dw, dh,
+                            _f32p(sub), _f32p(div), C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
+def ref_batch_muladd_sat(srcs, mul, add):
+    b = len(srcs)
+    fn = {4: "fklref_batch_muladd_sat_b4", 100: "fklref_batch_muladd_sat_b100"}[b]
+    h, w = srcs[0].shape[:2]
+    outs = [np.zeros((h, w, 3), np.uint8) for _ in range(b)]
+    sp = (C.c_void_p * b)(*[_ptr(s) for s in srcs])
+    op_ = (C.c_void_p * b)(*[_ptr(o) for o in outs])
+    rc = getattr(ref(), fn)(sp, w, h, srcs[0].strides[0], _f32p(mul), _f32p(add), op_, outs[0].strides[0])
+    assert rc == 0
+    return outs
+
+
+def ref_add_mul_chain(src, n_ops, addv, mulv, tf=0):
+    h, w = src.shape
+    out = np.zeros((h, w), np.float32)
+    rc = ref().fklref_add_mul_chain(C.c_void_p(_ptr(src)), w, h, src.strides[0], n_ops, C.c_float(addv),
+                                    C.c_float(mulv), C.c_void_p(_ptr(out)), out.strides[0], tf)
+    assert rc == 0
+    return out
+
+
+def ref_nv12_rgb_resize_split(nv12, width, height, dst, scale):
+    dw, dh = dst
+    out = np.zeros((3, dh, dw), np.float32)
+    rc = ref().fklref_nv12_rgb_resize_split(C.c_void_p(_ptr(nv12)), width, height, nv12.strides[0], dw, dh,
+                                            C.c_float(scale), C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
+def ref_crop_swap_u8(src, rects):
+    assert len(rects) == 4
+    cw, ch = int(rects[0][2]), int(rects[0][3])
+    out = np.zeros((4, ch, cw, 3), np.uint8)
+    rc = ref().fklref_crop_swap_u8_b4(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0],
+                                      _i32p(rects), C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
