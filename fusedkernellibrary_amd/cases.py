@@ -1,0 +1,94 @@
+"""Python handle on the benchmark chains spelled with the C++ host API (tests/cases/fkl_cases.cpp).
+
+Each function takes torch CUDA tensors (device memory only -- torch is plumbing here), enqueues ONE fused kernel
+through executeOperations<TransformDPP<>> on torch's current stream and returns without synchronising.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import ROOT_DIR, lib
+
+CASES_SO = os.path.join(ROOT_DIR, "tests", "cases", "libfkl_cases.so")
+_cases = None
+
+
+def cases() -> C.CDLL:
+    global _cases
+    if _cases is None:
+        lib()  # the C-ABI library first, so its symbols resolve
+        if not os.path.exists(CASES_SO):
+            raise RuntimeError(f"{CASES_SO} is missing: run __graft_entry__.build()")
+        c = C.CDLL(CASES_SO)
+        c.fklcase_last_error.restype = C.c_char_p
+        _cases = c
+    return _cases
+
+
+def _ok(rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(cases().fklcase_last_error().decode())
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def _host(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def crop_resize_par_u8(src, rects, dst, bg, mul, sub, out):
+    """src (H,W,3) u8 cuda; rects (5,4) int32 host; out (5,dh,dw,3) u8 cuda."""
+    assert len(rects) == 5
+    r, b, m, s = _host(rects, np.int32), _host(bg, np.float32), _host(mul, np.float32), _host(sub, np.float32)
+    _ok(cases().fklcase_crop_resize_par_u8_b5(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0),
+                                              r.ctypes.data_as(C.c_void_p), int(dst[0]), int(dst[1]),
+                                              b.ctypes.data_as(C.c_void_p), m.ctypes.data_as(C.c_void_p),
+                                              s.ctypes.data_as(C.c_void_p), _p(out)))
+
+
+def crop_resize_norm_split(src, rects, dst, sub, div, out):
+    """src (H,W,3) u8 cuda; rects (B,4) int32 host, B in {8,64}; out (B,3,dh,dw) f32 cuda."""
+    fn = {8: "fklcase_crop_resize_norm_split_b8", 64: "fklcase_crop_resize_norm_split_b64"}[len(rects)]
+    r, s, d = _host(rects, np.int32), _host(sub, np.float32), _host(div, np.float32)
+    _ok(getattr(cases(), fn)(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0), r.ctypes.data_as(C.c_void_p),
+                             int(dst[0]), int(dst[1]), s.ctypes.data_as(C.c_void_p), d.ctypes.data_as(C.c_void_p), _p(out)))
+
+
+def batch_muladd_sat(srcs, mul, add, outs):
+    """srcs/outs: lists of B (H,W,3) u8 cuda tensors, B in {4,100}; mul/add (B,3) f32 host."""
+    b = len(srcs)
+    fn = {4: "fklcase_batch_muladd_sat_b4", 100: "fklcase_batch_muladd_sat_b100"}[b]
+    m, a = _host(mul, np.float32), _host(add, np.float32)
+    sp = (C.c_void_p * b)(*[s.data_ptr() for s in srcs])
+    op = (C.c_void_p * b)(*[o.data_ptr() for o in outs])
+    _ok(getattr(cases(), fn)(_stream(), sp, srcs[0].shape[1], srcs[0].shape[0], srcs[0].stride(0),
+                             m.ctypes.data_as(C.c_void_p), a.ctypes.data_as(C.c_void_p), op, outs[0].stride(0)))
+
+
+def add_mul_chain(src, n_ops, addv, mulv, out, tf=0):
+    """src/out (H,W) f32 cuda."""
+    _ok(cases().fklcase_add_mul_chain(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, int(n_ops),
+                                      C.c_float(float(addv)), C.c_float(float(mulv)), _p(out), out.stride(0) * 4, int(tf)))
+
+
+def nv12_rgb_resize_split(nv12, width, height, dst, scale, out):
+    """nv12 (H*3/2, W) u8 cuda; out (3,dh,dw) f32 cuda."""
+    _ok(cases().fklcase_nv12_rgb_resize_split(_stream(), _p(nv12), int(width), int(height), nv12.stride(0), int(dst[0]),
+                                              int(dst[1]), C.c_float(float(scale)), _p(out)))
+
+
+def crop_swap_u8(src, rects, out):
+    assert len(rects) == 4
+    r = _host(rects, np.int32)
+    _ok(cases().fklcase_crop_swap_u8_b4(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0),
+                                        r.ctypes.data_as(C.c_void_p), _p(out)))

@@ -1,0 +1,628 @@
+// fkd/ops.hpp -- the operations of the fused data-parallel path, as device-side static structs.
+//
+// Each operation is a type with
+//   * Params : plain aggregate holding its run-time values (this part is also seen by the host compiler,
+//              which fills it in; layouts therefore agree by construction),
+//   * name() : the C++ spelling of the type inside namespace fkd (host only) -- the chain signature,
+//   * exec() : the per-element body (device only).
+// Semantics follow the reference library's CPU backend operation by operation; the file:line given with
+// each operation is the reference definition it restates (FK/ = include/fused_kernel/ of the reference).
+//
+// Floating point: the device code is built with -ffp-contract=off and HIP's default correctly rounded
+// fp32 division, so every + - * / below is one IEEE-754 binary32 rounding, as on the CPU backend.
+#pragma once
+
+#include "types.hpp"
+
+namespace fkd {
+
+enum : int { PRESERVE_AR = 0, IGNORE_AR = 1 };
+
+#if defined(FKD_HOST_NAMES)
+#define FKD_NAME(expr) static std::string name() { return expr; }
+inline std::string istr(long long v) { return std::to_string(v); }
+#else
+#define FKD_NAME(expr)
+#endif
+
+#if defined(FKD_DEVICE_CODE)
+namespace detail {
+
+template <class T> FKD_DEV T load_elem(const T* p) {
+    T v;
+    if constexpr (cn_v<T> == 1) {
+        v = *p;
+    } else {
+        const base_t<T>* b = reinterpret_cast<const base_t<T>*>(p);
+        chan<0>(v) = b[0];
+        chan<1>(v) = b[1];
+        if constexpr (cn_v<T> > 2) chan<2>(v) = b[2];
+        if constexpr (cn_v<T> > 3) chan<3>(v) = b[3];
+    }
+    return v;
+}
+template <class T> FKD_DEV void store_elem(T* p, const T& v) {
+    if constexpr (cn_v<T> == 1) {
+        *p = v;
+    } else {
+        base_t<T>* b = reinterpret_cast<base_t<T>*>(p);
+        b[0] = chan<0>(v);
+        b[1] = chan<1>(v);
+        if constexpr (cn_v<T> > 2) b[2] = chan<2>(v);
+        if constexpr (cn_v<T> > 3) b[3] = chan<3>(v);
+    }
+}
+
+template <int WORDS> struct alignas(4) Words { u32 w[WORDS]; };
+
+// V consecutive elements starting at p.  When the run is a whole number of dwords and p is dword aligned the
+// run moves as one wide access per <= 16 bytes (global_load_dwordx3 for four uchar3, dwordx4 for four floats),
+// which consecutive lanes make contiguous; otherwise element by element.
+template <class T, int V> FKD_DEV void load_run(const T* p, T (&out)[V]) {
+    constexpr int BYTES = int(sizeof(T)) * V;
+    if constexpr (V > 1 && BYTES % 4 == 0) {
+        if ((reinterpret_cast<uintptr_t>(p) & 3u) == 0) {
+            constexpr int W = BYTES / 4;
+            Words<W> w;
+            const Words<(W > 4 ? 4 : W)>* src = reinterpret_cast<const Words<(W > 4 ? 4 : W)>*>(p);
+            if constexpr (W <= 4) {
+                w = *reinterpret_cast<const Words<W>*>(p);
+            } else {
+                static_assert(W % 4 == 0, "wide runs are multiples of 16 bytes");
+#pragma unroll
+                for (int i = 0; i < W / 4; ++i) {
+                    const Words<4> t = src[i];
+                    w.w[4 * i + 0] = t.w[0]; w.w[4 * i + 1] = t.w[1]; w.w[4 * i + 2] = t.w[2]; w.w[4 * i + 3] = t.w[3];
+                }
+            }
+            __builtin_memcpy(&out[0], &w, BYTES);
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) out[i] = load_elem(p + i);
+}
+
+template <class T, int V> FKD_DEV void store_run(T* p, const T (&in)[V]) {
+    constexpr int BYTES = int(sizeof(T)) * V;
+    if constexpr (V > 1 && BYTES % 4 == 0) {
+        if ((reinterpret_cast<uintptr_t>(p) & 3u) == 0) {
+            constexpr int W = BYTES / 4;
+            Words<W> w;
+            __builtin_memcpy(&w, &in[0], BYTES);
+            if constexpr (W <= 4) {
+                *reinterpret_cast<Words<W>*>(p) = w;
+            } else {
+                static_assert(W % 4 == 0, "wide runs are multiples of 16 bytes");
+                Words<4>* dst = reinterpret_cast<Words<4>*>(p);
+#pragma unroll
+                for (int i = 0; i < W / 4; ++i) {
+                    Words<4> t;
+                    t.w[0] = w.w[4 * i + 0]; t.w[1] = w.w[4 * i + 1]; t.w[2] = w.w[4 * i + 2]; t.w[3] = w.w[4 * i + 3];
+                    dst[i] = t;
+                }
+            }
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) store_elem(p + i, in[i]);
+}
+
+template <class T> FKD_DEV const T* row_ptr(const T* data, u32 pitch, int x, int y) {
+    return reinterpret_cast<const T*>(reinterpret_cast<const char*>(data) + size_t(y) * pitch) + x;
+}
+template <class T> FKD_DEV T* row_ptr(T* data, u32 pitch, int x, int y) {
+    return reinterpret_cast<T*>(reinterpret_cast<char*>(data) + size_t(y) * pitch) + x;
+}
+
+} // namespace detail
+#endif // FKD_DEVICE_CODE
+
+// ===================================================================================================
+// Compute operations: In -> Out
+// ===================================================================================================
+
+// Add/Sub/Mul/Div<I,P,O,BinaryType>::exec: FK/algorithms/basic_ops/arithmetic.h:26-124, evaluated per channel
+// with the usual C++ promotions (FK/core/utils/vector_utils.h:508-563); a scalar P is broadcast.
+#define FKD_BINARY_OP(NAME, EXPR)                                                                         \
+    template <class I, class P, class O> struct NAME {                                                    \
+        using In = I; using Out = O;                                                                      \
+        struct Params { P v; };                                                                           \
+        FKD_NAME(#NAME "<" + type_name<I>() + "," + type_name<P>() + "," + type_name<O>() + ">")       \
+        FKD_DEV static O exec(const I& a, const Params& p) {                                              \
+            return map2<O>(a, p.v, [](auto x, auto y) { return static_cast<base_t<O>>(EXPR); });          \
+        }                                                                                                 \
+    };
+FKD_BINARY_OP(Add, x + y)
+FKD_BINARY_OP(Sub, x - y)
+FKD_BINARY_OP(Mul, x * y)
+FKD_BINARY_OP(Div, x / y)
+#undef FKD_BINARY_OP
+
+// Cast<I,O>: per-channel static_cast.  FK/algorithms/basic_ops/cast.h:22-33.
+template <class I, class O> struct Cast {
+    using In = I; using Out = O; using Params = Empty;
+    FKD_NAME("Cast<" + type_name<I>() + "," + type_name<O>() + ">")
+    FKD_DEV static O exec(const I& a, const Params&) {
+        return map1<O>(a, [](auto x) { return static_cast<base_t<O>>(x); });
+    }
+};
+
+// VectorReorder<T,i0,i1,i2,i3>: out[c] = in[idx[c]] (BGR<->RGB is 2,1,0).  FK/algorithms/basic_ops/vector_ops.h:43-56,
+// reached through ColorConversion<COLOR_BGR2RGB,...>, FK/algorithms/image_processing/color_conversion.h:472-476.
+template <class T, int I0, int I1, int I2 = 2, int I3 = 3> struct Reorder {
+    using In = T; using Out = T; using Params = Empty;
+    FKD_NAME("Reorder<" + type_name<T>() + "," + istr(I0) + "," + istr(I1) + "," + istr(I2) + "," + istr(I3) + ">")
+    FKD_DEV static T exec(const T& a, const Params&) {
+        T o;
+        chan<0>(o) = chan<I0>(a);
+        chan<1>(o) = chan<I1>(a);
+        if constexpr (cn_v<T> > 2) chan<2>(o) = chan<I2>(a);
+        if constexpr (cn_v<T> > 3) chan<3>(o) = chan<I3>(a);
+        return o;
+    }
+};
+
+// SaturateCast<I,O>: FK/algorithms/image_processing/saturate.h:25-36 -> cxp::saturate_cast,
+// FK/core/constexpr_libs/constexpr_saturate.h:68-150.  float -> integer: NaN -> 0, round half to even,
+// clamp; integer -> integer: clamp; float -> float / widening: plain cast.
+template <class I, class O> struct SaturateCast {
+    using In = I; using Out = O; using Params = Empty;
+    FKD_NAME("SaturateCast<" + type_name<I>() + "," + type_name<O>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    template <class D> struct Lim {
+        static constexpr bool is_signed = D(-1) < D(0);
+        static constexpr long long hi = is_signed ? (long long)((1ull << (8 * sizeof(D) - 1)) - 1)
+                                                  : (long long)(sizeof(D) >= 8 ? ~0ull >> 1 : (1ull << (8 * (sizeof(D) % 8))) - 1);
+        static constexpr long long lo = is_signed ? -(long long)(1ull << (8 * sizeof(D) - 1)) : 0ll;
+    };
+    template <class S, class D> FKD_DEV static D sat(S s) {
+        if constexpr (__is_same(S, D)) {
+            return s;
+        } else if constexpr (__is_floating_point(S) && __is_integral(D)) {
+            if (s != s) return D(0);
+            S r;  // round half to even under the default rounding mode (v_rndne_f32 / v_rndne_f64)
+            if constexpr (sizeof(S) == 4) r = __builtin_rintf(s); else r = __builtin_rint(s);
+            if (r >= S(Lim<D>::hi)) return D(Lim<D>::hi);
+            if (r <= S(Lim<D>::lo)) return D(Lim<D>::lo);
+            return static_cast<D>(r);
+        } else if constexpr (__is_integral(S) && __is_integral(D)) {
+            const long long v = (long long)s;
+            return v > Lim<D>::hi ? D(Lim<D>::hi) : (v < Lim<D>::lo ? D(Lim<D>::lo) : D(s));
+        } else {
+            return static_cast<D>(s);
+        }
+    }
+#endif
+    FKD_DEV static O exec(const I& a, const Params&) {
+#if defined(FKD_DEVICE_CODE)
+        return map1<O>(a, [](auto x) { return sat<decltype(x), base_t<O>>(x); });
+#else
+        (void)a; return O{};
+#endif
+    }
+};
+
+// ConvertYUVToRGB<p8bit, Full, bt709>: FK/algorithms/image_processing/color_conversion.h:150-174 with the
+// constexpr matrix of FK/algorithms/image_processing/itu_color.h:185-265 (all binary32) and
+// MxVFloat3<UnaryType>, FK/algorithms/basic_ops/algebraic.h:42-56: per row three products, (a+b)+c; no clamp.
+struct YUV2RGB709Full8 {
+    using In = Vec<u8, 3>; using Out = Vec<f32, 3>; using Params = Empty;
+    FKD_NAME("YUV2RGB709Full8")
+    FKD_DEV static Out exec(const In& a, const Params&) {
+        constexpr f32 Kr = 0.2126f, Kb = 0.0722f;
+        constexpr f32 Kg = 1.0f - Kr - Kb;
+        constexpr f32 m00 = 1.0f, m01 = 0.0f, m02 = 2.0f * (1.0f - Kr);
+        constexpr f32 m10 = 1.0f, m11 = -2.0f * Kb * (1.0f - Kb) / Kg, m12 = -2.0f * Kr * (1.0f - Kr) / Kg;
+        constexpr f32 m20 = 1.0f, m21 = 2.0f * (1.0f - Kb), m22 = 0.0f;
+        const f32 y = f32(a.x), u = f32(a.y) - 128.0f, v = f32(a.z) - 128.0f;
+        Out o;
+        o.x = (y * m00 + u * m01) + v * m02;
+        o.y = (y * m10 + u * m11) + v * m12;
+        o.z = (y * m20 + u * m21) + v * m22;
+        return o;
+    }
+};
+
+// Fold of compute operations over a value, left to right.  FK/core/execution_model/data_parallel_patterns.h:75-78.
+template <class... Ops> struct OpList {
+    using Params = Tup<typename Ops::Params...>;
+#if defined(FKD_HOST_NAMES)
+    static std::string names() { std::string s; ((s += "," + Ops::name()), ...); return s; }
+#endif
+};
+template <class In, class... Ops> struct FoldOut { using type = In; };
+template <class In, class Op, class... Rest> struct FoldOut<In, Op, Rest...> {
+    using type = typename FoldOut<typename Op::Out, Rest...>::type;
+    using first_in = typename Op::In;
+};
+#if defined(FKD_DEVICE_CODE)
+template <class V> FKD_DEV V fold(const V& v, const Tup<>&) { return v; }
+template <class Op, class... Rest, class V>
+FKD_DEV auto fold(const V& v, const Tup<typename Op::Params, typename Rest::Params...>& p) {
+    static_assert(__is_same(V, typename Op::In), "operation input type does not match the value it receives");
+    if constexpr (sizeof...(Rest) == 0) return Op::exec(v, p.head);
+    else return fold<Rest...>(Op::exec(v, p.head), p.tail);
+}
+#endif
+
+// A run of compute operations packaged as one (host side: FusedOperation of compute IOps).
+template <class... Ops> struct FusedCompute {
+    using In = typename FoldOut<void, Ops...>::first_in;
+    using Out = typename FoldOut<In, Ops...>::type;
+    using Params = Tup<typename Ops::Params...>;
+    FKD_NAME("FusedCompute<" + OpList<Ops...>::names().substr(1) + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static Out exec(const In& a, const Params& p) { return fold<Ops...>(a, p); }
+#endif
+};
+
+// ===================================================================================================
+// Read operations: (x, y, z) -> Out.  width()/height() give the extent a consumer may address.
+// ===================================================================================================
+
+// PerThreadRead<_2D,T>: FK/algorithms/basic_ops/memory_operations.h:26-67, addressing FK/core/data/rawptr.h:202-213.
+template <class T> struct Read2D {
+    using Out = T;
+    using Params = RawPtr2D<const T>;
+    static constexpr bool kStageable = true;
+    FKD_NAME("Read2D<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return int(p.width); }
+    FKD_DEV static int height(const Params& p) { return int(p.height); }
+    FKD_DEV static T exec(int x, int y, int, const Params& p) {
+        return detail::load_elem(detail::row_ptr(p.data, p.pitch, x, y));
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int, const Params& p, T (&out)[V]) {
+        detail::load_run<T, V>(detail::row_ptr(p.data, p.pitch, x, y), out);
+    }
+    // Staging hooks: the element as it lies in memory, and what the consumer sees of it.
+    using Raw = T;
+    FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
+    FKD_DEV static T finish(const Raw& r, const Params&) { return r; }
+#endif
+};
+
+// TensorRead<T> / PerThreadRead<_3D,T>: FK/algorithms/basic_ops/memory_operations.h:124-157,
+// addressing FK/core/data/rawptr.h:215-226.
+template <class T> struct Read3D {
+    using Out = T;
+    using Params = RawPtr3D<const T>;
+    static constexpr bool kStageable = false;
+    FKD_NAME("Read3D<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return int(p.width); }
+    FKD_DEV static int height(const Params& p) { return int(p.height); }
+    FKD_DEV static const T* plane(const Params& p, int z) {
+        return reinterpret_cast<const T*>(reinterpret_cast<const char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z);
+    }
+    FKD_DEV static T exec(int x, int y, int z, const Params& p) {
+        return detail::load_elem(detail::row_ptr(plane(p, z), p.pitch, x, y));
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, T (&out)[V]) {
+        detail::load_run<T, V>(detail::row_ptr(plane(p, z), p.pitch, x, y), out);
+    }
+#endif
+};
+
+// ReadYUV<NV12>: FK/algorithms/image_processing/color_conversion.h:219-238.  Y from the luma plane, (U,V) from
+// element x>>1 of chroma row y>>1; chroma base = data + pitch*height.
+struct ReadNV12 {
+    using Out = Vec<u8, 3>;
+    using Params = RawNV12;
+    static constexpr bool kStageable = true;
+    FKD_NAME("ReadNV12")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return int(p.width); }
+    FKD_DEV static int height(const Params& p) { return int(p.height); }
+    FKD_DEV static Out exec(int x, int y, int, const Params& p) {
+        Out o;
+        o.x = p.data[size_t(y) * p.pitch + x];
+        const u8* c = p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch + 2 * (x >> 1);
+        o.y = c[0];
+        o.z = c[1];
+        return o;
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i] = exec(x + i, y, z, p);
+    }
+    using Raw = Out;
+    FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
+    FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
+#endif
+};
+
+// Crop<BackIOp>: FK/algorithms/image_processing/crop.h:36-39.  Shifts by the rectangle origin, drops z,
+// clips nothing.
+template <class Back> struct Crop {
+    using Out = typename Back::Out;
+    struct Params { i32 x, y, w, h; typename Back::Params back; };
+    static constexpr bool kStageable = Back::kStageable;
+    FKD_NAME("Crop<" + Back::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return p.w; }
+    FKD_DEV static int height(const Params& p) { return p.h; }
+    FKD_DEV static Out exec(int x, int y, int, const Params& p) { return Back::exec(x + p.x, y + p.y, 0, p.back); }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Out (&out)[V]) {
+        Back::template exec_row<V>(x + p.x, y + p.y, 0, p.back, out);
+    }
+    using Raw = typename Back::Raw;
+    FKD_DEV static Raw exec_raw(int x, int y, int, const Params& p) { return Back::exec_raw(x + p.x, y + p.y, 0, p.back); }
+    FKD_DEV static Out finish(const Raw& r, const Params& p) { return Back::finish(r, p.back); }
+#endif
+};
+
+// FusedOperation<Read..., compute...> used as a Read: FK/core/execution_model/operation_model/fused_operation.h
+// as produced by Fuser::fuse, FK/core/execution_model/operation_model/iop_fuser.h:99-106.
+template <class Back, class... Ops> struct FusedRead {
+    using Out = typename FoldOut<typename Back::Out, Ops...>::type;
+    struct Params { typename Back::Params back; Tup<typename Ops::Params...> ops; };
+    static constexpr bool kStageable = Back::kStageable;
+    FKD_NAME("FusedRead<" + Back::name() + OpList<Ops...>::names() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
+    FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        return fold<Ops...>(Back::exec(x, y, z, p.back), p.ops);
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+        typename Back::Out t[V];
+        Back::template exec_row<V>(x, y, z, p.back, t);
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i] = fold<Ops...>(t[i], p.ops);
+    }
+    using Raw = typename Back::Raw;
+    FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return Back::exec_raw(x, y, z, p.back); }
+    FKD_DEV static Out finish(const Raw& r, const Params& p) { return fold<Ops...>(Back::finish(r, p.back), p.ops); }
+#endif
+};
+
+// ResizeComplete<AR, Ternary<InterpolateComplete<INTER_LINEAR, Back>>>:
+// FK/algorithms/image_processing/resize.h:86-98,117-123 (letterbox test, source coordinate = index * factor, no
+// half-pixel offset) and FK/algorithms/image_processing/interpolation.h:70-104 (floor, clamp of x2/y2 only,
+// weights from the unclamped x2/y2, four terms summed left to right).  Factors and letterbox rectangle are
+// computed on the host (resize.h:164-233).
+template <int AR, class Back> struct ResizeLinear {
+    using Src = typename Back::Out;
+    using Out = vec_t<f32, cn_v<Src>>;
+    struct Params {
+        i32 dst_w, dst_h;
+        f32 fx, fy;
+        i32 x1, y1, x2, y2;
+        Out bg;
+        typename Back::Params back;
+    };
+    static constexpr bool kStageable = false;
+    static constexpr int kAR = AR;
+    using BackOp = Back;
+    FKD_NAME("ResizeLinear<" + istr(AR) + "," + Back::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return p.dst_w; }
+    FKD_DEV static int height(const Params& p) { return p.dst_h; }
+
+    struct Taps { int x1, y1, x2r, y2r; f32 w00, w10, w01, w11; };
+    FKD_DEV static Taps taps(int x, int y, const Params& p, int sw, int sh) {
+        const f32 sx = f32(x) * p.fx;
+        const f32 sy = f32(y) * p.fy;
+        Taps t;
+        t.x1 = int(__builtin_floorf(sx));
+        t.y1 = int(__builtin_floorf(sy));
+        const int x2 = t.x1 + 1, y2 = t.y1 + 1;
+        t.x2r = x2 < sw - 1 ? x2 : sw - 1;
+        t.y2r = y2 < sh - 1 ? y2 : sh - 1;
+        const f32 ax = f32(x2) - sx, bx = sx - f32(t.x1);
+        const f32 ay = f32(y2) - sy, by = sy - f32(t.y1);
+        t.w00 = ax * ay; t.w10 = bx * ay; t.w01 = ax * by; t.w11 = bx * by;
+        return t;
+    }
+    FKD_DEV static Out blend(const Src& a, const Src& b, const Src& c, const Src& d, const Taps& t) {
+        Out o;
+        auto one = [&](auto pa, auto pb, auto pc, auto pd) {
+            return ((f32(pa) * t.w00 + f32(pb) * t.w10) + f32(pc) * t.w01) + f32(pd) * t.w11;
+        };
+        chan<0>(o) = one(chan<0>(a), chan<0>(b), chan<0>(c), chan<0>(d));
+        if constexpr (cn_v<Src> > 1) chan<1>(o) = one(chan<1>(a), chan<1>(b), chan<1>(c), chan<1>(d));
+        if constexpr (cn_v<Src> > 2) chan<2>(o) = one(chan<2>(a), chan<2>(b), chan<2>(c), chan<2>(d));
+        if constexpr (cn_v<Src> > 3) chan<3>(o) = one(chan<3>(a), chan<3>(b), chan<3>(c), chan<3>(d));
+        return o;
+    }
+    FKD_DEV static bool inside(int x, int y, const Params& p) {
+        if constexpr (AR == IGNORE_AR) return true;
+        else return x >= p.x1 && x <= p.x2 && y >= p.y1 && y <= p.y2;
+    }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        if (!inside(x, y, p)) return p.bg;
+        if constexpr (AR != IGNORE_AR) { x -= p.x1; y -= p.y1; }
+        const Taps t = taps(x, y, p, Back::width(p.back), Back::height(p.back));
+        const Src a = Back::exec(t.x1, t.y1, z, p.back);
+        const Src b = Back::exec(t.x2r, t.y1, z, p.back);
+        const Src c = Back::exec(t.x1, t.y2r, z, p.back);
+        const Src d = Back::exec(t.x2r, t.y2r, z, p.back);
+        return blend(a, b, c, d, t);
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i] = exec(x + i, y, z, p);
+    }
+#endif
+};
+
+// BatchRead<PROCESS_ALL, N, Op>: FK/core/execution_model/operation_model/batch_operations.h:164-219.  Plane z
+// uses its own parameter set; z is the workgroup's grid-z index, so the selection is wave uniform.
+template <int N, class PlaneOp> struct BatchRead {
+    using Out = typename PlaneOp::Out;
+    using Plane = PlaneOp;
+    static constexpr int kBatch = N;
+    struct Params { typename PlaneOp::Params plane[N]; };
+    static constexpr bool kStageable = false;
+    FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+        PlaneOp::template exec_row<V>(x, y, z, p.plane[z], out);
+    }
+#endif
+};
+
+// BatchRead<CONDITIONAL_WITH_DEFAULT, N, Op>: batch_operations.h:221-281.  Planes >= used yield a default.
+template <int N, class PlaneOp> struct BatchReadDefault {
+    using Out = typename PlaneOp::Out;
+    using Plane = PlaneOp;
+    static constexpr int kBatch = N;
+    struct Params { typename PlaneOp::Params plane[N]; i32 used; Out def; };
+    static constexpr bool kStageable = false;
+    FKD_NAME("BatchReadDefault<" + istr(N) + "," + PlaneOp::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        if (p.used <= z) return p.def;
+        return PlaneOp::exec(x, y, z, p.plane[z]);
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+        if (p.used <= z) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) out[i] = p.def;
+        } else {
+            PlaneOp::template exec_row<V>(x, y, z, p.plane[z], out);
+        }
+    }
+#endif
+};
+
+// ReadSet<T>: constant fill source.  FK/algorithms/basic_ops/set.h:29-80.
+template <class T> struct ReadSet {
+    using Out = T;
+    struct Params { T value; u32 width, height, planes; };
+    static constexpr bool kStageable = false;
+    FKD_NAME("ReadSet<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return int(p.width); }
+    FKD_DEV static int height(const Params& p) { return int(p.height); }
+    FKD_DEV static T exec(int, int, int, const Params& p) { return p.value; }
+    template <int V> FKD_DEV static void exec_row(int, int, int, const Params& p, T (&out)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i] = p.value;
+    }
+#endif
+};
+
+// ===================================================================================================
+// Write operations: (x, y, z, value) -> memory
+// ===================================================================================================
+
+// PerThreadWrite<_2D,T>: FK/algorithms/basic_ops/memory_operations.h:84-107.
+template <class T> struct Write2D {
+    using In = T;
+    using Params = RawPtr2D<T>;
+    FKD_NAME("Write2D<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static void exec(int x, int y, int, const T& v, const Params& p) {
+        detail::store_elem(detail::row_ptr(p.data, p.pitch, x, y), v);
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int, const T (&v)[V], const Params& p) {
+        detail::store_run<T, V>(detail::row_ptr(p.data, p.pitch, x, y), v);
+    }
+#endif
+};
+
+// TensorWrite<T> / PerThreadWrite<_3D,T>: FK/algorithms/basic_ops/memory_operations.h:159-179; plane z at
+// z*plane_pitch*color_planes (FK/core/data/rawptr.h:215-226).
+template <class T> struct TensorWrite {
+    using In = T;
+    using Params = RawPtr3D<T>;
+    FKD_NAME("TensorWrite<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static T* plane(const Params& p, int z) {
+        return reinterpret_cast<T*>(reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z);
+    }
+    FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
+        detail::store_elem(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const T (&v)[V], const Params& p) {
+        detail::store_run<T, V>(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
+    }
+#endif
+};
+
+// TensorSplit<T>: FK/algorithms/basic_ops/memory_operations.h:181-212.  Planar store: channel c of pixel
+// (x,y) of plane z goes to the 3-D address of (x,y,z) plus c*width*height base elements.
+template <class T> struct TensorSplit {
+    using In = T;
+    using B = base_t<T>;
+    using Params = RawPtr3D<B>;
+    FKD_NAME("TensorSplit<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static B* at(const Params& p, int x, int y, int z) {
+        return reinterpret_cast<B*>(reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z +
+                                    size_t(y) * p.pitch) + x;
+    }
+    FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
+        B* w = at(p, x, y, z);
+        const size_t px = size_t(p.width) * p.height;
+        w[0] = chan<0>(v);
+        w[px] = chan<1>(v);
+        if constexpr (cn_v<T> > 2) w[2 * px] = chan<2>(v);
+        if constexpr (cn_v<T> > 3) w[3 * px] = chan<3>(v);
+    }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const T (&v)[V], const Params& p) {
+        B* w = at(p, x, y, z);
+        const size_t px = size_t(p.width) * p.height;
+        B c0[V], c1[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) { c0[i] = chan<0>(v[i]); c1[i] = chan<1>(v[i]); }
+        detail::store_run<B, V>(w, c0);
+        detail::store_run<B, V>(w + px, c1);
+        if constexpr (cn_v<T> > 2) {
+            B c2[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) c2[i] = chan<2>(v[i]);
+            detail::store_run<B, V>(w + 2 * px, c2);
+        }
+        if constexpr (cn_v<T> > 3) {
+            B c3[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) c3[i] = chan<3>(v[i]);
+            detail::store_run<B, V>(w + 3 * px, c3);
+        }
+    }
+#endif
+};
+
+// BatchWrite<N, Op>: FK/core/execution_model/operation_model/batch_operations.h:463-512.
+template <int N, class W> struct BatchWrite {
+    using In = typename W::In;
+    struct Params { typename W::Params plane[N]; };
+    FKD_NAME("BatchWrite<" + istr(N) + "," + W::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, z, v, p.plane[z]); }
+    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const In (&v)[V], const Params& p) {
+        W::template exec_row<V>(x, y, z, v, p.plane[z]);
+    }
+#endif
+};
+
+// ===================================================================================================
+// A fused chain: one read, a fold of compute operations, one write, over an active grid.
+// ===================================================================================================
+template <class R, class Ops, class W> struct Chain;
+template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
+    using Read = R;
+    using Write = W;
+    using Value = typename FoldOut<typename R::Out, Ops...>::type;
+    struct Params {
+        u32 active_w, active_h, active_z, reserved;
+        typename R::Params read;
+        Tup<typename Ops::Params...> ops;
+        typename W::Params write;
+    };
+    FKD_NAME("Chain<" + R::name() + ",OpList<" + (sizeof...(Ops) ? OpList<Ops...>::names().substr(1) : std::string()) + ">," + W::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    static_assert(__is_same(Value, typename W::In), "the write operation does not take the type the chain produces");
+    FKD_DEV static Value compute(const typename R::Out& v, const Params& p) {
+        if constexpr (sizeof...(Ops) == 0) return v; else return fold<Ops...>(v, p.ops);
+    }
+#endif
+};
+
+} // namespace fkd

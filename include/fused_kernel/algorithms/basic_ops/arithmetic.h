@@ -1,0 +1,34 @@
+// Add / Sub / Mul / Div as Binary operations (value op parameter, channel-wise, a scalar parameter is broadcast).
+// Interface counterpart: FK/algorithms/basic_ops/arithmetic.h:26-124.  The tuple-input Unary forms of the
+// reference are not part of the fused data-parallel path and are not provided.
+#ifndef FK_AMD_ARITHMETIC_H
+#define FK_AMD_ARITHMETIC_H
+
+#include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+
+namespace fk {
+
+#define FK_AMD_ARITH(Name)                                                                                      \
+    template <typename I1, typename I2 = I1, typename O = I1, typename IT = BinaryType> struct Name;            \
+    template <typename I, typename P, typename O>                                                               \
+    struct Name<I, P, O, BinaryType> : BinaryOperation<I, P, O, Name<I, P, O, BinaryType>> {                    \
+        using Parent = BinaryOperation<I, P, O, Name<I, P, O, BinaryType>>;                                     \
+        FK_STATIC_STRUCT(Name, Name)                                                                            \
+    };                                                                                                          \
+    namespace amd {                                                                                             \
+    template <typename I, typename P, typename O> struct Lower<Name<I, P, O, BinaryType>> {                     \
+        static constexpr bool available = true;                                                                 \
+        using type = fkd::Name<dev_t<I>, dev_t<P>, dev_t<O>>;                                                   \
+        static typename type::Params params(const OperationData<Name<I, P, O, BinaryType>>& d) {                \
+            return typename type::Params{to_dev(d.params)};                                                     \
+        }                                                                                                       \
+    };                                                                                                          \
+    }
+FK_AMD_ARITH(Add)
+FK_AMD_ARITH(Sub)
+FK_AMD_ARITH(Mul)
+FK_AMD_ARITH(Div)
+#undef FK_AMD_ARITH
+
+} // namespace fk
+#endif

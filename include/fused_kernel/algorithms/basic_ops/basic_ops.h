@@ -1,0 +1,8 @@
+#ifndef FK_AMD_BASIC_OPS_H
+#define FK_AMD_BASIC_OPS_H
+#include <fused_kernel/algorithms/basic_ops/arithmetic.h>
+#include <fused_kernel/algorithms/basic_ops/cast.h>
+#include <fused_kernel/algorithms/basic_ops/memory_operations.h>
+#include <fused_kernel/algorithms/basic_ops/set.h>
+#include <fused_kernel/algorithms/basic_ops/vector_ops.h>
+#endif

@@ -1,0 +1,146 @@
+// Per-element memory operations: PerThreadRead / PerThreadWrite (pitched 1-D/2-D/3-D), TensorRead / TensorWrite,
+// TensorSplit (planar writer).  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:26-212.
+#ifndef FK_AMD_MEMORY_OPERATIONS_H
+#define FK_AMD_MEMORY_OPERATIONS_H
+
+#include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+
+namespace fk {
+
+template <ND D, typename T>
+struct PerThreadRead : ReadOperation<T, RawPtr<D, T>, T, TF::ENABLED, PerThreadRead<D, T>> {
+    using Parent = ReadOperation<T, RawPtr<D, T>, T, TF::ENABLED, PerThreadRead<D, T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(PerThreadRead, PerThreadRead)
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint num_elems_y(const Point, const OperationDataType& opData) {
+        if constexpr (D == ND::_1D) return 1; else return opData.params.dims.height;
+    }
+    static constexpr uint num_elems_z(const Point, const OperationDataType& opData) {
+        if constexpr (D == ND::_1D || D == ND::_2D) return 1; else return opData.params.dims.planes;
+    }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {num_elems_x(Point{0, 0, 0}, opData), num_elems_y(Point{0, 0, 0}, opData), num_elems_z(Point{0, 0, 0}, opData)};
+    }
+};
+
+template <ND D, typename T>
+struct PerThreadWrite : WriteOperation<T, RawPtr<D, T>, T, TF::ENABLED, PerThreadWrite<D, T>> {
+    using Parent = WriteOperation<T, RawPtr<D, T>, T, TF::ENABLED, PerThreadWrite<D, T>>;
+    using typename Parent::OperationDataType;
+    using typename Parent::InstantiableType;
+    FK_STATIC_STRUCT(PerThreadWrite, PerThreadWrite)
+    using Parent::build;
+    static InstantiableType build(const Ptr<D, T>& ptr) { return {{ptr.ptr()}}; }
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+};
+
+// Deduces dimension and element type from the pointer: ReadOp::build(ptr), WriteOp::build(ptr).
+struct ReadOp {
+    template <typename PtrType> static decltype(auto) build(PtrType&& ptr) {
+        using P = std::decay_t<PtrType>;
+        return PerThreadRead<P::nd, typename P::Type>::build(ptr.ptr());
+    }
+    template <typename PtrType, size_t N> static decltype(auto) build(const std::array<PtrType, N>& ptrs) {
+        return PerThreadRead<PtrType::nd, typename PtrType::Type>::build(ptrs);
+    }
+};
+struct WriteOp {
+    template <typename PtrType> static decltype(auto) build(PtrType&& ptr) {
+        using P = std::decay_t<PtrType>;
+        return PerThreadWrite<P::nd, typename P::Type>::build(ptr.ptr());
+    }
+    template <typename PtrType, size_t N> static decltype(auto) build(const std::array<PtrType, N>& ptrs) {
+        return PerThreadWrite<PtrType::nd, typename PtrType::Type>::build(ptrs);
+    }
+};
+
+template <typename T> struct TensorRead : ReadOperation<T, RawPtr<ND::_3D, T>, T, TF::ENABLED, TensorRead<T>> {
+    using Parent = ReadOperation<T, RawPtr<ND::_3D, T>, T, TF::ENABLED, TensorRead<T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(TensorRead, TensorRead)
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint num_elems_y(const Point, const OperationDataType& opData) { return opData.params.dims.height; }
+    static constexpr uint num_elems_z(const Point, const OperationDataType& opData) { return opData.params.dims.planes; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {opData.params.dims.width, opData.params.dims.height, opData.params.dims.planes};
+    }
+};
+
+template <typename T> struct TensorWrite : WriteOperation<T, RawPtr<ND::_3D, T>, T, TF::ENABLED, TensorWrite<T>> {
+    using Parent = WriteOperation<T, RawPtr<ND::_3D, T>, T, TF::ENABLED, TensorWrite<T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(TensorWrite, TensorWrite)
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+};
+
+// Planar writer: channel c of pixel (x, y, z) lands c * width * height base elements after the AoS position.
+template <typename T> struct TensorSplit : WriteOperation<T, RawPtr<ND::_3D, VBase<T>>, VBase<T>, TF::DISABLED, TensorSplit<T>> {
+    using Parent = WriteOperation<T, RawPtr<ND::_3D, VBase<T>>, VBase<T>, TF::DISABLED, TensorSplit<T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(TensorSplit, TensorSplit)
+    static_assert(cn<T> >= 2, "Wrong type for split tensor write. It must be one of <type>2, <type>3 or <type>4.");
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+};
+
+namespace amd {
+template <typename T> struct Lower<PerThreadRead<ND::_2D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::Read2D<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadRead<ND::_2D, T>>& d) { return to_dev<T, const dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<PerThreadRead<ND::_1D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::Read2D<dev_t<T>>;   // a 1-D array is a one-row image
+    static typename type::Params params(const OperationData<PerThreadRead<ND::_1D, T>>& d) {
+        return typename type::Params{reinterpret_cast<const dev_t<T>*>(d.params.data), d.params.dims.width, 1u, d.params.dims.pitch};
+    }
+};
+template <typename T> struct Lower<PerThreadRead<ND::_3D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::Read3D<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadRead<ND::_3D, T>>& d) { return to_dev3<T, const dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<TensorRead<T>> {
+    static constexpr bool available = true;
+    using type = fkd::Read3D<dev_t<T>>;
+    static typename type::Params params(const OperationData<TensorRead<T>>& d) { return to_dev3<T, const dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<PerThreadWrite<ND::_2D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::Write2D<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadWrite<ND::_2D, T>>& d) { return to_dev<T, dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<PerThreadWrite<ND::_1D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::Write2D<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadWrite<ND::_1D, T>>& d) {
+        return typename type::Params{reinterpret_cast<dev_t<T>*>(d.params.data), d.params.dims.width, 1u, d.params.dims.pitch};
+    }
+};
+template <typename T> struct Lower<PerThreadWrite<ND::_3D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorWrite<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadWrite<ND::_3D, T>>& d) { return to_dev3<T, dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<TensorWrite<T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorWrite<dev_t<T>>;
+    static typename type::Params params(const OperationData<TensorWrite<T>>& d) { return to_dev3<T, dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<TensorSplit<T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorSplit<dev_t<T>>;
+    static typename type::Params params(const OperationData<TensorSplit<T>>& d) {
+        return to_dev3<VBase<T>, typename DevType<VBase<T>>::type>(d.params);
+    }
+};
+} // namespace amd
+
+} // namespace fk
+#endif

@@ -1,0 +1,33 @@
+// ReadSet<T>: a read that yields one constant for every element of an active grid.
+// Interface counterpart: FK/algorithms/basic_ops/set.h:29-80.
+#ifndef FK_AMD_SET_H
+#define FK_AMD_SET_H
+#include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+namespace fk {
+template <typename T> struct ReadSetParams {
+    T value;
+    ActiveThreads size;
+};
+template <typename T> struct ReadSet : ReadOperation<T, ReadSetParams<T>, T, TF::DISABLED, ReadSet<T>> {
+    using Parent = ReadOperation<T, ReadSetParams<T>, T, TF::DISABLED, ReadSet<T>>;
+    using typename Parent::OperationDataType;
+    using typename Parent::InstantiableType;
+    FK_STATIC_STRUCT(ReadSet, ReadSet)
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.size.x; }
+    static constexpr uint num_elems_y(const Point, const OperationDataType& opData) { return opData.params.size.y; }
+    static constexpr uint num_elems_z(const Point, const OperationDataType& opData) { return opData.params.size.z; }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) { return opData.params.size; }
+    using Parent::build;
+    static constexpr InstantiableType build(const T& value, const ActiveThreads& activeThreads) { return {{{value, activeThreads}}}; }
+};
+namespace amd {
+template <typename T> struct Lower<ReadSet<T>> {
+    static constexpr bool available = true;
+    using type = fkd::ReadSet<dev_t<T>>;
+    static typename type::Params params(const OperationData<ReadSet<T>>& d) {
+        return typename type::Params{to_dev(d.params.value), d.params.size.x, d.params.size.y, d.params.size.z};
+    }
+};
+} // namespace amd
+} // namespace fk
+#endif

@@ -1,0 +1,46 @@
+// Colour-format vocabulary: colour spaces, ranges, primaries, depths and pixel formats, with the per-format
+// traits the NV12 reader needs.  Interface counterpart: FK/algorithms/image_processing/itu_color.h:21-101.
+// The YCbCr->RGB matrix itself is evaluated inside the device code (fkd::YUV2RGB709Full8), in binary32 and in
+// the reference's expression order (itu_color.h:185-265).
+#ifndef FK_AMD_ITU_COLOR_H
+#define FK_AMD_ITU_COLOR_H
+
+#include <fused_kernel/core/utils/vector_utils.h>
+
+namespace fk {
+
+enum class ColorSpace { YUV420, YUV422, YUV444, RGB, RGBA };
+enum class ColorRange { Limited, Full };
+enum class ColorPrimitives { bt601, bt709, bt2020 };
+enum class ColorDepth { p8bit, p10bit, p12bit, fn8bit, fn10bit, fn12bit };
+enum class PixelFormat { NV12, NV21, YV12, P010, P016, P216, P210, Y216, Y210, Y416, UYVY };
+
+template <ColorDepth CD> struct ColorDepthTraits;
+template <> struct ColorDepthTraits<ColorDepth::p8bit> { using base = uchar; using pixel = uchar3; };
+template <> struct ColorDepthTraits<ColorDepth::p10bit> { using base = ushort; using pixel = ushort3; };
+template <> struct ColorDepthTraits<ColorDepth::p12bit> { using base = ushort; using pixel = ushort3; };
+template <> struct ColorDepthTraits<ColorDepth::fn8bit> { using base = float; using pixel = float3; };
+template <> struct ColorDepthTraits<ColorDepth::fn10bit> { using base = float; using pixel = float3; };
+template <> struct ColorDepthTraits<ColorDepth::fn12bit> { using base = float; using pixel = float3; };
+template <ColorDepth CD> using ColorDepthPixelBaseType = typename ColorDepthTraits<CD>::base;
+template <ColorDepth CD> using ColorDepthPixelType = typename ColorDepthTraits<CD>::pixel;
+
+// Number of base-type elements per image column / row of the backing buffer.
+struct ResolutionFactors { float width_f; float height_f; };
+
+template <PixelFormat PF> struct PixelFormatTraits;
+template <> struct PixelFormatTraits<PixelFormat::NV12> {
+    static constexpr ColorSpace space = ColorSpace::YUV420;
+    static constexpr ColorDepth depth = ColorDepth::p8bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{1.f, 1.5f};
+};
+template <> struct PixelFormatTraits<PixelFormat::NV21> {
+    static constexpr ColorSpace space = ColorSpace::YUV420;
+    static constexpr ColorDepth depth = ColorDepth::p8bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{1.f, 1.5f};
+};
+
+} // namespace fk
+#endif

@@ -1,0 +1,132 @@
+// Executor<TransformDPP<ParArch::GPU_AMD, TF>>: turns an argument list of IOps into one launch of a gfx950 kernel.
+//
+//   1. BackFuser::fuse_back collapses the Read + ReadBack... prefix into one Read IOp (backwards vertical fusion).
+//   2. Every IOp is lowered to its device counterpart; together they spell the type fkd::Chain<Read, OpList<...>,
+//      Write>.  Its name() is the kernel signature; its Params, filled from the IOps' values, is the kernel argument.
+//   3. fklhip_launch_handle copies the parameter block and enqueues the kernel on the stream (asynchronous, like the
+//      CUDA backend's <<<>>> launch); a failure surfaces as std::runtime_error("GPU Error: ...").
+//
+// Interface counterpart: FK/core/execution_model/executors.h:53-143 (overload family), :311-358 (GPU executor).
+#ifndef FK_AMD_EXECUTORS_H
+#define FK_AMD_EXECUTORS_H
+
+#include <string>
+
+#include <fused_kernel/core/execution_model/data_parallel_patterns.h>
+#include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+#include <fused_kernel/core/execution_model/stream.h>
+#include <fused_kernel/algorithms/basic_ops/memory_operations.h>
+
+namespace fk {
+
+namespace amd {
+
+// The device chain type of a fused IOp list (read, compute..., write).
+template <typename ReadIOp, typename... Rest> struct ChainOf;
+template <typename ReadIOp, typename WriteIOp, typename... Compute>
+struct ChainBuilder {
+    using type = fkd::Chain<device_op_t<ReadIOp>, fkd::OpList<device_op_t<Compute>...>, device_op_t<WriteIOp>>;
+};
+
+template <typename Chain> const void* kernel_handle() {
+    // Resolved once per chain type; thread-safe by the rules of function-local statics.
+    static const void* handle = [] {
+        const std::string sig = Chain::name();
+        const void* h = nullptr;
+        const int rc = fklhip_lookup(sig.c_str(), &h);
+        if (rc != FKLHIP_OK) {
+            throw std::runtime_error(std::string("GPU Error: ") + fklhip_error_string(rc) + "\n  signature: " + sig + "\n");
+        }
+        return h;
+    }();
+    return handle;
+}
+
+template <size_t... Is, typename Tuple>
+auto lower_compute(std::index_sequence<Is...>, const Tuple& t) {
+    return make_tup(lower_iop(std::get<Is + 1>(t))...);
+}
+
+template <typename... IOps> void launch_fused(void* stream, const IOps&... iOps) {
+    constexpr size_t N = sizeof...(IOps);
+    static_assert(N >= 2, "a chain needs at least a read and a write operation");
+    const auto all = std::forward_as_tuple(iOps...);
+    using Tuple = std::tuple<const IOps&...>;
+    using ReadIOp = std::decay_t<std::tuple_element_t<0, Tuple>>;
+    using WriteIOp = std::decay_t<std::tuple_element_t<N - 1, Tuple>>;
+    static_assert(isAnyCompleteReadType<ReadIOp>, "the first operation must be a complete Read or ReadBack operation");
+    static_assert(opIs<WriteType, WriteIOp>, "the last operation must be a Write operation");
+
+    [&]<size_t... Is>(std::index_sequence<Is...>) {
+        static_assert((isComputeType<std::decay_t<std::tuple_element_t<Is + 1, Tuple>>> && ...),
+                      "only Unary/Binary/Ternary operations may sit between the read and the write");
+        using Chain = fkd::Chain<device_op_t<ReadIOp>,
+                                 fkd::OpList<device_op_t<std::decay_t<std::tuple_element_t<Is + 1, Tuple>>>...>,
+                                 device_op_t<WriteIOp>>;
+        typename Chain::Params p{};
+        const ActiveThreads active = std::get<0>(all).getActiveThreads();
+        p.active_w = active.x;
+        p.active_h = active.y;
+        p.active_z = active.z;
+        p.read = lower_iop(std::get<0>(all));
+        p.ops = make_tup(lower_iop(std::get<Is + 1>(all))...);
+        p.write = lower_iop(std::get<N - 1>(all));
+        gpuErrchk(fklhip_launch_handle(kernel_handle<Chain>(), &p, sizeof(p), stream));
+    }(std::make_index_sequence<N - 2>{});
+}
+
+} // namespace amd
+
+template <typename Child> struct BaseExecutor {
+    template <ParArch PA, typename... IOps> static void executeOperations(Stream_<PA>& stream, const IOps&... iOps) {
+        const auto fused = BackFuser::fuse_back(iOps...);
+        std::apply([&](const auto&... f) { Child::executeOperations_helper(stream, f...); }, fused);
+    }
+    template <ParArch PA, ND D, typename I, typename... IOps>
+    static void executeOperations(const Ptr<D, I>& input, Stream_<PA>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<D, I>::build(input.ptr()), iOps...);
+    }
+    template <ParArch PA, ND D, typename I, typename O, typename... IOps>
+    static void executeOperations(const Ptr<D, I>& input, const Ptr<D, O>& output, Stream_<PA>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<D, I>::build(input.ptr()), iOps..., PerThreadWrite<D, O>::build(output.ptr()));
+    }
+    template <ParArch PA, typename I, size_t BATCH, typename... IOps>
+    static void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const int& activeBatch, const I& defaultValue,
+                                  Stream_<PA>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(activeBatch, defaultValue, input), iOps...);
+    }
+    template <ParArch PA, typename I, size_t BATCH, typename... IOps>
+    static void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, Stream_<PA>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(input), iOps...);
+    }
+    template <ParArch PA, typename I, typename O, size_t Batch, typename... IOps>
+    static void executeOperations(const std::array<Ptr2D<I>, Batch>& input, const int& activeBatch, const I& defaultValue,
+                                  const Tensor<O>& output, Stream_<PA>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(activeBatch, defaultValue, input), iOps...,
+                          PerThreadWrite<ND::_3D, O>::build(output.ptr()));
+    }
+    template <ParArch PA, typename I, typename O, size_t Batch, typename... IOps>
+    static void executeOperations(const std::array<Ptr2D<I>, Batch>& input, const Tensor<O>& output, Stream_<PA>& stream,
+                                  const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(input), iOps..., PerThreadWrite<ND::_3D, O>::build(output.ptr()));
+    }
+};
+
+template <typename DataParallelPattern> struct Executor {
+    static_assert(DataParallelPattern::PAR_ARCH == ParArch::GPU_AMD,
+                  "this build of the library provides the GPU_AMD (MI355X) backend only");
+};
+
+template <TF TFEN> struct Executor<TransformDPP<ParArch::GPU_AMD, TFEN, void>> : BaseExecutor<Executor<TransformDPP<ParArch::GPU_AMD, TFEN, void>>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::GPU_AMD; }
+
+private:
+    friend struct BaseExecutor<Executor<TransformDPP<ParArch::GPU_AMD, TFEN, void>>>;
+    template <typename... IOps> static void executeOperations_helper(Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        amd::launch_fused(stream.getNativeStream(), iOps...);
+    }
+};
+
+} // namespace fk
+#endif

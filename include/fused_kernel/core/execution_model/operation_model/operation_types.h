@@ -1,0 +1,5 @@
+// Part of the operation model; the definitions live in operation_model.h.
+#ifndef FK_AMD_FWD_OPERATION_TYPES_H
+#define FK_AMD_FWD_OPERATION_TYPES_H
+#include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+#endif

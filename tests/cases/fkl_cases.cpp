@@ -1,0 +1,204 @@
+// fkl_cases.cpp -- the benchmark chains spelled with the library's C++ host API, exactly as a user of the
+// reference library writes them (same names, same argument order), behind extern "C" drivers so pytest and
+// bench.py can hand in device pointers.  Everything here runs through executeOperations<TransformDPP<>> ->
+// host-side fusion -> fklhip_launch_handle -> gfx950 kernel; nothing computes on the CPU.
+//
+// Compiled by g++ (no HIP headers): g++ -std=c++20 -I include tests/cases/fkl_cases.cpp -L... -lfklhip
+#include <fused_kernel/algorithms/basic_ops/memory_operations.h>
+#include <fused_kernel/algorithms/basic_ops/arithmetic.h>
+#include <fused_kernel/algorithms/basic_ops/cast.h>
+#include <fused_kernel/algorithms/image_processing/crop.h>
+#include <fused_kernel/algorithms/image_processing/color_conversion.h>
+#include <fused_kernel/algorithms/image_processing/resize.h>
+#include <fused_kernel/algorithms/image_processing/saturate.h>
+#include <fused_kernel/algorithms/image_processing/image.h>
+#include <fused_kernel/fused_kernel.h>
+
+#include <array>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <exception>
+#include <utility>
+
+using namespace fk;
+
+namespace {
+
+thread_local char g_error[2048] = "";
+
+template <typename F> int guarded(F body) {
+    try {
+        body();
+        return 0;
+    } catch (const std::exception& e) {
+        std::snprintf(g_error, sizeof(g_error), "%s", e.what());
+        return 1;
+    }
+}
+
+template <typename T> Ptr2D<T> dev2d(const void* data, int w, int h, int pitch) {
+    return Ptr2D<T>(reinterpret_cast<T*>(const_cast<void*>(data)), uint(w), uint(h), uint(pitch), MemType::Device, 0);
+}
+
+template <size_t B> std::array<Rect, B> rects_from(const int32_t* r) {
+    std::array<Rect, B> a{};
+    for (size_t i = 0; i < B; ++i) a[i] = Rect(r[4 * i + 0], r[4 * i + 1], r[4 * i + 2], r[4 * i + 3]);
+    return a;
+}
+
+// Configuration 1 (README chain).
+template <size_t B>
+void crop_resize_par_u8(void* stream_, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                        const float* bg, const float* mul, const float* sub, uint8_t* out) {
+    Stream stream(stream_);
+    const auto in = dev2d<uchar3>(src, w, h, pitch);
+    Tensor<uchar3> o(reinterpret_cast<uchar3*>(out), uint(dw), uint(dh), uint(B), 1, MemType::Device, 0);
+    const auto crops = rects_from<B>(rects);
+    executeOperations<TransformDPP<>>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
+        Crop<>::build(crops),
+        Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(dw, dh), float3{bg[0], bg[1], bg[2]}),
+        Mul<float3>::build(make_<float3>(mul[0], mul[1], mul[2])),
+        Sub<float3>::build(make_<float3>(sub[0], sub[1], sub[2])),
+        SaturateCast<float3, uchar3>::build(),
+        TensorWrite<uchar3>::build(o.ptr()));
+}
+
+// Configuration 3.
+template <size_t B>
+void crop_resize_norm_split(void* stream_, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                            const float* sub, const float* div, float* out) {
+    Stream stream(stream_);
+    const auto in = dev2d<uchar3>(src, w, h, pitch);
+    Tensor<float> o(out, uint(dw), uint(dh), uint(B), 3, MemType::Device, 0);
+    const auto crops = rects_from<B>(rects);
+    executeOperations<TransformDPP<>>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
+        Crop<>::build(crops),
+        Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
+        ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, float3, float3>::build(),
+        Sub<float3>::build(make_<float3>(sub[0], sub[1], sub[2])),
+        Div<float3>::build(make_<float3>(div[0], div[1], div[2])),
+        TensorSplit<float3>::build(o.ptr()));
+}
+
+// Configuration 4.
+template <size_t B>
+void batch_muladd_sat(void* stream_, const uint8_t* const* srcs, int w, int h, int pitch, const float* mul, const float* add,
+                      uint8_t* const* outs, int out_pitch) {
+    Stream stream(stream_);
+    using PlaneIOp = decltype(PerThreadRead<ND::_2D, uchar3>::build(std::declval<RawPtr<ND::_2D, uchar3>>())
+                                  .then(Mul<uchar3, float3, float3>::build(float3{}))
+                                  .then(Add<float3>::build(float3{})));
+    std::array<PlaneIOp, B> planes{};
+    std::array<Ptr2D<uchar3>, B> outPtrs{};
+    for (size_t i = 0; i < B; ++i) {
+        const auto in = dev2d<uchar3>(srcs[i], w, h, pitch);
+        planes[i] = PerThreadRead<ND::_2D, uchar3>::build(in.ptr())
+                        .then(Mul<uchar3, float3, float3>::build(make_<float3>(mul[3 * i], mul[3 * i + 1], mul[3 * i + 2])))
+                        .then(Add<float3>::build(make_<float3>(add[3 * i], add[3 * i + 1], add[3 * i + 2])));
+        outPtrs[i] = dev2d<uchar3>(outs[i], w, h, out_pitch);
+    }
+    executeOperations<TransformDPP<>>(stream,
+        BatchRead<PlanePolicy::PROCESS_ALL>::build(planes),
+        SaturateCast<float3, uchar3>::build(),
+        PerThreadWrite<ND::_2D, uchar3>::build(outPtrs));
+}
+
+// Configuration 2.
+template <typename DPP, size_t... Is>
+void add_mul_chain(Stream& stream, const Ptr2D<float>& in, const Ptr2D<float>& out, float addv, float mulv,
+                   std::index_sequence<Is...>) {
+    const auto pick = [&](auto idx) {
+        if constexpr (decltype(idx)::value % 2 == 0) return Add<float>::build(addv);
+        else return Mul<float>::build(mulv);
+    };
+    executeOperations<DPP>(stream, PerThreadRead<ND::_2D, float>::build(in.ptr()),
+                           pick(std::integral_constant<size_t, Is>{})...,
+                           PerThreadWrite<ND::_2D, float>::build(out.ptr()));
+}
+
+template <size_t N>
+void add_mul_n(void* stream_, const float* in, int w, int h, int pitch, float addv, float mulv, float* out, int out_pitch, int tf) {
+    Stream stream(stream_);
+    const auto i = dev2d<float>(in, w, h, pitch);
+    const auto o = dev2d<float>(out, w, h, out_pitch);
+    if (tf) add_mul_chain<TransformDPP<ParArch::GPU_AMD, TF::ENABLED>>(stream, i, o, addv, mulv, std::make_index_sequence<N>{});
+    else add_mul_chain<TransformDPP<>>(stream, i, o, addv, mulv, std::make_index_sequence<N>{});
+}
+
+// Integer-only chain.
+template <size_t B>
+void crop_swap_u8(void* stream_, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
+    Stream stream(stream_);
+    const auto in = dev2d<uchar3>(src, w, h, pitch);
+    Tensor<uchar3> o(reinterpret_cast<uchar3*>(out), uint(rects[2]), uint(rects[3]), uint(B), 1, MemType::Device, 0);
+    const auto crops = rects_from<B>(rects);
+    executeOperations<TransformDPP<>>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr()).then(Crop<>::build(crops)),
+        ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, uchar3, uchar3>::build(),
+        TensorWrite<uchar3>::build(o.ptr()));
+}
+
+} // namespace
+
+extern "C" {
+
+const char* fklcase_last_error(void) { return g_error; }
+
+int fklcase_crop_resize_par_u8_b5(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw,
+                                  int dh, const float* bg, const float* mul, const float* sub, uint8_t* out) {
+    return guarded([&] { crop_resize_par_u8<5>(stream, src, w, h, pitch, rects, dw, dh, bg, mul, sub, out); });
+}
+int fklcase_crop_resize_norm_split_b8(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects,
+                                      int dw, int dh, const float* sub, const float* div, float* out) {
+    return guarded([&] { crop_resize_norm_split<8>(stream, src, w, h, pitch, rects, dw, dh, sub, div, out); });
+}
+int fklcase_crop_resize_norm_split_b64(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects,
+                                       int dw, int dh, const float* sub, const float* div, float* out) {
+    return guarded([&] { crop_resize_norm_split<64>(stream, src, w, h, pitch, rects, dw, dh, sub, div, out); });
+}
+int fklcase_batch_muladd_sat_b4(void* stream, const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,
+                                const float* add, uint8_t* const* outs, int out_pitch) {
+    return guarded([&] { batch_muladd_sat<4>(stream, srcs, w, h, pitch, mul, add, outs, out_pitch); });
+}
+int fklcase_batch_muladd_sat_b100(void* stream, const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,
+                                  const float* add, uint8_t* const* outs, int out_pitch) {
+    return guarded([&] { batch_muladd_sat<100>(stream, srcs, w, h, pitch, mul, add, outs, out_pitch); });
+}
+int fklcase_add_mul_chain(void* stream, const float* in, int w, int h, int pitch, int n_ops, float addv, float mulv,
+                          float* out, int out_pitch, int tf) {
+    return guarded([&] {
+        switch (n_ops) {
+        case 1: add_mul_n<1>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 2: add_mul_n<2>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 3: add_mul_n<3>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 10: add_mul_n<10>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 50: add_mul_n<50>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 100: add_mul_n<100>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        default: throw std::runtime_error("add_mul_chain: unsupported operation count");
+        }
+    });
+}
+// Configuration 5.
+int fklcase_nv12_rgb_resize_split(void* stream_, const uint8_t* nv12, int w, int h, int pitch, int dw, int dh, float scale,
+                                  float* out) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const Ptr2D<uchar> data(const_cast<uchar*>(nv12), uint(w), uint(h + h / 2), uint(pitch), MemType::Device, 0);
+        const Image<PixelFormat::NV12> img(data, uint(w), uint(h));
+        Tensor<float> o(out, uint(dw), uint(dh), 1, 3, MemType::Device, 0);
+        executeOperations<TransformDPP<>>(stream,
+            ReadYUV<PixelFormat::NV12>::build(img.ptr()),
+            ConvertYUVToRGB<ColorDepth::p8bit, ColorRange::Full, ColorPrimitives::bt709>::build(),
+            Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
+            Mul<float3, float>::build(scale),
+            TensorSplit<float3>::build(o.ptr()));
+    });
+}
+int fklcase_crop_swap_u8_b4(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
+    return guarded([&] { crop_swap_u8<4>(stream, src, w, h, pitch, rects, out); });
+}
+
+} // extern "C"
