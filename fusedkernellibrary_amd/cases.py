@@ -33,6 +33,11 @@ def _ok(rc: int) -> None:
         raise RuntimeError(cases().fklcase_last_error().decode())
 
 
+def set_reps(reps: int) -> None:
+    """The next chain call enqueues its kernel `reps` times back to back through the C++ host API."""
+    cases().fklcase_set_reps(int(reps))
+
+
 def _stream():
     import torch
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)

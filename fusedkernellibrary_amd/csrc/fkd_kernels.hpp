@@ -55,7 +55,7 @@ template <class Chain> constexpr bool is_staged_chain() {
 constexpr int kRowsBX = 64;   // lanes along x: one wave per row segment
 constexpr int kRowsBY = 4;    // waves per workgroup
 
-template <class Chain, int V, int ROWS>
+template <class Chain, int V, int ROWS, bool ALIGNED>
 __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain::Params p) {
     using R = typename Chain::Read;
     using W = typename Chain::Write;
@@ -63,23 +63,23 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
     const int x0 = (blockIdx.x * kRowsBX + threadIdx.x) * V;
     const int ybase = (blockIdx.y * kRowsBY + threadIdx.y) * ROWS;
     const int aw = int(p.active_w), ah = int(p.active_h);
-    if (x0 >= aw) return;
+    if (x0 >= aw || ybase >= ah) return;
     if (x0 + V <= aw) {
-        typename R::Out in[ROWS][V];
+        // All loads first, unconditionally (rows past the end re-read the last row, which is in bounds), so every
+        // lane has ROWS independent wide loads in flight before the first use; only the stores are predicated.
+        Slot<typename R::Out> in[ROWS][V];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            const int y = ybase + r;
-            if (y < ah) R::template exec_row<V>(x0, y, z, p.read, in[r]);
+            const int y = ybase + r < ah ? ybase + r : ah - 1;
+            R::template exec_row<V, ALIGNED>(x0, y, z, p.read, in[r]);
         }
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
             const int y = ybase + r;
-            if (y < ah) {
-                typename Chain::Value out[V];
+            Slot<typename Chain::Value> out[V];
 #pragma unroll
-                for (int i = 0; i < V; ++i) out[i] = Chain::compute(in[r][i], p);
-                W::template exec_row<V>(x0, y, z, out, p.write);
-            }
+            for (int i = 0; i < V; ++i) out[i].v = Chain::compute(in[r][i].v, p);
+            if (y < ah) W::template exec_row<V, ALIGNED>(x0, y, z, out, p.write);
         }
     } else {
         for (int r = 0; r < ROWS; ++r) {
@@ -163,11 +163,32 @@ __global__ __launch_bounds__(kStagedBX * kStagedBY) void k_staged(const typename
         fh = int(__builtin_floorf(f32(ye) * q.fy)) + 1 - fy0 + 1;
         staged = fx0 >= 0 && fy0 >= 0 && fw > 0 && fh > 0 && u32(fw) * u32(fh) <= g.lds_slots;
         if (staged) {
-            for (int r = threadIdx.y; r < fh; r += kStagedBY) {
-                const int sy = fy0 + r < sh - 1 ? fy0 + r : sh - 1;
-                for (int c = threadIdx.x; c < fw; c += kStagedBX) {
-                    const int sx = fx0 + c < sw - 1 ? fx0 + c : sw - 1;
-                    lds[r * fw + c] = lds_pack<Raw>(Back::exec_raw(sx, sy, z, q.back));
+            // RU x CU raw elements per thread and step: all their loads are issued before the first LDS write.
+            // Coordinates are clamped into the source, so even the predicated-off positions load in bounds.
+            constexpr int RU = 2, CU = 2;
+            for (int r0 = threadIdx.y; r0 < fh; r0 += kStagedBY * RU) {
+                for (int c0 = threadIdx.x; c0 < fw; c0 += kStagedBX * CU) {
+                    Raw v[RU][CU];
+#pragma unroll
+                    for (int i = 0; i < RU; ++i) {
+                        const int r = r0 + kStagedBY * i;
+                        const int sy = fy0 + r < sh - 1 ? fy0 + r : sh - 1;
+#pragma unroll
+                        for (int j = 0; j < CU; ++j) {
+                            const int c = c0 + kStagedBX * j;
+                            const int sx = fx0 + c < sw - 1 ? fx0 + c : sw - 1;
+                            v[i][j] = Back::exec_raw(sx, sy, z, q.back);
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < RU; ++i) {
+                        const int r = r0 + kStagedBY * i;
+#pragma unroll
+                        for (int j = 0; j < CU; ++j) {
+                            const int c = c0 + kStagedBX * j;
+                            if (r < fh && c < fw) lds[r * fw + c] = lds_pack<Raw>(v[i][j]);
+                        }
+                    }
                 }
             }
         }
@@ -210,8 +231,13 @@ template <class Chain> struct RowsConfig {
     // Four elements per thread wherever the chain reads rows; a bilinear read that cannot be staged keeps one
     // element per thread (its taps are gathers, wider threads would only spread them further apart).
     static constexpr int V = ResizeRoot<typename Chain::Read>::value ? 1 : 4;
-    static constexpr int ROWS = ResizeRoot<typename Chain::Read>::value ? 1 : 4;
+#ifndef FKD_ROWS
+#define FKD_ROWS 4
+#endif
+    static constexpr int ROWS = ResizeRoot<typename Chain::Read>::value ? 1 : FKD_ROWS;
 };
+
+inline const char* aligned_name(bool aligned) { return aligned ? "rows" : "rows_unaligned"; }
 
 template <class Chain>
 hipError_t launch_rows(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
@@ -219,10 +245,13 @@ hipError_t launch_rows(const typename Chain::Params& p, hipStream_t stream, Laun
     const unsigned gx = (p.active_w + kRowsBX * V - 1) / (kRowsBX * V);
     const unsigned gy = (p.active_h + kRowsBY * ROWS - 1) / (kRowsBY * ROWS);
     const dim3 grid(gx, gy, p.active_z), block(kRowsBX, kRowsBY, 1);
-    if (info) *info = LaunchInfo{"rows", {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
+    // Wide (dwordx3/x4) accesses need every row start dword aligned; checked here, once per launch, on the host.
+    const bool aligned = Chain::Read::rows_aligned(p.read, 0) && Chain::Write::rows_aligned(p.write);
+    if (info) *info = LaunchInfo{aligned_name(aligned), {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
     if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
     if (grid.y > 65535u || grid.z > 65535u) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((k_rows<Chain, V, ROWS>), grid, block, 0, stream, p);
+    if (aligned) hipLaunchKernelGGL((k_rows<Chain, V, ROWS, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((k_rows<Chain, V, ROWS, false>), grid, block, 0, stream, p);
     return hipGetLastError();
 }
 

@@ -25,6 +25,11 @@ inline std::string istr(long long v) { return std::to_string(v); }
 #define FKD_NAME(expr)
 #endif
 
+// In-register home of one element inside per-thread arrays.  Elements whose size is not a multiple of 4 (uchar3,
+// uchar, ushort3 ...) are padded to whole dwords: arrays of 3-byte structs make the optimiser form 24-bit integer
+// vectors that the backend can only legalise through scratch or LDS.
+template <class T> struct alignas(sizeof(T) % 4 != 0 ? 4 : alignof(T)) Slot { T v; };
+
 #if defined(FKD_DEVICE_CODE)
 namespace detail {
 
@@ -53,61 +58,157 @@ template <class T> FKD_DEV void store_elem(T* p, const T& v) {
     }
 }
 
-template <int WORDS> struct alignas(4) Words { u32 w[WORDS]; };
+// Dword vectors that may sit at any dword-aligned address: one global_load/store_dwordx{2,3,4} each.
+typedef u32 u32x2_t __attribute__((ext_vector_type(2)));
+typedef u32 u32x3_t __attribute__((ext_vector_type(3)));
+typedef u32 u32x4_t __attribute__((ext_vector_type(4)));
+typedef u32x2_t u32x2_a4 __attribute__((aligned(4)));
+typedef u32x3_t u32x3_a4 __attribute__((aligned(4)));
+typedef u32x4_t u32x4_a4 __attribute__((aligned(4)));
 
-// V consecutive elements starting at p.  When the run is a whole number of dwords and p is dword aligned the
-// run moves as one wide access per <= 16 bytes (global_load_dwordx3 for four uchar3, dwordx4 for four floats),
-// which consecutive lanes make contiguous; otherwise element by element.
-template <class T, int V> FKD_DEV void load_run(const T* p, T (&out)[V]) {
-    constexpr int BYTES = int(sizeof(T)) * V;
-    if constexpr (V > 1 && BYTES % 4 == 0) {
-        if ((reinterpret_cast<uintptr_t>(p) & 3u) == 0) {
-            constexpr int W = BYTES / 4;
-            Words<W> w;
-            const Words<(W > 4 ? 4 : W)>* src = reinterpret_cast<const Words<(W > 4 ? 4 : W)>*>(p);
-            if constexpr (W <= 4) {
-                w = *reinterpret_cast<const Words<W>*>(p);
-            } else {
-                static_assert(W % 4 == 0, "wide runs are multiples of 16 bytes");
+template <int W> FKD_DEV void load_words(const void* p, u32 (&w)[W]) {
+    static_assert(W >= 1 && (W <= 4 || W % 4 == 0), "runs are 1-4 dwords or whole 16-byte groups");
+    if constexpr (W == 1) {
+        w[0] = *reinterpret_cast<const u32*>(p);
+    } else if constexpr (W == 2) {
+        const u32x2_t v = *reinterpret_cast<const u32x2_a4*>(p);
+        w[0] = v.x; w[1] = v.y;
+    } else if constexpr (W == 3) {
+        const u32x3_t v = *reinterpret_cast<const u32x3_a4*>(p);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z;
+    } else {
 #pragma unroll
-                for (int i = 0; i < W / 4; ++i) {
-                    const Words<4> t = src[i];
-                    w.w[4 * i + 0] = t.w[0]; w.w[4 * i + 1] = t.w[1]; w.w[4 * i + 2] = t.w[2]; w.w[4 * i + 3] = t.w[3];
-                }
-            }
-            __builtin_memcpy(&out[0], &w, BYTES);
-            return;
+        for (int i = 0; i < W / 4; ++i) {
+            const u32x4_t v = reinterpret_cast<const u32x4_a4*>(p)[i];
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
         }
     }
-#pragma unroll
-    for (int i = 0; i < V; ++i) out[i] = load_elem(p + i);
 }
-
-template <class T, int V> FKD_DEV void store_run(T* p, const T (&in)[V]) {
-    constexpr int BYTES = int(sizeof(T)) * V;
-    if constexpr (V > 1 && BYTES % 4 == 0) {
-        if ((reinterpret_cast<uintptr_t>(p) & 3u) == 0) {
-            constexpr int W = BYTES / 4;
-            Words<W> w;
-            __builtin_memcpy(&w, &in[0], BYTES);
-            if constexpr (W <= 4) {
-                *reinterpret_cast<Words<W>*>(p) = w;
-            } else {
-                static_assert(W % 4 == 0, "wide runs are multiples of 16 bytes");
-                Words<4>* dst = reinterpret_cast<Words<4>*>(p);
+template <int W> FKD_DEV void store_words(void* p, const u32 (&w)[W]) {
+    static_assert(W >= 1 && (W <= 4 || W % 4 == 0), "runs are 1-4 dwords or whole 16-byte groups");
+    if constexpr (W == 1) {
+        *reinterpret_cast<u32*>(p) = w[0];
+    } else if constexpr (W == 2) {
+        u32x2_t v; v.x = w[0]; v.y = w[1];
+        *reinterpret_cast<u32x2_a4*>(p) = v;
+    } else if constexpr (W == 3) {
+        u32x3_t v; v.x = w[0]; v.y = w[1]; v.z = w[2];
+        *reinterpret_cast<u32x3_a4*>(p) = v;
+    } else {
 #pragma unroll
-                for (int i = 0; i < W / 4; ++i) {
-                    Words<4> t;
-                    t.w[0] = w.w[4 * i + 0]; t.w[1] = w.w[4 * i + 1]; t.w[2] = w.w[4 * i + 2]; t.w[3] = w.w[4 * i + 3];
-                    dst[i] = t;
-                }
-            }
-            return;
+        for (int i = 0; i < W / 4; ++i) {
+            u32x4_t v; v.x = w[4 * i]; v.y = w[4 * i + 1]; v.z = w[4 * i + 2]; v.w = w[4 * i + 3];
+            reinterpret_cast<u32x4_a4*>(p)[i] = v;
         }
     }
-#pragma unroll
-    for (int i = 0; i < V; ++i) store_elem(p + i, in[i]);
 }
+
+// Bit image of one base element as an unsigned integer of the same width, and back.
+template <class B> FKD_DEV auto to_bits(B v) {
+    if constexpr (sizeof(B) == 1) return u32(__builtin_bit_cast(u8, v));
+    else if constexpr (sizeof(B) == 2) return u32(__builtin_bit_cast(u16, v));
+    else if constexpr (sizeof(B) == 4) return __builtin_bit_cast(u32, v);
+    else return __builtin_bit_cast(unsigned long long, v);
+}
+template <class T, int C> FKD_DEV base_t<T> chan_at(const T& v) { return chan<C>(v); }
+
+// Elements <-> packed dwords.  Every index is a compile-time constant (integer sequences, no loops over arrays
+// of sub-dword structs), so the element arrays never leave registers: byte extraction folds into
+// v_cvt_f32_ubyteN / v_bfe, packing into v_lshl_or / v_perm.
+template <class I, I... Is> struct IntSeq {};
+template <int N> using MakeSeq = __make_integer_seq<IntSeq, int, N>;
+
+template <int K, class T, int V> FKD_DEV base_t<T> run_elem(const Slot<T> (&in)[V]) {   // K-th base element of the run
+    return chan<K % cn_v<T>>(in[K / cn_v<T>].v);
+}
+template <int I, class T, int V> FKD_DEV u32 pack_word(const Slot<T> (&in)[V]) {        // I-th dword of the run
+    using B = base_t<T>;
+    if constexpr (sizeof(B) == 1) {
+        return to_bits(run_elem<4 * I>(in)) | (to_bits(run_elem<4 * I + 1>(in)) << 8) |
+               (to_bits(run_elem<4 * I + 2>(in)) << 16) | (to_bits(run_elem<4 * I + 3>(in)) << 24);
+    } else if constexpr (sizeof(B) == 2) {
+        return to_bits(run_elem<2 * I>(in)) | (to_bits(run_elem<2 * I + 1>(in)) << 16);
+    } else if constexpr (sizeof(B) == 4) {
+        return to_bits(run_elem<I>(in));
+    } else {
+        return u32(to_bits(run_elem<I / 2>(in)) >> (32 * (I % 2)));
+    }
+}
+template <class T, int V, int W, int... Is> FKD_DEV void pack_words_impl(const Slot<T> (&in)[V], u32 (&w)[W], IntSeq<int, Is...>) {
+    ((w[Is] = pack_word<Is>(in)), ...);
+}
+template <class T, int V, int W> FKD_DEV void pack_words(const Slot<T> (&in)[V], u32 (&w)[W]) {
+    pack_words_impl<T, V, W>(in, w, MakeSeq<W>{});
+}
+
+template <int K, class B, int W> FKD_DEV B unpack_elem(const u32 (&w)[W]) {       // K-th base element of the run
+    if constexpr (sizeof(B) == 1) return __builtin_bit_cast(B, u8((w[K / 4] >> (8 * (K % 4))) & 0xffu));
+    else if constexpr (sizeof(B) == 2) return __builtin_bit_cast(B, u16((w[K / 2] >> (16 * (K % 2))) & 0xffffu));
+    else if constexpr (sizeof(B) == 4) return __builtin_bit_cast(B, w[K]);
+    else return __builtin_bit_cast(B, (unsigned long long)w[2 * K] | ((unsigned long long)w[2 * K + 1] << 32));
+}
+template <int I, class T, int W> FKD_DEV T unpack_one(const u32 (&w)[W]) {        // I-th element of the run
+    using B = base_t<T>;
+    constexpr int N = cn_v<T>;
+    T o;
+    chan<0>(o) = unpack_elem<I * N, B>(w);
+    if constexpr (N > 1) chan<1>(o) = unpack_elem<I * N + 1, B>(w);
+    if constexpr (N > 2) chan<2>(o) = unpack_elem<I * N + 2, B>(w);
+    if constexpr (N > 3) chan<3>(o) = unpack_elem<I * N + 3, B>(w);
+    return o;
+}
+template <class T, int V, int W, int... Is> FKD_DEV void unpack_words_impl(const u32 (&w)[W], Slot<T> (&out)[V], IntSeq<int, Is...>) {
+    ((out[Is].v = unpack_one<Is, T>(w)), ...);
+}
+template <class T, int V, int W> FKD_DEV void unpack_words(const u32 (&w)[W], Slot<T> (&out)[V]) {
+    unpack_words_impl<T, V, W>(w, out, MakeSeq<V>{});
+}
+
+// V consecutive elements starting at p.  ALIGNED promises that p is dword aligned (the launcher checks every
+// row start of every plane on the host before it picks the kernel variant): the run then moves as one wide
+// access per <= 16 bytes (global_load_dwordx3 for four uchar3, dwordx4 for four floats), which consecutive
+// lanes make contiguous.  Without the promise, or when the run is not a whole number of dwords, elements move
+// one by one.
+template <class T> constexpr bool wide_ok(int v) {
+    const int bytes = int(sizeof(T)) * v;
+    return v > 1 && bytes % 4 == 0 && (bytes <= 16 || bytes % 16 == 0) && sizeof(T) == sizeof(base_t<T>) * cn_v<T>;
+}
+template <class T, int V, bool ALIGNED> FKD_DEV void load_run(const T* p, Slot<T> (&out)[V]) {
+    if constexpr (ALIGNED && wide_ok<T>(V)) {
+        constexpr int W = int(sizeof(T)) * V / 4;
+        u32 w[W];
+        load_words<W>(p, w);
+        if constexpr (sizeof(base_t<T>) < 4) {
+            // Keep each dword an opaque scalar: otherwise the optimiser rewrites "shift and mask a vector lane"
+            // into byte-vector extracts (<12 x i8>), which the backend can only legalise through scratch memory.
+#pragma unroll
+            for (int i = 0; i < W; ++i) asm("" : "+v"(w[i]));
+        }
+        unpack_words<T, V, W>(w, out);
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i].v = load_elem(p + i);
+    }
+}
+template <class T, int V, bool ALIGNED> FKD_DEV void store_run(T* p, const Slot<T> (&in)[V]) {
+    if constexpr (ALIGNED && wide_ok<T>(V)) {
+        constexpr int W = int(sizeof(T)) * V / 4;
+        u32 w[W];
+        pack_words<T, V, W>(in, w);
+        if constexpr (sizeof(base_t<T>) < 4) {
+            // Same reason as in load_run: keep the packed dwords opaque so the store stays one dwordx{2,3,4}
+            // instead of becoming a vector of 24-bit elements.
+#pragma unroll
+            for (int i = 0; i < W; ++i) asm("" : "+v"(w[i]));
+        }
+        store_words<W>(p, w);
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) store_elem(p + i, in[i].v);
+    }
+}
+
+FKD_HD bool dword_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 template <class T> FKD_DEV const T* row_ptr(const T* data, u32 pitch, int x, int y) {
     return reinterpret_cast<const T*>(reinterpret_cast<const char*>(data) + size_t(y) * pitch) + x;
@@ -180,13 +281,27 @@ template <class I, class O> struct SaturateCast {
     template <class S, class D> FKD_DEV static D sat(S s) {
         if constexpr (__is_same(S, D)) {
             return s;
+        } else if constexpr (__is_same(S, f32) && __is_same(D, u8)) {
+            // v_cvt_pk_u8_f32: round half to even, clamp to [0, 255], NaN -> 0 in one instruction.  Checked against
+            // the reference rule for all 2^32 float bit patterns (tests/test_gpu_saturate.py).
+            return u8(__builtin_amdgcn_cvt_pk_u8_f32(s, 0u, 0u));
         } else if constexpr (__is_floating_point(S) && __is_integral(D)) {
-            if (s != s) return D(0);
-            S r;  // round half to even under the default rounding mode (v_rndne_f32 / v_rndne_f64)
+            // Branch free.  Round half to even under the default rounding mode (v_rndne_f32 / v_rndne_f64), then
+            // clamp: fmax/fmin return the non-NaN operand, so NaN leaves the clamp as lo; for destination types whose
+            // bounds are exact in S (8/16-bit) the clamp alone is the saturation.
+            S r;
             if constexpr (sizeof(S) == 4) r = __builtin_rintf(s); else r = __builtin_rint(s);
-            if (r >= S(Lim<D>::hi)) return D(Lim<D>::hi);
-            if (r <= S(Lim<D>::lo)) return D(Lim<D>::lo);
-            return static_cast<D>(r);
+            if constexpr (sizeof(D) <= 2) {
+                if constexpr (sizeof(S) == 4) r = __builtin_fminf(__builtin_fmaxf(r, S(Lim<D>::lo)), S(Lim<D>::hi));
+                else r = __builtin_fmin(__builtin_fmax(r, S(Lim<D>::lo)), S(Lim<D>::hi));
+                const D v = static_cast<D>(static_cast<int>(r));
+                return (s != s) ? D(0) : v;
+            } else {
+                const bool over = r >= S(Lim<D>::hi), under = r <= S(Lim<D>::lo), nan = s != s;
+                const S safe = (over || under || nan) ? S(0) : r;
+                const D v = static_cast<D>(safe);
+                return nan ? D(0) : (over ? D(Lim<D>::hi) : (under ? D(Lim<D>::lo) : v));
+            }
         } else if constexpr (__is_integral(S) && __is_integral(D)) {
             const long long v = (long long)s;
             return v > Lim<D>::hi ? D(Lim<D>::hi) : (v < Lim<D>::lo ? D(Lim<D>::lo) : D(s));
@@ -274,8 +389,13 @@ template <class T> struct Read2D {
     FKD_DEV static T exec(int x, int y, int, const Params& p) {
         return detail::load_elem(detail::row_ptr(p.data, p.pitch, x, y));
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int, const Params& p, T (&out)[V]) {
-        detail::load_run<T, V>(detail::row_ptr(p.data, p.pitch, x, y), out);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<T> (&out)[V]) {
+        detail::load_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), out);
+    }
+    // True when every row start (shifted by xoff elements) is dword aligned: the launcher's licence to use
+    // the wide-access kernel variant.
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) {
+        return detail::dword_aligned(reinterpret_cast<const char*>(p.data) + ptrdiff_t(xoff) * ptrdiff_t(sizeof(T))) && p.pitch % 4 == 0;
     }
     // Staging hooks: the element as it lies in memory, and what the consumer sees of it.
     using Raw = T;
@@ -300,8 +420,12 @@ template <class T> struct Read3D {
     FKD_DEV static T exec(int x, int y, int z, const Params& p) {
         return detail::load_elem(detail::row_ptr(plane(p, z), p.pitch, x, y));
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, T (&out)[V]) {
-        detail::load_run<T, V>(detail::row_ptr(plane(p, z), p.pitch, x, y), out);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
+        detail::load_run<T, V, A>(detail::row_ptr(plane(p, z), p.pitch, x, y), out);
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) {
+        return detail::dword_aligned(reinterpret_cast<const char*>(p.data) + ptrdiff_t(xoff) * ptrdiff_t(sizeof(T))) && p.pitch % 4 == 0 &&
+               (size_t(p.plane_pitch) * p.color_planes) % 4 == 0;
     }
 #endif
 };
@@ -324,13 +448,14 @@ struct ReadNV12 {
         o.z = c[1];
         return o;
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i] = exec(x + i, y, z, p);
+        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
     using Raw = Out;
     FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
+    FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // gathers element-wise either way
 #endif
 };
 
@@ -345,9 +470,10 @@ template <class Back> struct Crop {
     FKD_DEV static int width(const Params& p) { return p.w; }
     FKD_DEV static int height(const Params& p) { return p.h; }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) { return Back::exec(x + p.x, y + p.y, 0, p.back); }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Out (&out)[V]) {
-        Back::template exec_row<V>(x + p.x, y + p.y, 0, p.back, out);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<Out> (&out)[V]) {
+        Back::template exec_row<V, A>(x + p.x, y + p.y, 0, p.back, out);
     }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff + p.x); }
     using Raw = typename Back::Raw;
     FKD_DEV static Raw exec_raw(int x, int y, int, const Params& p) { return Back::exec_raw(x + p.x, y + p.y, 0, p.back); }
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return Back::finish(r, p.back); }
@@ -367,12 +493,13 @@ template <class Back, class... Ops> struct FusedRead {
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
         return fold<Ops...>(Back::exec(x, y, z, p.back), p.ops);
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
-        typename Back::Out t[V];
-        Back::template exec_row<V>(x, y, z, p.back, t);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        Slot<typename Back::Out> t[V];
+        Back::template exec_row<V, A>(x, y, z, p.back, t);
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i] = fold<Ops...>(t[i], p.ops);
+        for (int i = 0; i < V; ++i) out[i].v = fold<Ops...>(t[i].v, p.ops);
     }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
     using Raw = typename Back::Raw;
     FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return Back::exec_raw(x, y, z, p.back); }
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return fold<Ops...>(Back::finish(r, p.back), p.ops); }
@@ -442,10 +569,11 @@ template <int AR, class Back> struct ResizeLinear {
         const Src d = Back::exec(t.x2r, t.y2r, z, p.back);
         return blend(a, b, c, d, t);
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i] = exec(x + i, y, z, p);
+        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
+    FKD_HD static bool rows_aligned(const Params&, int) { return true; }
 #endif
 };
 
@@ -460,8 +588,12 @@ template <int N, class PlaneOp> struct BatchRead {
     FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
-        PlaneOp::template exec_row<V>(x, y, z, p.plane[z], out);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        PlaneOp::template exec_row<V, A>(x, y, z, p.plane[z], out);
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) {
+        for (int i = 0; i < N; ++i) if (!PlaneOp::rows_aligned(p.plane[i], xoff)) return false;
+        return true;
     }
 #endif
 };
@@ -479,13 +611,17 @@ template <int N, class PlaneOp> struct BatchReadDefault {
         if (p.used <= z) return p.def;
         return PlaneOp::exec(x, y, z, p.plane[z]);
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Out (&out)[V]) {
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         if (p.used <= z) {
 #pragma unroll
-            for (int i = 0; i < V; ++i) out[i] = p.def;
+            for (int i = 0; i < V; ++i) out[i].v = p.def;
         } else {
-            PlaneOp::template exec_row<V>(x, y, z, p.plane[z], out);
+            PlaneOp::template exec_row<V, A>(x, y, z, p.plane[z], out);
         }
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) {
+        for (int i = 0; i < N && i < p.used; ++i) if (!PlaneOp::rows_aligned(p.plane[i], xoff)) return false;
+        return true;
     }
 #endif
 };
@@ -500,10 +636,11 @@ template <class T> struct ReadSet {
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static T exec(int, int, int, const Params& p) { return p.value; }
-    template <int V> FKD_DEV static void exec_row(int, int, int, const Params& p, T (&out)[V]) {
+    template <int V, bool A> FKD_DEV static void exec_row(int, int, int, const Params& p, Slot<T> (&out)[V]) {
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i] = p.value;
+        for (int i = 0; i < V; ++i) out[i].v = p.value;
     }
+    FKD_HD static bool rows_aligned(const Params&, int) { return true; }
 #endif
 };
 
@@ -520,9 +657,10 @@ template <class T> struct Write2D {
     FKD_DEV static void exec(int x, int y, int, const T& v, const Params& p) {
         detail::store_elem(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int, const T (&v)[V], const Params& p) {
-        detail::store_run<T, V>(detail::row_ptr(p.data, p.pitch, x, y), v);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int, const Slot<T> (&v)[V], const Params& p) {
+        detail::store_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
+    FKD_HD static bool rows_aligned(const Params& p) { return detail::dword_aligned(p.data) && p.pitch % 4 == 0; }
 #endif
 };
 
@@ -539,8 +677,11 @@ template <class T> struct TensorWrite {
     FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
         detail::store_elem(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const T (&v)[V], const Params& p) {
-        detail::store_run<T, V>(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
+        detail::store_run<T, V, A>(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
+    }
+    FKD_HD static bool rows_aligned(const Params& p) {
+        return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0;
     }
 #endif
 };
@@ -565,26 +706,30 @@ template <class T> struct TensorSplit {
         if constexpr (cn_v<T> > 2) w[2 * px] = chan<2>(v);
         if constexpr (cn_v<T> > 3) w[3 * px] = chan<3>(v);
     }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const T (&v)[V], const Params& p) {
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         B* w = at(p, x, y, z);
         const size_t px = size_t(p.width) * p.height;
-        B c0[V], c1[V];
+        Slot<B> c0[V], c1[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) { c0[i] = chan<0>(v[i]); c1[i] = chan<1>(v[i]); }
-        detail::store_run<B, V>(w, c0);
-        detail::store_run<B, V>(w + px, c1);
+        for (int i = 0; i < V; ++i) { c0[i].v = chan<0>(v[i].v); c1[i].v = chan<1>(v[i].v); }
+        detail::store_run<B, V, A>(w, c0);
+        detail::store_run<B, V, A>(w + px, c1);
         if constexpr (cn_v<T> > 2) {
-            B c2[V];
+            Slot<B> c2[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) c2[i] = chan<2>(v[i]);
-            detail::store_run<B, V>(w + 2 * px, c2);
+            for (int i = 0; i < V; ++i) c2[i].v = chan<2>(v[i].v);
+            detail::store_run<B, V, A>(w + 2 * px, c2);
         }
         if constexpr (cn_v<T> > 3) {
-            B c3[V];
+            Slot<B> c3[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) c3[i] = chan<3>(v[i]);
-            detail::store_run<B, V>(w + 3 * px, c3);
+            for (int i = 0; i < V; ++i) c3[i].v = chan<3>(v[i].v);
+            detail::store_run<B, V, A>(w + 3 * px, c3);
         }
+    }
+    FKD_HD static bool rows_aligned(const Params& p) {
+        return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 &&
+               (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
     }
 #endif
 };
@@ -596,8 +741,12 @@ template <int N, class W> struct BatchWrite {
     FKD_NAME("BatchWrite<" + istr(N) + "," + W::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, z, v, p.plane[z]); }
-    template <int V> FKD_DEV static void exec_row(int x, int y, int z, const In (&v)[V], const Params& p) {
-        W::template exec_row<V>(x, y, z, v, p.plane[z]);
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+        W::template exec_row<V, A>(x, y, z, v, p.plane[z]);
+    }
+    FKD_HD static bool rows_aligned(const Params& p) {
+        for (int i = 0; i < N; ++i) if (!W::rows_aligned(p.plane[i])) return false;
+        return true;
     }
 #endif
 };

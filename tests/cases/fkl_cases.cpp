@@ -26,12 +26,15 @@ using namespace fk;
 namespace {
 
 thread_local char g_error[2048] = "";
+thread_local int g_reps = 1;   // how many times the next chain is enqueued (benchmarks time the whole run)
 
 template <typename F> int guarded(F body) {
     try {
         body();
+        g_reps = 1;
         return 0;
     } catch (const std::exception& e) {
+        g_reps = 1;
         std::snprintf(g_error, sizeof(g_error), "%s", e.what());
         return 1;
     }
@@ -55,7 +58,7 @@ void crop_resize_par_u8(void* stream_, const uint8_t* src, int w, int h, int pit
     const auto in = dev2d<uchar3>(src, w, h, pitch);
     Tensor<uchar3> o(reinterpret_cast<uchar3*>(out), uint(dw), uint(dh), uint(B), 1, MemType::Device, 0);
     const auto crops = rects_from<B>(rects);
-    executeOperations<TransformDPP<>>(stream,
+    for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
         PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
         Crop<>::build(crops),
         Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(dw, dh), float3{bg[0], bg[1], bg[2]}),
@@ -73,7 +76,7 @@ void crop_resize_norm_split(void* stream_, const uint8_t* src, int w, int h, int
     const auto in = dev2d<uchar3>(src, w, h, pitch);
     Tensor<float> o(out, uint(dw), uint(dh), uint(B), 3, MemType::Device, 0);
     const auto crops = rects_from<B>(rects);
-    executeOperations<TransformDPP<>>(stream,
+    for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
         PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
         Crop<>::build(crops),
         Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
@@ -100,7 +103,7 @@ void batch_muladd_sat(void* stream_, const uint8_t* const* srcs, int w, int h, i
                         .then(Add<float3>::build(make_<float3>(add[3 * i], add[3 * i + 1], add[3 * i + 2])));
         outPtrs[i] = dev2d<uchar3>(outs[i], w, h, out_pitch);
     }
-    executeOperations<TransformDPP<>>(stream,
+    for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
         BatchRead<PlanePolicy::PROCESS_ALL>::build(planes),
         SaturateCast<float3, uchar3>::build(),
         PerThreadWrite<ND::_2D, uchar3>::build(outPtrs));
@@ -114,7 +117,7 @@ void add_mul_chain(Stream& stream, const Ptr2D<float>& in, const Ptr2D<float>& o
         if constexpr (decltype(idx)::value % 2 == 0) return Add<float>::build(addv);
         else return Mul<float>::build(mulv);
     };
-    executeOperations<DPP>(stream, PerThreadRead<ND::_2D, float>::build(in.ptr()),
+    for (int rep = 0; rep < g_reps; ++rep) executeOperations<DPP>(stream, PerThreadRead<ND::_2D, float>::build(in.ptr()),
                            pick(std::integral_constant<size_t, Is>{})...,
                            PerThreadWrite<ND::_2D, float>::build(out.ptr()));
 }
@@ -135,7 +138,7 @@ void crop_swap_u8(void* stream_, const uint8_t* src, int w, int h, int pitch, co
     const auto in = dev2d<uchar3>(src, w, h, pitch);
     Tensor<uchar3> o(reinterpret_cast<uchar3*>(out), uint(rects[2]), uint(rects[3]), uint(B), 1, MemType::Device, 0);
     const auto crops = rects_from<B>(rects);
-    executeOperations<TransformDPP<>>(stream,
+    for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
         PerThreadRead<ND::_2D, uchar3>::build(in.ptr()).then(Crop<>::build(crops)),
         ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, uchar3, uchar3>::build(),
         TensorWrite<uchar3>::build(o.ptr()));
@@ -146,6 +149,9 @@ void crop_swap_u8(void* stream_, const uint8_t* src, int w, int h, int pitch, co
 extern "C" {
 
 const char* fklcase_last_error(void) { return g_error; }
+// The next driver call on this thread enqueues its chain `reps` times back to back (through the full host API
+// each time); resets to 1 afterwards.
+void fklcase_set_reps(int reps) { g_reps = reps > 0 ? reps : 1; }
 
 int fklcase_crop_resize_par_u8_b5(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw,
                                   int dh, const float* bg, const float* mul, const float* sub, uint8_t* out) {
@@ -189,7 +195,7 @@ int fklcase_nv12_rgb_resize_split(void* stream_, const uint8_t* nv12, int w, int
         const Ptr2D<uchar> data(const_cast<uchar*>(nv12), uint(w), uint(h + h / 2), uint(pitch), MemType::Device, 0);
         const Image<PixelFormat::NV12> img(data, uint(w), uint(h));
         Tensor<float> o(out, uint(dw), uint(dh), 1, 3, MemType::Device, 0);
-        executeOperations<TransformDPP<>>(stream,
+        for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
             ReadYUV<PixelFormat::NV12>::build(img.ptr()),
             ConvertYUVToRGB<ColorDepth::p8bit, ColorRange::Full, ColorPrimitives::bt709>::build(),
             Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
