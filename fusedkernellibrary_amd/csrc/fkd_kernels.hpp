@@ -92,23 +92,51 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
 
 // ---- staged (LDS) bilinear kernel ----------------------------------------------------------------------
 
+// One staged source element in LDS: whole dwords, so a tap is one ds_read_b32 (uchar3, uchar, uchar4), b64 or b96.
 template <class Raw> struct LdsSlot {
     static constexpr int kWords = (int(sizeof(Raw)) + 3) / 4;
     u32 w[kWords];
 };
 template <class Raw> FKD_DEV LdsSlot<Raw> lds_pack(const Raw& r) {
     LdsSlot<Raw> s;
+    if constexpr (sizeof(base_t<Raw>) < 4 && sizeof(Raw) <= 4) {
+        // sub-dword element: assemble the dword in registers (bytes beyond the element are zero)
+        u32 word = 0;
+        if constexpr (sizeof(base_t<Raw>) == 1) {
+            word = detail::to_bits(chan<0>(r));
+            if constexpr (cn_v<Raw> > 1) word |= detail::to_bits(chan<1>(r)) << 8;
+            if constexpr (cn_v<Raw> > 2) word |= detail::to_bits(chan<2>(r)) << 16;
+            if constexpr (cn_v<Raw> > 3) word |= detail::to_bits(chan<3>(r)) << 24;
+        } else {
+            word = detail::to_bits(chan<0>(r));
+            if constexpr (cn_v<Raw> > 1) word |= detail::to_bits(chan<1>(r)) << 16;
+        }
+        s.w[0] = word;
+    } else {
 #pragma unroll
-    for (int i = 0; i < LdsSlot<Raw>::kWords; ++i) s.w[i] = 0;
-    __builtin_memcpy(&s, &r, sizeof(Raw));
+        for (int i = 0; i < LdsSlot<Raw>::kWords; ++i) s.w[i] = 0;
+        __builtin_memcpy(&s, &r, sizeof(Raw));
+    }
     return s;
 }
 template <class Raw> FKD_DEV Raw lds_unpack(const LdsSlot<Raw>& s) {
-    Raw r;
-    __builtin_memcpy(&r, &s, sizeof(Raw));
-    return r;
+    if constexpr (sizeof(base_t<Raw>) < 4 && sizeof(Raw) <= 4) {
+        u32 w[1] = {s.w[0]};
+        asm("" : "+v"(w[0]));   // keep the dword whole: one ds_read_b32, bytes come out with v_cvt_f32_ubyteN / v_bfe
+        return detail::unpack_one<0, Raw>(w);
+    } else {
+        Raw r;
+        __builtin_memcpy(&r, &s, sizeof(Raw));
+        return r;
+    }
 }
 
+#ifndef FKD_STAGED_XI
+#define FKD_STAGED_XI 2
+#endif
+#ifndef FKD_STAGED_YI
+#define FKD_STAGED_YI 2
+#endif
 constexpr int kStagedBX = 64;
 constexpr int kStagedBY = 4;
 
@@ -167,18 +195,20 @@ __global__ __launch_bounds__(kStagedBX * kStagedBY) void k_staged(const typename
             // Coordinates are clamped into the source, so even the predicated-off positions load in bounds.
             constexpr int RU = 2, CU = 2;
             for (int r0 = threadIdx.y; r0 < fh; r0 += kStagedBY * RU) {
+                typename Back::RawRow rows[RU];
+#pragma unroll
+                for (int i = 0; i < RU; ++i) {
+                    const int r = r0 + kStagedBY * i;
+                    rows[i] = Back::raw_row(fy0 + r < sh - 1 ? fy0 + r : sh - 1, z, q.back);
+                }
                 for (int c0 = threadIdx.x; c0 < fw; c0 += kStagedBX * CU) {
                     Raw v[RU][CU];
 #pragma unroll
-                    for (int i = 0; i < RU; ++i) {
-                        const int r = r0 + kStagedBY * i;
-                        const int sy = fy0 + r < sh - 1 ? fy0 + r : sh - 1;
+                    for (int j = 0; j < CU; ++j) {
+                        const int c = c0 + kStagedBX * j;
+                        const int sx = fx0 + c < sw - 1 ? fx0 + c : sw - 1;
 #pragma unroll
-                        for (int j = 0; j < CU; ++j) {
-                            const int c = c0 + kStagedBX * j;
-                            const int sx = fx0 + c < sw - 1 ? fx0 + c : sw - 1;
-                            v[i][j] = Back::exec_raw(sx, sy, z, q.back);
-                        }
+                        for (int i = 0; i < RU; ++i) v[i][j] = Back::raw_at(rows[i], sx, q.back);
                     }
 #pragma unroll
                     for (int i = 0; i < RU; ++i) {
@@ -195,32 +225,49 @@ __global__ __launch_bounds__(kStagedBX * kStagedBY) void k_staged(const typename
     }
     __syncthreads();
 
+    // Interpolation.  Everything that depends on the row only (source y, vertical weights, LDS row, output row
+    // address) is formed once per row; per pixel remain the horizontal coordinate, four weights, four LDS reads,
+    // the blend, the chain's compute operations and the store.  float(x1) and float(x1 + 1) are taken as floor(sx)
+    // and floor(sx) + 1, which are the same numbers (exact integers below 2^24).
 #pragma unroll
     for (int j = 0; j < YI; ++j) {
         const int y = ty0 + int(threadIdx.y) + kStagedBY * j;
         if (y >= ah) continue;
+        const typename W::RowRef orow = W::row(y, z, p.write);
+        bool yin = true;
+        if constexpr (RZ::kAR != IGNORE_AR) yin = y >= q.y1 && y <= q.y2;
+        const f32 sy = f32(y - oy) * q.fy;
+        const f32 fy1 = __builtin_floorf(sy);
+        const f32 ay = (fy1 + 1.0f) - sy, by = sy - fy1;
+        const int y1 = int(fy1);
+        const Slot* lrow0 = lds + (y1 - fy0) * fw - fx0;
+        const Slot* lrow1 = lrow0 + fw;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             const int x = tx0 + int(threadIdx.x) + kStagedBX * i;
             if (x >= aw) continue;
             typename RZ::Out v;
-            if (!RZ::inside(x, y, q)) {
+            bool in = yin;
+            if constexpr (RZ::kAR != IGNORE_AR) in = in && x >= q.x1 && x <= q.x2;
+            if (!in) {
                 v = q.bg;
             } else if (!staged) {
                 v = RZ::exec(x, y, z, q);
             } else {
-                const typename RZ::Taps tp = RZ::taps(x - ox, y - oy, q, sw, sh);
+                const f32 sx = f32(x - ox) * q.fx;
+                const f32 fx1 = __builtin_floorf(sx);
+                const f32 ax = (fx1 + 1.0f) - sx, bx = sx - fx1;
+                const int x1 = int(fx1);
+                typename RZ::Taps tp;
+                tp.w00 = ax * ay; tp.w10 = bx * ay; tp.w01 = ax * by; tp.w11 = bx * by;
                 // Unclamped +1 taps: the staged rectangle carries one replicated column/row past the edge.
-                const int c0 = tp.x1 - fx0, r0 = tp.y1 - fy0;
-                const Slot* row0 = lds + r0 * fw + c0;
-                const Slot* row1 = row0 + fw;
-                const auto a = Back::finish(lds_unpack<Raw>(row0[0]), q.back);
-                const auto b = Back::finish(lds_unpack<Raw>(row0[1]), q.back);
-                const auto c = Back::finish(lds_unpack<Raw>(row1[0]), q.back);
-                const auto d = Back::finish(lds_unpack<Raw>(row1[1]), q.back);
+                const auto a = Back::finish(lds_unpack<Raw>(lrow0[x1]), q.back);
+                const auto b = Back::finish(lds_unpack<Raw>(lrow0[x1 + 1]), q.back);
+                const auto c = Back::finish(lds_unpack<Raw>(lrow1[x1]), q.back);
+                const auto d = Back::finish(lds_unpack<Raw>(lrow1[x1 + 1]), q.back);
                 v = RZ::blend(a, b, c, d, tp);
             }
-            W::exec(x, y, z, Chain::compute(v, p), p.write);
+            W::put(orow, x, Chain::compute(v, p));
         }
     }
 }
@@ -270,7 +317,7 @@ template <class Chain>
 hipError_t launch_staged(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
     using Root = ResizeRoot<typename Chain::Read>;
     using Slot = LdsSlot<typename Root::Resize::BackOp::Raw>;
-    constexpr int XI = 2, YI = 2;
+    constexpr int XI = FKD_STAGED_XI, YI = FKD_STAGED_YI;
     constexpr int TW = kStagedBX * XI, TH = kStagedBY * YI;
     unsigned slots = 0;
     if constexpr (Root::batched) {

@@ -401,6 +401,10 @@ template <class T> struct Read2D {
     using Raw = T;
     FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
     FKD_DEV static T finish(const Raw& r, const Params&) { return r; }
+    // Row cursor for staging loops: the row address is formed once, each element costs one add.
+    struct RawRow { const T* p; };
+    FKD_DEV static RawRow raw_row(int y, int, const Params& p) { return RawRow{detail::row_ptr(p.data, p.pitch, 0, y)}; }
+    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params&) { return detail::load_elem(r.p + x); }
 #endif
 };
 
@@ -456,6 +460,18 @@ struct ReadNV12 {
     FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
     FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // gathers element-wise either way
+    struct RawRow { const u8* luma; const u8* chroma; };
+    FKD_DEV static RawRow raw_row(int y, int, const Params& p) {
+        return RawRow{p.data + size_t(y) * p.pitch, p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch};
+    }
+    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params&) {
+        Out o;
+        o.x = r.luma[x];
+        const u8* c = r.chroma + 2 * (x >> 1);
+        o.y = c[0];
+        o.z = c[1];
+        return o;
+    }
 #endif
 };
 
@@ -477,6 +493,9 @@ template <class Back> struct Crop {
     using Raw = typename Back::Raw;
     FKD_DEV static Raw exec_raw(int x, int y, int, const Params& p) { return Back::exec_raw(x + p.x, y + p.y, 0, p.back); }
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return Back::finish(r, p.back); }
+    using RawRow = typename Back::RawRow;
+    FKD_DEV static RawRow raw_row(int y, int, const Params& p) { return Back::raw_row(y + p.y, 0, p.back); }
+    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params& p) { return Back::raw_at(r, x + p.x, p.back); }
 #endif
 };
 
@@ -503,6 +522,9 @@ template <class Back, class... Ops> struct FusedRead {
     using Raw = typename Back::Raw;
     FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return Back::exec_raw(x, y, z, p.back); }
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return fold<Ops...>(Back::finish(r, p.back), p.ops); }
+    using RawRow = typename Back::RawRow;
+    FKD_DEV static RawRow raw_row(int y, int z, const Params& p) { return Back::raw_row(y, z, p.back); }
+    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params& p) { return Back::raw_at(r, x, p.back); }
 #endif
 };
 
@@ -661,6 +683,10 @@ template <class T> struct Write2D {
         detail::store_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
     FKD_HD static bool rows_aligned(const Params& p) { return detail::dword_aligned(p.data) && p.pitch % 4 == 0; }
+    // Row cursor: one address computation per row, one add per element.
+    struct RowRef { T* p; };
+    FKD_DEV static RowRef row(int y, int, const Params& p) { return RowRef{detail::row_ptr(p.data, p.pitch, 0, y)}; }
+    FKD_DEV static void put(const RowRef& r, int x, const T& v) { detail::store_elem(r.p + x, v); }
 #endif
 };
 
@@ -683,6 +709,9 @@ template <class T> struct TensorWrite {
     FKD_HD static bool rows_aligned(const Params& p) {
         return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0;
     }
+    struct RowRef { T* p; };
+    FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{detail::row_ptr(plane(p, z), p.pitch, 0, y)}; }
+    FKD_DEV static void put(const RowRef& r, int x, const T& v) { detail::store_elem(r.p + x, v); }
 #endif
 };
 
@@ -731,6 +760,15 @@ template <class T> struct TensorSplit {
         return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 &&
                (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
     }
+    struct RowRef { B* p; u32 px; };
+    FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), p.width * p.height}; }
+    FKD_DEV static void put(const RowRef& r, int x, const T& v) {
+        B* w = r.p + x;
+        w[0] = chan<0>(v);
+        w[r.px] = chan<1>(v);
+        if constexpr (cn_v<T> > 2) w[2u * size_t(r.px)] = chan<2>(v);
+        if constexpr (cn_v<T> > 3) w[3u * size_t(r.px)] = chan<3>(v);
+    }
 #endif
 };
 
@@ -748,6 +786,9 @@ template <int N, class W> struct BatchWrite {
         for (int i = 0; i < N; ++i) if (!W::rows_aligned(p.plane[i])) return false;
         return true;
     }
+    using RowRef = typename W::RowRef;
+    FKD_DEV static RowRef row(int y, int z, const Params& p) { return W::row(y, z, p.plane[z]); }
+    FKD_DEV static void put(const RowRef& r, int x, const In& v) { W::put(r, x, v); }
 #endif
 };
 

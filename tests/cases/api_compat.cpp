@@ -1,0 +1,148 @@
+// api_compat.cpp -- compile-only check that code written against the reference library's public API builds against
+// this backend's headers with a plain host compiler, and that host-side fusion produces the same TYPES the
+// reference documents (README "Sample code" walk-through; type expectations as in
+// utests/core/execution_model/utest_executors.h:36-89 and tests/algorithm/test_crop.h:23-46).
+#include <fused_kernel/core/execution_model/memory_operations.h>
+#include <fused_kernel/algorithms/basic_ops/arithmetic.h>
+#include <fused_kernel/algorithms/basic_ops/cast.h>
+#include <fused_kernel/algorithms/basic_ops/set.h>
+#include <fused_kernel/algorithms/image_processing/crop.h>
+#include <fused_kernel/algorithms/image_processing/color_conversion.h>
+#include <fused_kernel/algorithms/image_processing/resize.h>
+#include <fused_kernel/algorithms/image_processing/saturate.h>
+#include <fused_kernel/algorithms/image_processing/image.h>
+#include <fused_kernel/fused_kernel.h>
+#include <fused_kernel/core/execution_model/execution_model.h>
+#include <fused_kernel/algorithms/algorithms.h>
+
+#include <type_traits>
+
+using namespace fk;
+
+// ---- fusion types -------------------------------------------------------------------------------------------
+constexpr RawPtr<ND::_2D, uchar3> input{nullptr, {128, 128, 0}};
+constexpr auto readOp = PerThreadRead<ND::_2D, uchar3>::build({input});
+constexpr auto cropOp = Crop<>::build(Rect(0, 0, 16, 16));
+constexpr auto resizeOp = Resize<InterpolationType::INTER_LINEAR>::build(Size(1024, 1024));
+constexpr auto castU3F3 = Cast<uchar3, float3>::build();
+constexpr auto mulOpU3 = Mul<uchar3>::build(uchar3{2, 2, 2});
+constexpr auto mulOpF3 = Mul<float3>::build(float3{2, 2, 2});
+constexpr RawPtr<ND::_2D, float3> outputF3{nullptr, {1024, 1024, 0}};
+constexpr auto writeF3 = PerThreadWrite<ND::_2D, float3>::build({outputF3});
+
+static_assert(std::is_same_v<std::decay_t<decltype(readOp)>, Read<PerThreadRead<ND::_2D, uchar3>>>);
+static_assert(std::is_same_v<std::decay_t<decltype(cropOp)>, IncompleteReadBack<Crop<>>>);
+static_assert(std::is_same_v<std::decay_t<decltype(mulOpF3)>, Binary<Mul<float3, float3, float3, BinaryType>>>);
+static_assert(std::is_same_v<std::decay_t<decltype(castU3F3)>, Unary<Cast<uchar3, float3>>>);
+
+// read & crop -> ReadBack<Crop<Read<...>>>
+static_assert(std::is_same_v<std::decay_t<decltype(readOp.then(cropOp))>, ReadBack<Crop<std::decay_t<decltype(readOp)>>>>);
+static_assert(std::is_same_v<std::decay_t<decltype(readOp & cropOp)>, std::decay_t<decltype(fuse(readOp, cropOp))>>);
+
+void fusion_types() {
+    // no read-back in the list: nothing is fused
+    const auto t1 = BackFuser::fuse_back(readOp, castU3F3, mulOpF3, writeF3);
+    static_assert(std::is_same_v<std::decay_t<decltype(get<0>(t1))>, std::decay_t<decltype(readOp)>>);
+    // read, crop, compute, write: the crop is pulled into the read
+    const auto t2 = BackFuser::fuse_back(readOp, cropOp, castU3F3, writeF3);
+    static_assert(std::is_same_v<std::decay_t<decltype(get<0>(t2))>, ReadBack<Crop<std::decay_t<decltype(readOp)>>>>);
+    static_assert(std::tuple_size_v<std::decay_t<decltype(t2)>> == 3);
+    // read, crop, compute, resize, ...: everything up to the resize becomes the resize's source
+    const auto t3 = BackFuser::fuse_back(readOp, cropOp, mulOpU3, resizeOp, mulOpF3, writeF3);
+    using Fused3 = std::decay_t<decltype(get<0>(t3))>;
+    using Expected3 = ReadBack<ResizeComplete<AspectRatio::IGNORE_AR, Ternary<InterpolateComplete<InterpolationType::INTER_LINEAR,
+        Read<FusedOperation<ReadBack<Crop<Read<PerThreadRead<ND::_2D, uchar3>>>>, Binary<Mul<uchar3>>>>>>>>;
+    static_assert(std::is_same_v<Fused3, Expected3>);
+    static_assert(Fused3::Operation::BackIOp::Operation::BackIOp::Operation::IS_FUSED_OP);
+    (void)t1; (void)t2; (void)t3;
+}
+
+void batch_types() {
+    constexpr std::array<Rect, 2> crops{Rect(0, 0, 34, 25), Rect(10, 10, 70, 15)};
+    const auto batchCrop = Crop<>::build(crops);
+    static_assert(std::is_same_v<std::decay_t<decltype(batchCrop)>, Read<BatchRead<PlanePolicy::PROCESS_ALL, 2, TypeList<Crop<>>>>>);
+    const auto fused = readOp.then(batchCrop).then(Resize<InterpolationType::INTER_LINEAR>::build(Size(100, 100)));
+    using F = std::decay_t<decltype(fused)>;
+    static_assert(isBatchOperation<F::Operation> && F::Operation::BATCH == 2);
+    const ActiveThreads at = fused.getActiveThreads();   // 100 x 100 x 2, as tests/algorithm/test_crop.h expects
+    (void)at;
+    static_assert(std::is_same_v<F, Read<BatchRead<PlanePolicy::PROCESS_ALL, 2,
+        ResizeComplete<AspectRatio::IGNORE_AR, Ternary<InterpolateComplete<InterpolationType::INTER_LINEAR,
+            ReadBack<Crop<Read<PerThreadRead<ND::_2D, uchar3>>>>>>>>>>);
+}
+
+// ---- the README program, as written there ------------------------------------------------------------------
+void readme_program() {
+    Stream stream;
+    constexpr Size outputSize(60, 60);
+    constexpr int BATCH = 5;
+    Ptr2D<uchar3> inputImage(3840, 2160);
+    Tensor<float3> output(outputSize.width, outputSize.height, BATCH);
+    constexpr std::array<Rect, BATCH> crops{Rect(0, 0, 34, 25), Rect(10, 10, 70, 15), Rect(20, 20, 60, 59),
+                                            Rect(30, 30, 20, 23), Rect(40, 40, 12, 11)};
+    constexpr float3 backgroundColor{0.f, 0.f, 0.f};
+    constexpr float3 mulValue = make_set<float3>(1.4f);
+    constexpr float3 subValue = make_set<float3>(0.5f);
+    constexpr float3 divValue = make_set<float3>(255.f);
+    const auto mySender = PerThreadRead<ND::_2D, uchar3>::build(inputImage)
+                              .then(Crop<>::build(crops))
+                              .then(Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(outputSize, backgroundColor))
+                              .then(Mul<float3>::build(mulValue))
+                              .then(Sub<float3>::build(subValue))
+                              .then(Div<float3>::build(divValue))
+                              .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
+    const auto myReceiver = TensorWrite<float3>::build(output);
+    executeOperations<fk::TransformDPP<>>(stream, mySender, myReceiver);
+    stream.sync();
+}
+
+// ---- the compiler-explorer example: executeOperations(input, stream, ops...) --------------------------------
+void lts_example() {
+    Ptr2D<uchar4> in(1920, 1080);
+    std::array<Rect, 5> crops{Rect(0, 0, 120, 40), Rect(100, 200, 60, 40), Rect(400, 20, 30, 50), Rect(1000, 800, 30, 30), Rect(40, 40, 40, 40)};
+    Tensor<uchar4> output(64, 64, 5);
+    Stream stream;
+    executeOperations<TransformDPP<>>(in, stream, Crop<>::build(crops), Resize<InterpolationType::INTER_LINEAR>::build(Size(64, 64)),
+                                      Mul<float4>::build(make_set<float4>(1.f / 255.f)), Mul<float4>::build(make_set<float4>(0.33f)),
+                                      Add<float4>::build(make_set<float4>(0.5f)), Mul<float4>::build(make_set<float4>(255.f)),
+                                      SaturateCast<float4, uchar4>::build(), TensorWrite<uchar4>::build(output));
+    stream.sync();
+}
+
+// ---- two spellings of read -> crop -> resize -> mul, and the (input, output, stream, ops...) overload --------
+void two_spellings() {
+    Stream stream;
+    Ptr2D<float2> in(1920, 1080), out1(16, 16), out2(16, 16);
+    in.at(3, 4) = make_<float2>(3.f, 4.f);
+    in.upload(stream);
+    const auto r = PerThreadRead<ND::_2D, float2>::build(in);
+    const auto c = Crop<>::build(Rect(128, 256, 64, 64));
+    const auto z = Resize<InterpolationType::INTER_LINEAR>::build(Size(16, 16));
+    const auto m = Mul<float2>::build(make_<float2>(3.f, 5.f));
+    Executor<TransformDPP<>>::executeOperations(stream, r, c, z, m, PerThreadWrite<ND::_2D, float2>::build(out1));
+    Executor<TransformDPP<>>::executeOperations(stream, r.then(c).then(z), m, PerThreadWrite<ND::_2D, float2>::build(out2));
+    out1.download(stream);
+    stream.sync();
+    Ptr2D<float> a(64, 64), b(64, 64);
+    executeOperations<TransformDPP<ParArch::GPU_AMD, TF::ENABLED>>(a, b, stream, Add<float>::build(0.5f), Mul<float>::build(2.f));
+    const bool same = out1.at(0, 0) == out2.at(0, 0);
+    (void)same;
+}
+
+// ---- horizontal fusion over separate images, NV12 --------------------------------------------------------------
+void batch_and_video() {
+    Stream stream;
+    std::array<Ptr2D<uchar3>, 3> ins{Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32)};
+    std::array<Ptr2D<uchar3>, 3> outs{Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32)};
+    executeOperations<TransformDPP<>>(ins, stream, Cast<uchar3, float3>::build(), Mul<float3>::build(make_set<float3>(2.f)),
+                                      SaturateCast<float3, uchar3>::build(), PerThreadWrite<ND::_2D, uchar3>::build(outs));
+    Tensor<float3> t(64, 32, 3);
+    executeOperations<TransformDPP<>>(ins, t, stream, Cast<uchar3, float3>::build());
+    Image<PixelFormat::NV12> frame(256, 128);
+    Tensor<float> planar(128, 64, 1, 3);
+    executeOperations<TransformDPP<>>(stream, ReadYUV<PixelFormat::NV12>::build(frame),
+                                      ConvertYUVToRGB<ColorDepth::p8bit, ColorRange::Full, ColorPrimitives::bt709>::build(),
+                                      Resize<InterpolationType::INTER_LINEAR>::build(Size(128, 64)), Mul<float3, float>::build(1.f / 255.f),
+                                      TensorSplit<float3>::build(planar));
+    stream.sync();
+}
