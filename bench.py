@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused data-parallel path on one MI355X.
+
+A step is ONE pass of the hot path over one batch of synthetic input already resident in HBM: the DNN
+preprocessing chain of configuration 3 (64 crops of a 1920x1080 BGR image -> bilinear resize to 224x224 ->
+BGR->RGB -> (x - mean) / std -> planar float32 64x3x224x224), issued through the C++ host API
+(executeOperations<TransformDPP<>>) -> C ABI -> one gfx950 kernel.
+
+Prints ONE JSON line.  `value` is output Mpix/s of the whole job; `roofline` prices the kernel's algorithmic bytes
+against the 8 TB/s HBM peak using the launch duration measured with HIP events on the launch stream;
+`cpu_baseline` is the same chain on the reference library's single-threaded CPU backend (oracle/_ref, when built)
+or on the plain-C oracle, timed on this machine's host cores.  `others` carries the same measurements for the
+remaining four configurations.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5 (c3 is always run)")
+    return ap.parse_args()
+
+
+class Timer:
+    """K back-to-back launches through the host API, bracketed by events on the launch stream and by wall clock."""
+
+    def __init__(self, torch, fkl, cases):
+        self.torch, self.fkl, self.cases = torch, fkl, cases
+        self.lib = fkl.lib()
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        fkl.check(self.lib.fklhip_event_create(C.byref(self.e0)), "event_create")
+        fkl.check(self.lib.fklhip_event_create(C.byref(self.e1)), "event_create")
+
+    def run(self, fn, steps, warmup):
+        torch = self.torch
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        if warmup > 0:
+            self.cases.set_reps(warmup)
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        self.fkl.check(self.lib.fklhip_event_record(self.e0, stream), "event_record")
+        self.cases.set_reps(steps)
+        fn()
+        self.fkl.check(self.lib.fklhip_event_record(self.e1, stream), "event_record")
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        ms = C.c_float()
+        self.fkl.check(self.lib.fklhip_event_elapsed_ms(C.byref(ms), self.e0, self.e1), "event_elapsed")
+        return wall_ms / steps, ms.value / steps   # per step: wall clock, device events
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this path runs on ONE GPU (asked for {args.gpus}); every output pixel is independent, "
+              "so more GPUs would only split the batch. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import fusedkernellibrary_amd as fkl
+    from fusedkernellibrary_amd import cases, workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    fkl.lib()   # raises if the HIP library is missing: there is no fallback
+    dev = torch.device("cuda:0")
+    timer = Timer(torch, fkl, cases)
+    only = set(filter(None, args.only.split(","))) or {"c1", "c2", "c3", "c4", "c5"}
+    results = {}
+
+    def record(name, out_px, alg_bytes, fn, steps, warmup):
+        wall_ms, dev_ms = timer.run(fn, steps, warmup)
+        ll = fkl.last_launch()
+        results[name] = {
+            "mpix_per_s": out_px / 1e6 / (wall_ms * 1e-3),
+            "ms_per_step": wall_ms,
+            "kernel_us": dev_ms * 1e3,
+            "algorithmic_bytes": alg_bytes,
+            "achieved_gbs": alg_bytes / (dev_ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": alg_bytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "kernel": ll["kernel"], "grid": ll["grid"], "block": ll["block"], "lds_bytes": ll["lds_bytes"],
+        }
+        return results[name]
+
+    # ---- configuration 3: the headline workload -------------------------------------------------------------
+    c3 = wl.config3()
+    union_px = wl.config3_union_pixels(c3["rects"], 1920, 1080)
+    a3 = 64 * 3 * 224 * 224 * 4 + 3 * union_px
+    src3 = torch.from_numpy(c3["src"]).to(dev)
+    out3 = torch.zeros((64, 3, 224, 224), dtype=torch.float32, device=dev)
+    f3 = lambda: cases.crop_resize_norm_split(src3, c3["rects"], c3["dst"], c3["sub"], c3["div"], out3)
+    r3 = record("c3", 64 * 224 * 224, a3, f3, args.steps, args.warmup)
+    got3 = out3.cpu().numpy()
+
+    # ---- the other four configurations (reported under "others") ------------------------------------------------
+    if "c1" in only:
+        c = wl.config1()
+        s = torch.from_numpy(c["src"]).to(dev)
+        o = torch.zeros((5, 64, 128, 3), dtype=torch.uint8, device=dev)
+        a1 = 128 * 64 * 5 * 3 + int((c["rects"][:, 2] * c["rects"][:, 3]).sum()) * 3
+        record("c1", 128 * 64 * 5, a1, lambda: cases.crop_resize_par_u8(s, c["rects"], c["dst"], c["bg"], c["mul"], c["sub"], o),
+               args.steps, args.warmup)
+    if "c2" in only:
+        c = wl.config2()
+        s = torch.from_numpy(c["src"]).to(dev)
+        o = torch.zeros_like(s)
+        for n in c["n_ops"]:
+            record(f"c2_n{n}", 3840 * 2160, 2 * 3840 * 2160 * 4, lambda n=n: cases.add_mul_chain(s, n, c["add"], c["mul"], o),
+                   args.steps, args.warmup)
+        record("copy_f32_4k", 3840 * 2160, 2 * 3840 * 2160 * 4, lambda: cases.copy_f32(s, o), args.steps, args.warmup)
+    if "c5" in only:
+        c = wl.config5()
+        s = torch.from_numpy(c["nv12"]).to(dev)
+        o = torch.zeros((3, 1080, 1920), dtype=torch.float32, device=dev)
+        record("c5", 1920 * 1080, 3840 * 2160 * 3 // 2 + 3 * 1080 * 1920 * 4,
+               lambda: cases.nv12_rgb_resize_split(s, c["width"], c["height"], c["dst"], c["scale"], o), args.steps, args.warmup)
+    if "c4" in only:
+        # 100 images of uniform random bytes (generated on the GPU: the content does not affect the timing and the
+        # seeded host generator of the parity tests needs several seconds for 622 MB)
+        g = torch.Generator(device=dev)
+        g.manual_seed(4)
+        srcs = [torch.randint(0, 256, (1080, 1920, 3), dtype=torch.uint8, device=dev, generator=g) for _ in range(100)]
+        outs = [torch.empty_like(t) for t in srcs]
+        p = wl.RawMT(44)
+        mul = np.stack([p.range_floats(3, 0.5, 2.0) for _ in range(100)])
+        add = np.stack([p.range_floats(3, -64.0, 64.0) for _ in range(100)])
+        record("c4", 100 * 1920 * 1080, 2 * 100 * 1920 * 1080 * 3, lambda: cases.batch_muladd_sat(srcs, mul, add, outs),
+               max(10, args.steps // 10), max(2, args.warmup // 10))
+        del srcs, outs
+
+    # ---- CPU baseline: the same chain on this machine's host cores, one thread, bounded sample --------------------
+    cpu = None
+    if not args.no_cpu:
+        import oracle_lib as ol
+        kind = "reference" if ol.have_ref() else "port"
+        fn = ol.ref_crop_resize_norm_split if kind == "reference" else ol.oracle_crop_resize_norm_split
+        want = fn(c3["src"], c3["rects"], c3["dst"], c3["sub"], c3["div"])   # warm-up, and the parity check of this run
+        if want.tobytes() != got3.tobytes():
+            denom = np.maximum(np.abs(want), np.float32(1e-30))
+            rel = float(np.max(np.abs(got3 - want) / denom))
+            if rel > 1e-5:
+                print(f"bench.py: GPU output differs from the CPU baseline (max rel {rel:.3e})", file=sys.stderr)
+                sys.exit(3)
+        iters, t_total = 0, 0.0
+        best = 1e9
+        while t_total < 12.0 and iters < 200:
+            t0 = time.perf_counter()
+            fn(c3["src"], c3["rects"], c3["dst"], c3["sub"], c3["div"])
+            dt = time.perf_counter() - t0
+            best = min(best, dt)
+            t_total += dt
+            iters += 1
+        cpu = {"value": 64 * 224 * 224 / 1e6 / best, "unit": "Mpix/s", "cores": 1, "kind": kind,
+               "sample": f"configuration 3 at full size, best of {iters} single-threaded passes ({t_total:.1f} s of CPU work)",
+               "ms_per_step": best * 1e3}
+
+    line = {
+        "metric": "fused-pipeline output Mpix/s (DNN preprocessing batch, configuration 3) on 1 MI355X",
+        "value": r3["mpix_per_s"], "unit": "Mpix/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": r3["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic (seeded uniform random pixels and crop rectangles)",
+        "config": {"workload": "configs[2]: 64 crops of uchar3 BGR 1920x1080 -> bilinear 224x224 IGNORE_AR -> BGR2RGB -> "
+                               "(x-mean)/std -> TensorSplit planar float32 64x3x224x224, one fused launch per step",
+                   "output_pixels_per_step": 64 * 224 * 224, "union_source_pixels": union_px},
+        "roofline": {"bound": "hbm", "achieved": r3["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": r3["frac_of_hbm_peak"], "traffic": TRAFFIC_C3_BYTES,
+                     "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"]},
+        "cpu_baseline": cpu,
+        "others": {k: v for k, v in results.items() if k != "c3"},
+    }
+    print(json.dumps(line))
+
+
+# HBM bytes one launch of configuration 3 moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE scaled by what the
+# same counters read for the plain copy chain of known size (profiles/k_staged_config3_traffic.txt); None until measured.
+TRAFFIC_C3_BYTES = 51689000
+
+if __name__ == "__main__":
+    main()

@@ -97,3 +97,8 @@ def crop_swap_u8(src, rects, out):
     r = _host(rects, np.int32)
     _ok(cases().fklcase_crop_swap_u8_b4(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0),
                                         r.ctypes.data_as(C.c_void_p), _p(out)))
+
+
+def copy_f32(src, out):
+    """src/out (H,W) f32 cuda: read -> write with no compute operation."""
+    _ok(cases().fklcase_copy_f32(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, _p(out), out.stride(0) * 4))

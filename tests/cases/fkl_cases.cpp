@@ -203,6 +203,15 @@ int fklcase_nv12_rgb_resize_split(void* stream_, const uint8_t* nv12, int w, int
             TensorSplit<float3>::build(o.ptr()));
     });
 }
+// Plain pitched copy of a float image: read, no compute operation, write.
+int fklcase_copy_f32(void* stream_, const float* in, int w, int h, int pitch, float* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<float>(in, w, h, pitch);
+        const auto o = dev2d<float>(out, w, h, out_pitch);
+        for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(i, o, stream);
+    });
+}
 int fklcase_crop_swap_u8_b4(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
     return guarded([&] { crop_swap_u8<4>(stream, src, w, h, pitch, rects, out); });
 }
