@@ -9,13 +9,13 @@
 //                 Plane z = workgroup index in z: horizontal (batch) fusion, per-plane parameters are wave
 //                 uniform and come out of the kernel-argument segment through scalar loads.
 //
-//  staged kernel  for chains whose read is a bilinear resize: a workgroup owns a TW x TH tile of the output of
-//                 one plane, first copies the source rectangle its taps fall in into LDS (replicating the last
-//                 column/row once, which reproduces the reference's clamp of the +1 taps), then interpolates
-//                 out of LDS.  Source pixels are staged raw (as they lie in memory, one dword per uchar3) and
-//                 whatever was fused into the read (colour conversion, per-plane arithmetic) is applied per tap,
-//                 in the reference's order.  Workgroups are renumbered so each XCD works on a contiguous run of
-//                 tiles and planes and its L2 sees one set of crops.
+//  gather kernel  for chains whose read is a bilinear resize: a workgroup owns a tile of the output of one plane,
+//                 a wave owns whole output rows of it, so source rows, vertical weights and all row addresses are
+//                 wave uniform (scalar registers); a lane reads the four taps of each of its pixels straight from
+//                 global memory as whole elements at byte granularity.  Whatever was fused into the read (colour
+//                 conversion, per-plane arithmetic) is applied per tap, in the reference's order.  Workgroups are
+//                 renumbered so each XCD works on a contiguous run of a plane's tiles and its L2 sees the source
+//                 rows those tiles share.
 //
 // Reference being replaced: TransformDPP<GPU_NVIDIA>::exec and launchTransformDPP_Kernel,
 // FK/core/execution_model/data_parallel_patterns.h:223-242 and executor_details/executor_kernels.h:26-30;
@@ -23,6 +23,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include <fkd/launch_info.hpp>
 #include <fkd/ops.hpp>
@@ -43,9 +45,9 @@ template <int N, int AR, class Back> struct ResizeRoot<BatchRead<N, ResizeLinear
     using Resize = ResizeLinear<AR, Back>;
 };
 
-template <class Chain> constexpr bool is_staged_chain() {
+template <class Chain> constexpr bool is_gather_chain() {
     if constexpr (ResizeRoot<typename Chain::Read>::value)
-        return ResizeRoot<typename Chain::Read>::Resize::BackOp::kStageable;
+        return ResizeRoot<typename Chain::Read>::Resize::BackOp::kTapCursor;
     else
         return false;
 }
@@ -78,204 +80,165 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
             const int y = ybase + r;
             Slot<typename Chain::Value> out[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) out[i].v = Chain::compute(in[r][i].v, p);
+            for (int i = 0; i < V; ++i) out[i].v = Chain::compute_checked(in[r][i].v, p);
             if (y < ah) W::template exec_row<V, ALIGNED>(x0, y, z, out, p.write);
         }
     } else {
         for (int r = 0; r < ROWS; ++r) {
             const int y = ybase + r;
             if (y >= ah) break;
-            for (int x = x0; x < aw; ++x) W::exec(x, y, z, Chain::compute(R::exec(x, y, z, p.read), p), p.write);
+            for (int x = x0; x < aw; ++x) W::exec(x, y, z, Chain::compute_checked(R::exec(x, y, z, p.read), p), p.write);
         }
     }
 }
 
-// ---- staged (LDS) bilinear kernel ----------------------------------------------------------------------
+// ---- gather bilinear kernel ----------------------------------------------------------------------------
 
-// One staged source element in LDS: whole dwords, so a tap is one ds_read_b32 (uchar3, uchar, uchar4), b64 or b96.
-template <class Raw> struct LdsSlot {
-    static constexpr int kWords = (int(sizeof(Raw)) + 3) / 4;
-    u32 w[kWords];
-};
-template <class Raw> FKD_DEV LdsSlot<Raw> lds_pack(const Raw& r) {
-    LdsSlot<Raw> s;
-    if constexpr (sizeof(base_t<Raw>) < 4 && sizeof(Raw) <= 4) {
-        // sub-dword element: assemble the dword in registers (bytes beyond the element are zero)
-        u32 word = 0;
-        if constexpr (sizeof(base_t<Raw>) == 1) {
-            word = detail::to_bits(chan<0>(r));
-            if constexpr (cn_v<Raw> > 1) word |= detail::to_bits(chan<1>(r)) << 8;
-            if constexpr (cn_v<Raw> > 2) word |= detail::to_bits(chan<2>(r)) << 16;
-            if constexpr (cn_v<Raw> > 3) word |= detail::to_bits(chan<3>(r)) << 24;
-        } else {
-            word = detail::to_bits(chan<0>(r));
-            if constexpr (cn_v<Raw> > 1) word |= detail::to_bits(chan<1>(r)) << 16;
-        }
-        s.w[0] = word;
-    } else {
-#pragma unroll
-        for (int i = 0; i < LdsSlot<Raw>::kWords; ++i) s.w[i] = 0;
-        __builtin_memcpy(&s, &r, sizeof(Raw));
-    }
-    return s;
-}
-template <class Raw> FKD_DEV Raw lds_unpack(const LdsSlot<Raw>& s) {
-    if constexpr (sizeof(base_t<Raw>) < 4 && sizeof(Raw) <= 4) {
-        u32 w[1] = {s.w[0]};
-        asm("" : "+v"(w[0]));   // keep the dword whole: one ds_read_b32, bytes come out with v_cvt_f32_ubyteN / v_bfe
-        return detail::unpack_one<0, Raw>(w);
-    } else {
-        Raw r;
-        __builtin_memcpy(&r, &s, sizeof(Raw));
-        return r;
-    }
-}
-
-#ifndef FKD_STAGED_XI
-#define FKD_STAGED_XI 2
+#ifndef FKD_GATHER_XI
+#define FKD_GATHER_XI 2
 #endif
-#ifndef FKD_STAGED_YI
-#define FKD_STAGED_YI 2
+#ifndef FKD_GATHER_YI
+#define FKD_GATHER_YI 4
 #endif
-constexpr int kStagedBX = 64;
-constexpr int kStagedBY = 4;
+constexpr int kGatherBX = 64;
+constexpr int kGatherBY = 4;
 
-struct StagedGeom {
-    u32 tiles_x, tiles_y, n_tiles, lds_slots;
+struct TileGeom {
+    u32 tiles_x, tiles_y, n_tiles;
 };
 
-// XI, YI: outputs per thread along x (stride 64) and y (stride 4): tile = 64*XI by 4*YI outputs.
+// A workgroup owns a (64*XI) x (4*YI) tile of the output of one plane; wave w owns rows w*YI .. w*YI+YI-1 of it, so
+// everything that depends on the row (source rows, vertical weights, row addresses of source and destination) is
+// wave uniform and lives in scalar registers.  A lane produces XI pixels (64 apart, so stores of a wave are
+// contiguous) in each of its YI rows; the horizontal coordinate work is shared by the rows.  The four taps of a
+// pixel are read straight from global memory as whole elements (a uchar3 comes in as one dword whose top byte is
+// ignored); neighbouring lanes and rows hit the same cache lines, so HBM sees each source line about once.
+// All loads of a lane are issued before the first use and are unconditional (coordinates are clamped into the
+// source); only stores are predicated.
 template <class Chain, int XI, int YI>
-__global__ __launch_bounds__(kStagedBX * kStagedBY) void k_staged(const typename Chain::Params p, const StagedGeom g) {
+__global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename Chain::Params p, const TileGeom g) {
     using Root = ResizeRoot<typename Chain::Read>;
     using RZ = typename Root::Resize;
     using Back = typename RZ::BackOp;
     using Raw = typename Back::Raw;
-    using Slot = LdsSlot<Raw>;
     using W = typename Chain::Write;
-    constexpr int TW = kStagedBX * XI, TH = kStagedBY * YI;
-    extern __shared__ u32 lds_words[];
-    Slot* lds = reinterpret_cast<Slot*>(lds_words);
+    constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
 
-    // Renumber workgroups: hardware deals consecutive workgroup ids round-robin to the 8 XCDs; give XCD k the
-    // k-th contiguous eighth of the tile list so neighbouring tiles (which share source rows) share an L2.
-    const u32 chunk = (g.n_tiles + 7u) / 8u;
-    const u32 t = (blockIdx.x % 8u) * chunk + blockIdx.x / 8u;
-    if (t >= g.n_tiles || blockIdx.x / 8u >= chunk) return;
+    // The plane is the grid's z index, known at wave start, so the plane's parameters are fetched together with the
+    // first kernel arguments instead of after them.  Within a plane workgroups are renumbered: hardware deals
+    // consecutive workgroup ids round-robin to the 8 XCDs (the grid's x extent is a multiple of 8); XCD k gets the
+    // k-th contiguous eighth of the plane's tiles so neighbouring tiles (which share source rows) share an L2.
+    const int z = int(blockIdx.z);
     const u32 per_plane = g.tiles_x * g.tiles_y;
-    const int z = int(t / per_plane);
-    const u32 tin = t % per_plane;
+    const u32 chunk = (per_plane + 7u) / 8u;
+    const u32 tin = (blockIdx.x % 8u) * chunk + blockIdx.x / 8u;
+    if (tin >= per_plane) return;
     const int tx0 = int(tin % g.tiles_x) * TW;
-    const int ty0 = int(tin / g.tiles_x) * TH;
+    const int wy = __builtin_amdgcn_readfirstlane(int(threadIdx.y));
+    const int y0 = int(tin / g.tiles_x) * TH + wy * YI;
 
     const typename RZ::Params* rp;
     if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
     const typename RZ::Params& q = *rp;
     const int aw = int(p.active_w), ah = int(p.active_h);
-
-    // Output range of this tile that actually interpolates (inside the letterbox), relative to its origin.
-    int ox = 0, oy = 0, lx2 = aw - 1, ly2 = ah - 1;
-    if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; lx2 = q.x2 < lx2 ? q.x2 : lx2; ly2 = q.y2 < ly2 ? q.y2 : ly2; }
-    const int xs = (tx0 > ox ? tx0 : ox) - ox;
-    const int ys = (ty0 > oy ? ty0 : oy) - oy;
-    const int xe = (tx0 + TW - 1 < lx2 ? tx0 + TW - 1 : lx2) - ox;
-    const int ye = (ty0 + TH - 1 < ly2 ? ty0 + TH - 1 : ly2) - oy;
+    if (y0 >= ah) return;
+    int ox = 0, oy = 0;
+    if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; }
     const int sw = Back::width(q.back), sh = Back::height(q.back);
 
-    int fx0 = 0, fy0 = 0, fw = 0, fh = 0;
-    bool staged = false;
-    if (xs <= xe && ys <= ye) {
-        fx0 = int(__builtin_floorf(f32(xs) * q.fx));
-        fy0 = int(__builtin_floorf(f32(ys) * q.fy));
-        fw = int(__builtin_floorf(f32(xe) * q.fx)) + 1 - fx0 + 1;
-        fh = int(__builtin_floorf(f32(ye) * q.fy)) + 1 - fy0 + 1;
-        staged = fx0 >= 0 && fy0 >= 0 && fw > 0 && fh > 0 && u32(fw) * u32(fh) <= g.lds_slots;
-        if (staged) {
-            // RU x CU raw elements per thread and step: all their loads are issued before the first LDS write.
-            // Coordinates are clamped into the source, so even the predicated-off positions load in bounds.
-            constexpr int RU = 2, CU = 2;
-            for (int r0 = threadIdx.y; r0 < fh; r0 += kStagedBY * RU) {
-                typename Back::RawRow rows[RU];
+    // Horizontal part, per lane, shared by the YI rows.  float(x1) and float(x1 + 1) are taken as floor(sx) and
+    // floor(sx) + 1, the same numbers (exact integers below 2^24).
+    int x1[XI], x2[XI];
+    f32 ax[XI], bx[XI];
+    bool xin[XI];
 #pragma unroll
-                for (int i = 0; i < RU; ++i) {
-                    const int r = r0 + kStagedBY * i;
-                    rows[i] = Back::raw_row(fy0 + r < sh - 1 ? fy0 + r : sh - 1, z, q.back);
-                }
-                for (int c0 = threadIdx.x; c0 < fw; c0 += kStagedBX * CU) {
-                    Raw v[RU][CU];
-#pragma unroll
-                    for (int j = 0; j < CU; ++j) {
-                        const int c = c0 + kStagedBX * j;
-                        const int sx = fx0 + c < sw - 1 ? fx0 + c : sw - 1;
-#pragma unroll
-                        for (int i = 0; i < RU; ++i) v[i][j] = Back::raw_at(rows[i], sx, q.back);
-                    }
-#pragma unroll
-                    for (int i = 0; i < RU; ++i) {
-                        const int r = r0 + kStagedBY * i;
-#pragma unroll
-                        for (int j = 0; j < CU; ++j) {
-                            const int c = c0 + kStagedBX * j;
-                            if (r < fh && c < fw) lds[r * fw + c] = lds_pack<Raw>(v[i][j]);
-                        }
-                    }
-                }
-            }
-        }
+    for (int i = 0; i < XI; ++i) {
+        const int x = tx0 + int(threadIdx.x) + kGatherBX * i;
+        xin[i] = true;
+        if constexpr (RZ::kAR != IGNORE_AR) xin[i] = x >= q.x1 && x <= q.x2;
+        const f32 sx = f32(x - ox) * q.fx;
+        const f32 f1 = __builtin_floorf(sx);
+        ax[i] = (f1 + 1.0f) - sx;
+        bx[i] = sx - f1;
+        const int xi = int(f1);
+        x1[i] = xi < 0 ? 0 : (xi < sw - 1 ? xi : sw - 1);       // no-op wherever the reference is in bounds
+        x2[i] = x1[i] + 1 < sw - 1 ? x1[i] + 1 : sw - 1;
     }
-    __syncthreads();
 
-    // Interpolation.  Everything that depends on the row only (source y, vertical weights, LDS row, output row
-    // address) is formed once per row; per pixel remain the horizontal coordinate, four weights, four LDS reads,
-    // the blend, the chain's compute operations and the store.  float(x1) and float(x1 + 1) are taken as floor(sx)
-    // and floor(sx) + 1, which are the same numbers (exact integers below 2^24).
+    // Rows, software pipelined: the taps of row y+1 are requested before row y is blended, so once the first row
+    // has arrived a wave always has data to work on while its next loads are in flight.  Two tap sets alternate
+    // (the loop handles two rows per trip), so no registers are copied.
+    struct RowTaps {
+        typename Back::TapBits a[XI], b[XI], c[XI], d[XI];
+        f32 ay, by;
+    };
+    const int yend = y0 + YI < ah ? y0 + YI : ah;
+    auto rows = [&](auto over) {
+        constexpr bool OVER = decltype(over)::value;
+        auto request = [&](int yrow, RowTaps& t) {
+            const int y = yrow < ah ? yrow : ah - 1;     // rows past the end re-read the last one; never stored
+            const f32 sy = f32(y - oy) * q.fy;
+            const f32 f1 = __builtin_floorf(sy);
+            t.ay = (f1 + 1.0f) - sy;
+            t.by = sy - f1;
+            const int yi = __builtin_amdgcn_readfirstlane(int(f1));
+            const int ya = yi < 0 ? 0 : (yi < sh - 1 ? yi : sh - 1);
+            const int yb = ya + 1 < sh - 1 ? ya + 1 : sh - 1;
+            const typename Back::TapRow ra = Back::tap_row(0, ya, z, q.back);
+            const typename Back::TapRow rb = Back::tap_row(0, yb, z, q.back);
 #pragma unroll
-    for (int j = 0; j < YI; ++j) {
-        const int y = ty0 + int(threadIdx.y) + kStagedBY * j;
-        if (y >= ah) continue;
-        const typename W::RowRef orow = W::row(y, z, p.write);
-        bool yin = true;
-        if constexpr (RZ::kAR != IGNORE_AR) yin = y >= q.y1 && y <= q.y2;
-        const f32 sy = f32(y - oy) * q.fy;
-        const f32 fy1 = __builtin_floorf(sy);
-        const f32 ay = (fy1 + 1.0f) - sy, by = sy - fy1;
-        const int y1 = int(fy1);
-        const Slot* lrow0 = lds + (y1 - fy0) * fw - fx0;
-        const Slot* lrow1 = lrow0 + fw;
-#pragma unroll
-        for (int i = 0; i < XI; ++i) {
-            const int x = tx0 + int(threadIdx.x) + kStagedBX * i;
-            if (x >= aw) continue;
-            typename RZ::Out v;
-            bool in = yin;
-            if constexpr (RZ::kAR != IGNORE_AR) in = in && x >= q.x1 && x <= q.x2;
-            if (!in) {
-                v = q.bg;
-            } else if (!staged) {
-                v = RZ::exec(x, y, z, q);
-            } else {
-                const f32 sx = f32(x - ox) * q.fx;
-                const f32 fx1 = __builtin_floorf(sx);
-                const f32 ax = (fx1 + 1.0f) - sx, bx = sx - fx1;
-                const int x1 = int(fx1);
-                typename RZ::Taps tp;
-                tp.w00 = ax * ay; tp.w10 = bx * ay; tp.w01 = ax * by; tp.w11 = bx * by;
-                // Unclamped +1 taps: the staged rectangle carries one replicated column/row past the edge.
-                const auto a = Back::finish(lds_unpack<Raw>(lrow0[x1]), q.back);
-                const auto b = Back::finish(lds_unpack<Raw>(lrow0[x1 + 1]), q.back);
-                const auto c = Back::finish(lds_unpack<Raw>(lrow1[x1]), q.back);
-                const auto d = Back::finish(lds_unpack<Raw>(lrow1[x1 + 1]), q.back);
-                v = RZ::blend(a, b, c, d, tp);
+            for (int i = 0; i < XI; ++i) {
+                t.a[i] = Back::template tap_load<OVER>(ra, x1[i], q.back);
+                t.b[i] = Back::template tap_load<OVER>(ra, x2[i], q.back);
+                t.c[i] = Back::template tap_load<OVER>(rb, x1[i], q.back);
+                t.d[i] = Back::template tap_load<OVER>(rb, x2[i], q.back);
             }
-            W::put(orow, x, Chain::compute(v, p));
+        };
+        auto produce = [&](int y, const RowTaps& t) {
+            if (y >= yend) return;
+            bool yin = true;
+            if constexpr (RZ::kAR != IGNORE_AR) yin = y >= q.y1 && y <= q.y2;
+            const typename W::RowRef orow = W::row(y, z, p.write);
+#pragma unroll
+            for (int i = 0; i < XI; ++i) {
+                const int x = tx0 + int(threadIdx.x) + kGatherBX * i;
+                typename RZ::Taps tp;
+                tp.w00 = ax[i] * t.ay; tp.w10 = bx[i] * t.ay; tp.w01 = ax[i] * t.by; tp.w11 = bx[i] * t.by;
+                typename RZ::Out v = RZ::blend(Back::finish(Back::tap_value(t.a[i]), q.back), Back::finish(Back::tap_value(t.b[i]), q.back),
+                                               Back::finish(Back::tap_value(t.c[i]), q.back), Back::finish(Back::tap_value(t.d[i]), q.back), tp);
+                if constexpr (RZ::kAR != IGNORE_AR) { if (!(yin && xin[i])) v = q.bg; }
+                const typename Chain::Value r = Chain::compute_checked(v, p);
+                if (x < aw) W::put(orow, x, r);
+            }
+        };
+        RowTaps t0, t1;
+        request(y0, t0);
+#pragma unroll 1
+        for (int y = y0; y < yend; y += 2) {
+            request(y + 1, t1);
+            produce(y, t0);
+            request(y + 2, t0);
+            produce(y + 1, t1);
         }
+    };
+    if constexpr (Back::kTapOverread) {
+        // Whole-dword reads of 3- and 6-byte elements touch up to 3 bytes past the element.  Inside the image that
+        // is the next element or row; only in the image's last row it could leave the allocation, so waves whose
+        // taps reach that row read channel by channel instead.
+        const int ylast = y0 + YI + 1 < ah - 1 ? y0 + YI + 1 : ah - 1;    // last row the pipeline may request
+        const int yl = int(__builtin_floorf(f32(ylast - oy) * q.fy));
+        const int yb = yl + 1 < sh - 1 ? yl + 1 : sh - 1;
+        if (Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back))) rows(std::false_type{});
+        else rows(std::true_type{});
+    } else {
+        rows(std::false_type{});
     }
 }
 
 // ---- host-side launchers -------------------------------------------------------------------------------
 
 template <class Chain> struct RowsConfig {
-    // Four elements per thread wherever the chain reads rows; a bilinear read that cannot be staged keeps one
+    // Four elements per thread wherever the chain reads rows; a bilinear read without a tap cursor keeps one
     // element per thread (its taps are gathers, wider threads would only spread them further apart).
     static constexpr int V = ResizeRoot<typename Chain::Read>::value ? 1 : 4;
 #ifndef FKD_ROWS
@@ -302,48 +265,26 @@ hipError_t launch_rows(const typename Chain::Params& p, hipStream_t stream, Laun
     return hipGetLastError();
 }
 
-template <class RZParams> inline void staged_need(const RZParams& q, int tw, int th, unsigned& slots) {
-    // Upper bound of the staged rectangle of any tile of this plane (two extra columns/rows: the +1 tap and
-    // float rounding of the two floor() calls).
-    const long long fw = (long long)__builtin_ceilf(float(tw - 1) * q.fx) + 3;
-    const long long fh = (long long)__builtin_ceilf(float(th - 1) * q.fy) + 3;
-    const long long n = fw * fh;
-    if (n > (long long)slots) slots = n > 0x7fffffffLL ? 0x7fffffffu : unsigned(n);
-}
-
-constexpr unsigned kStagedLdsBudget = 64u * 1024u;
-
 template <class Chain>
-hipError_t launch_staged(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
-    using Root = ResizeRoot<typename Chain::Read>;
-    using Slot = LdsSlot<typename Root::Resize::BackOp::Raw>;
-    constexpr int XI = FKD_STAGED_XI, YI = FKD_STAGED_YI;
-    constexpr int TW = kStagedBX * XI, TH = kStagedBY * YI;
-    unsigned slots = 0;
-    if constexpr (Root::batched) {
-        for (unsigned z = 0; z < p.active_z && z < unsigned(Root::batched ? Chain::Read::kBatch : 1); ++z)
-            staged_need(p.read.plane[z], TW, TH, slots);
-    } else {
-        staged_need(p.read, TW, TH, slots);
-    }
-    const unsigned long long bytes = (unsigned long long)slots * sizeof(Slot);
-    if (bytes > kStagedLdsBudget) return launch_rows<Chain>(p, stream, info);   // very strong downscale
-    StagedGeom g;
+hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
+    constexpr int XI = FKD_GATHER_XI, YI = FKD_GATHER_YI;
+    constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
+    TileGeom g;
     g.tiles_x = (p.active_w + TW - 1) / TW;
     g.tiles_y = (p.active_h + TH - 1) / TH;
     g.n_tiles = g.tiles_x * g.tiles_y * p.active_z;
-    g.lds_slots = slots;
-    const unsigned chunk = (g.n_tiles + 7u) / 8u;
-    const dim3 grid(chunk * 8u, 1, 1), block(kStagedBX, kStagedBY, 1);
-    if (info) *info = LaunchInfo{"staged", {grid.x, 1, 1}, {block.x, block.y, 1}, unsigned(bytes)};
+    const unsigned chunk = (g.tiles_x * g.tiles_y + 7u) / 8u;
+    const dim3 grid(chunk * 8u, 1, p.active_z), block(kGatherBX, kGatherBY, 1);
+    if (info) *info = LaunchInfo{"gather", {grid.x, 1, grid.z}, {block.x, block.y, 1}, 0};
     if (g.n_tiles == 0) return hipSuccess;
-    hipLaunchKernelGGL((k_staged<Chain, XI, YI>), grid, block, unsigned(bytes), stream, p, g);
+    if (grid.z > 65535u) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_gather<Chain, XI, YI>), grid, block, 0, stream, p, g);
     return hipGetLastError();
 }
 
 template <class Chain>
 hipError_t launch_chain(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
-    if constexpr (is_staged_chain<Chain>()) return launch_staged<Chain>(p, stream, info);
+    if constexpr (is_gather_chain<Chain>()) return launch_gather<Chain>(p, stream, info);
     else return launch_rows<Chain>(p, stream, info);
 }
 

@@ -4,7 +4,7 @@
 namespace fkd {
 
 struct LaunchInfo {
-    const char* kernel;   // "rows" or "staged"
+    const char* kernel;   // "rows", "rows_unaligned" or "gather"
     unsigned grid[3], block[3];
     unsigned lds_bytes;
 };

@@ -119,7 +119,8 @@ template <class I, I... Is> struct IntSeq {};
 template <int N> using MakeSeq = __make_integer_seq<IntSeq, int, N>;
 
 template <int K, class T, int V> FKD_DEV base_t<T> run_elem(const Slot<T> (&in)[V]) {   // K-th base element of the run
-    return chan<K % cn_v<T>>(in[K / cn_v<T>].v);
+    if constexpr (K < V * cn_v<T>) return chan<K % cn_v<T>>(in[K / cn_v<T>].v);
+    else return base_t<T>(0);   // padding of a last, partly filled dword
 }
 template <int I, class T, int V> FKD_DEV u32 pack_word(const Slot<T> (&in)[V]) {        // I-th dword of the run
     using B = base_t<T>;
@@ -208,6 +209,92 @@ template <class T, int V, bool ALIGNED> FKD_DEV void store_run(T* p, const Slot<
     }
 }
 
+// One element at byte offset `off` of a (typically wave-uniform) base address: the form a gather wants, because
+// the base stays in scalar registers and the lane supplies a 32-bit offset.  The element arrives as raw dwords
+// (ElemBits) and is taken apart later, at its point of use (bits_value), so a consumer can keep many such loads in
+// flight.  The hardware takes global accesses at any byte alignment, so an element whose size is 1, 2 or a
+// multiple of 4 moves as one access.  Sizes 3 and 6 (uchar3, ushort3 ...) move as one or two whole dwords when
+// OVERREAD allows touching up to 3 bytes past the element (the caller guarantees those bytes are inside the
+// allocation); otherwise channel by channel.
+typedef u16 u16_a1 __attribute__((aligned(1)));
+typedef u32 u32_a1 __attribute__((aligned(1)));
+typedef u32x2_t u32x2_a1 __attribute__((aligned(1)));
+typedef u32x3_t u32x3_a1 __attribute__((aligned(1)));
+typedef u32x4_t u32x4_a1 __attribute__((aligned(1)));
+template <class T> constexpr int overread_bytes() {
+    constexpr int n = int(sizeof(T));
+    return (n == 1 || n == 2 || n % 4 == 0 || n > 16) ? 0 : (n + 3) / 4 * 4 - n;
+}
+template <class T> struct ElemBits {
+    static_assert(sizeof(T) == sizeof(base_t<T>) * cn_v<T>, "elements are packed channel arrays");
+    static constexpr int kWords = (int(sizeof(T)) + 3) / 4;
+    u32 w[kWords];
+};
+template <class T, bool OVERREAD> FKD_DEV ElemBits<T> load_bits_at(const char* base, u32 off) {
+    constexpr int n = int(sizeof(T));
+    constexpr int W = ElemBits<T>::kWords;
+    // Keeps the offset a 32-bit per-lane value next to the access, so base + offset selects the scalar-base
+    // addressing form instead of a hoisted 64-bit per-lane pointer.
+    asm volatile("" : "+v"(off));
+    const char* a = base + off;
+    ElemBits<T> e;
+    if constexpr (n == 1) {
+        e.w[0] = u32(*reinterpret_cast<const u8*>(a));
+    } else if constexpr (n == 2) {
+        e.w[0] = u32(*reinterpret_cast<const u16_a1*>(a));
+    } else if constexpr (n > 16 || (overread_bytes<T>() > 0 && !OVERREAD)) {
+        Slot<T> one[1];
+        one[0].v = load_elem(reinterpret_cast<const T*>(a));
+        pack_words<T, 1, W>(one, e.w);
+    } else if constexpr (W == 1) {
+        e.w[0] = *reinterpret_cast<const u32_a1*>(a);
+    } else if constexpr (W == 2) {
+        const u32x2_t v = *reinterpret_cast<const u32x2_a1*>(a); e.w[0] = v.x; e.w[1] = v.y;
+    } else if constexpr (W == 3) {
+        const u32x3_t v = *reinterpret_cast<const u32x3_a1*>(a); e.w[0] = v.x; e.w[1] = v.y; e.w[2] = v.z;
+    } else {
+        const u32x4_t v = *reinterpret_cast<const u32x4_a1*>(a); e.w[0] = v.x; e.w[1] = v.y; e.w[2] = v.z; e.w[3] = v.w;
+    }
+    return e;
+}
+template <class T> FKD_DEV T bits_value(const ElemBits<T>& e) {
+    constexpr int W = ElemBits<T>::kWords;
+    u32 w[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) w[i] = e.w[i];
+    if constexpr (sizeof(base_t<T>) < 4) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) asm("" : "+v"(w[i]));   // keep dwords whole: bytes leave through v_cvt_f32_ubyteN / v_bfe
+    }
+    return unpack_one<0, T>(w);
+}
+
+// Store counterpart of load_bits_at: element sizes 2 and multiples of 4 (up to 16) leave as one access.
+template <class T> FKD_DEV void store_elem_at(char* base, u32 off, const T& v) {
+    constexpr int n = int(sizeof(T));
+    constexpr bool packed = sizeof(T) == sizeof(base_t<T>) * cn_v<T>;
+    asm volatile("" : "+v"(off));   // as in load_bits_at: keep the scalar-base addressing form
+    char* a = base + off;
+    if constexpr (!packed || n > 16 || (n % 4 != 0 && n != 2) || cn_v<T> == 1) {
+        store_elem(reinterpret_cast<T*>(a), v);
+    } else {
+        Slot<T> one[1];
+        one[0].v = v;
+        constexpr int W = (n + 3) / 4;
+        u32 w[W];
+        if constexpr (n == 2) {
+            w[0] = to_bits(chan<0>(v)) | (to_bits(chan<1>(v)) << 8);
+            *reinterpret_cast<u16_a1*>(a) = u16(w[0]);
+        } else {
+            pack_words<T, 1, W>(one, w);
+            if constexpr (W == 1) { *reinterpret_cast<u32_a1*>(a) = w[0]; }
+            else if constexpr (W == 2) { u32x2_t q; q.x = w[0]; q.y = w[1]; *reinterpret_cast<u32x2_a1*>(a) = q; }
+            else if constexpr (W == 3) { u32x3_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; *reinterpret_cast<u32x3_a1*>(a) = q; }
+            else { u32x4_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3]; *reinterpret_cast<u32x4_a1*>(a) = q; }
+        }
+    }
+}
+
 FKD_HD bool dword_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 template <class T> FKD_DEV const T* row_ptr(const T* data, u32 pitch, int x, int y) {
@@ -238,8 +325,86 @@ template <class T> FKD_DEV T* row_ptr(T* data, u32 pitch, int x, int y) {
 FKD_BINARY_OP(Add, x + y)
 FKD_BINARY_OP(Sub, x - y)
 FKD_BINARY_OP(Mul, x * y)
-FKD_BINARY_OP(Div, x / y)
 #undef FKD_BINARY_OP
+
+// Div<I,P,O>: FK/algorithms/basic_ops/arithmetic.h:96-124, x / y per channel, correctly rounded.
+//
+// The divisor is a launch-time constant, the same for every element, so for all-fp32 divisions the host also
+// stores r = RN(1/y) and the device replaces the generic division (two scalings, a reciprocal estimate, its
+// refinement, fix-ups: ~10 instructions) by five:
+//     q0 = x*r;  e0 = fma(-y, q0, x);  q1 = fma(e0, r, q0);  e1 = fma(-y, q1, x);  q = fma(e1, r, q1)
+// q0 is within 1.5 ulp of x/y, so q1 is within 0.5 ulp + 2^-23 ulp (faithful), e1 is then exact and, r being the
+// correctly rounded reciprocal, the last step yields RN(x/y) (Markstein's theorem on the final division step).
+// That argument needs every intermediate free of underflow and overflow: the host enables the path only for
+// 2^-40 <= |y| <= 2^40, and the device takes it only for elements with 2^-60 <= |x| <= 2^60 in every channel;
+// everything else (zeros, denormals, infinities, NaNs, extreme magnitudes) goes through the generic division.
+template <class I, class P, class O> struct Div {
+    using In = I; using Out = O;
+    static constexpr bool kReciprocal = __is_same(base_t<I>, f32) && __is_same(base_t<P>, f32) && __is_same(base_t<O>, f32);
+    struct Params { P v; P rcp; i32 fast; };
+    FKD_NAME("Div<" + type_name<I>() + "," + type_name<P>() + "," + type_name<O>() + ">")
+
+#if !defined(FKD_DEVICE_CODE)
+    // RN(1/d) for a normal d: the double quotient rounded to float is off by at most one float; 1 - d*c is exact in
+    // double for the three candidates, so the smallest residual names the correctly rounded one.
+    static f32 exact_reciprocal(f32 d) {
+        const f32 c0 = f32(1.0 / double(d));
+        f32 best = c0;
+        double err = __builtin_fabs(1.0 - double(d) * double(c0));
+        for (const f32 c : {__builtin_nextafterf(c0, -__builtin_inff()), __builtin_nextafterf(c0, __builtin_inff())}) {
+            const double e = __builtin_fabs(1.0 - double(d) * double(c));
+            if (e < err) { err = e; best = c; }
+        }
+        return best;
+    }
+    static Params make(const P& v) {
+        Params p{};
+        p.v = v;
+        p.fast = 0;
+        if constexpr (kReciprocal) {
+            bool ok = true;
+            auto one = [&](f32 d) {
+                const f32 a = __builtin_fabsf(d);
+                if (!(a >= 0x1p-40f && a <= 0x1p40f)) { ok = false; return 0.0f; }
+                return exact_reciprocal(d);
+            };
+            p.rcp = map1<P>(v, one);
+            p.fast = ok ? 1 : 0;
+        }
+        return p;
+    }
+#endif
+
+    FKD_DEV static O exec(const I& a, const Params& p) {
+        return map2<O>(a, p.v, [](auto x, auto y) { return static_cast<base_t<O>>(x / y); });
+    }
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static f32 quick1(f32 x, f32 y, f32 r) {
+        const f32 q0 = x * r;
+        const f32 e0 = __builtin_fmaf(-y, q0, x);
+        const f32 q1 = __builtin_fmaf(e0, r, q0);
+        const f32 e1 = __builtin_fmaf(-y, q1, x);
+        return __builtin_fmaf(e1, r, q1);
+    }
+    // Straight-line variant: always returns the five-instruction result and clears `ok` when that result may not be
+    // the correctly rounded quotient for this element; the caller then recomputes the element with exec().
+    static constexpr bool kQuick = kReciprocal;
+    FKD_DEV static O exec_quick(const I& a, const Params& p, bool& ok) {
+        // sum of magnitudes <= 2^60 bounds every channel from above and is false for NaN and infinity
+        f32 sum = __builtin_fabsf(chan<0>(a)), least = sum;
+        if constexpr (cn_v<I> > 1) { sum += __builtin_fabsf(chan<1>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<1>(a))); }
+        if constexpr (cn_v<I> > 2) { sum += __builtin_fabsf(chan<2>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<2>(a))); }
+        if constexpr (cn_v<I> > 3) { sum += __builtin_fabsf(chan<3>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<3>(a))); }
+        ok = ok && p.fast != 0 && sum <= 0x1p60f && least >= 0x1p-60f;
+        O o;
+        chan<0>(o) = quick1(chan<0>(a), chan_or_scalar<0>(p.v), chan_or_scalar<0>(p.rcp));
+        if constexpr (cn_v<O> > 1) chan<1>(o) = quick1(chan<1>(a), chan_or_scalar<1>(p.v), chan_or_scalar<1>(p.rcp));
+        if constexpr (cn_v<O> > 2) chan<2>(o) = quick1(chan<2>(a), chan_or_scalar<2>(p.v), chan_or_scalar<2>(p.rcp));
+        if constexpr (cn_v<O> > 3) chan<3>(o) = quick1(chan<3>(a), chan_or_scalar<3>(p.v), chan_or_scalar<3>(p.rcp));
+        return o;
+    }
+#endif
+};
 
 // Cast<I,O>: per-channel static_cast.  FK/algorithms/basic_ops/cast.h:22-33.
 template <class I, class O> struct Cast {
@@ -360,6 +525,22 @@ FKD_DEV auto fold(const V& v, const Tup<typename Op::Params, typename Rest::Para
     if constexpr (sizeof...(Rest) == 0) return Op::exec(v, p.head);
     else return fold<Rest...>(Op::exec(v, p.head), p.tail);
 }
+
+// The same fold through each operation's straight-line variant where it has one (see Div).  `ok` comes back false
+// when some operation could not vouch for its quick result; the value must then be recomputed with fold().
+template <class Op> constexpr bool has_quick() {
+    if constexpr (requires { Op::kQuick; }) return Op::kQuick; else return false;
+}
+template <class... Ops> constexpr bool any_quick() { return (false || ... || has_quick<Ops>()); }
+template <class V> FKD_DEV V fold_quick(const V& v, const Tup<>&, bool&) { return v; }
+template <class Op, class... Rest, class V>
+FKD_DEV auto fold_quick(const V& v, const Tup<typename Op::Params, typename Rest::Params...>& p, bool& ok) {
+    auto step = [&] {
+        if constexpr (has_quick<Op>()) return Op::exec_quick(v, p.head, ok); else return Op::exec(v, p.head);
+    };
+    if constexpr (sizeof...(Rest) == 0) return step();
+    else return fold_quick<Rest...>(step(), p.tail, ok);
+}
 #endif
 
 // A run of compute operations packaged as one (host side: FusedOperation of compute IOps).
@@ -381,7 +562,7 @@ template <class... Ops> struct FusedCompute {
 template <class T> struct Read2D {
     using Out = T;
     using Params = RawPtr2D<const T>;
-    static constexpr bool kStageable = true;
+    static constexpr bool kTapCursor = true;
     FKD_NAME("Read2D<" + type_name<T>() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -397,14 +578,22 @@ template <class T> struct Read2D {
     FKD_HD static bool rows_aligned(const Params& p, int xoff) {
         return detail::dword_aligned(reinterpret_cast<const char*>(p.data) + ptrdiff_t(xoff) * ptrdiff_t(sizeof(T))) && p.pitch % 4 == 0;
     }
-    // Staging hooks: the element as it lies in memory, and what the consumer sees of it.
     using Raw = T;
-    FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
     FKD_DEV static T finish(const Raw& r, const Params&) { return r; }
-    // Row cursor for staging loops: the row address is formed once, each element costs one add.
-    struct RawRow { const T* p; };
-    FKD_DEV static RawRow raw_row(int y, int, const Params& p) { return RawRow{detail::row_ptr(p.data, p.pitch, 0, y)}; }
-    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params&) { return detail::load_elem(r.p + x); }
+    // Tap cursor for gathers: the address of element (x0, y), wave uniform when y is; tap_load adds a 32-bit byte
+    // offset and returns the element's raw bits, tap_value takes them apart where they are used.  `last` marks the last row of the image, the only row in which reading a few bytes past an element
+    // could leave the allocation; kTapOverread says whether tap_load<true> reads past elements at all.
+    static constexpr bool kTapOverread = detail::overread_bytes<T>() > 0;
+    struct TapRow { const char* p; bool last; };
+    FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) {
+        return TapRow{reinterpret_cast<const char*>(detail::row_ptr(p.data, p.pitch, x0, y)), y >= int(p.height) - 1};
+    }
+    FKD_DEV static bool tap_last(const TapRow& r) { return r.last; }
+    using TapBits = detail::ElemBits<T>;
+    template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params&) {
+        return detail::load_bits_at<T, OVER>(r.p, u32(x) * u32(sizeof(T)));
+    }
+    FKD_DEV static Raw tap_value(const TapBits& b) { return detail::bits_value<T>(b); }
 #endif
 };
 
@@ -413,7 +602,7 @@ template <class T> struct Read2D {
 template <class T> struct Read3D {
     using Out = T;
     using Params = RawPtr3D<const T>;
-    static constexpr bool kStageable = false;
+    static constexpr bool kTapCursor = false;
     FKD_NAME("Read3D<" + type_name<T>() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -439,7 +628,7 @@ template <class T> struct Read3D {
 struct ReadNV12 {
     using Out = Vec<u8, 3>;
     using Params = RawNV12;
-    static constexpr bool kStageable = true;
+    static constexpr bool kTapCursor = true;
     FKD_NAME("ReadNV12")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -457,19 +646,29 @@ struct ReadNV12 {
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
     using Raw = Out;
-    FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return exec(x, y, z, p); }
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
     FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // gathers element-wise either way
-    struct RawRow { const u8* luma; const u8* chroma; };
-    FKD_DEV static RawRow raw_row(int y, int, const Params& p) {
-        return RawRow{p.data + size_t(y) * p.pitch, p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch};
+    static constexpr bool kTapOverread = false;
+    struct TapRow { const char* luma; const char* chroma; int x0; };
+    FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) {
+        const char* d = reinterpret_cast<const char*>(p.data);
+        return TapRow{d + size_t(y) * p.pitch, d + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch, x0};
     }
-    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params&) {
+    FKD_DEV static bool tap_last(const TapRow&) { return false; }
+    struct TapBits { u32 y, uv; };
+    template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params&) {
+        u32 xs = u32(r.x0 + x), xc = xs & ~1u;
+        asm volatile("" : "+v"(xs), "+v"(xc));      // 32-bit lane offsets against scalar row addresses
+        TapBits b;
+        b.y = u32(*reinterpret_cast<const u8*>(r.luma + xs));
+        b.uv = u32(*reinterpret_cast<const detail::u16_a1*>(r.chroma + xc));   // (U,V) pair in one access
+        return b;
+    }
+    FKD_DEV static Raw tap_value(const TapBits& b) {
         Out o;
-        o.x = r.luma[x];
-        const u8* c = r.chroma + 2 * (x >> 1);
-        o.y = c[0];
-        o.z = c[1];
+        o.x = u8(b.y);
+        o.y = u8(b.uv & 0xffu);
+        o.z = u8(b.uv >> 8);
         return o;
     }
 #endif
@@ -480,7 +679,7 @@ struct ReadNV12 {
 template <class Back> struct Crop {
     using Out = typename Back::Out;
     struct Params { i32 x, y, w, h; typename Back::Params back; };
-    static constexpr bool kStageable = Back::kStageable;
+    static constexpr bool kTapCursor = Back::kTapCursor;
     FKD_NAME("Crop<" + Back::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return p.w; }
@@ -491,11 +690,16 @@ template <class Back> struct Crop {
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff + p.x); }
     using Raw = typename Back::Raw;
-    FKD_DEV static Raw exec_raw(int x, int y, int, const Params& p) { return Back::exec_raw(x + p.x, y + p.y, 0, p.back); }
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return Back::finish(r, p.back); }
-    using RawRow = typename Back::RawRow;
-    FKD_DEV static RawRow raw_row(int y, int, const Params& p) { return Back::raw_row(y + p.y, 0, p.back); }
-    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params& p) { return Back::raw_at(r, x + p.x, p.back); }
+    static constexpr bool kTapOverread = Back::kTapOverread;
+    using TapRow = typename Back::TapRow;
+    FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) { return Back::tap_row(x0 + p.x, y + p.y, 0, p.back); }
+    FKD_DEV static bool tap_last(const TapRow& r) { return Back::tap_last(r); }
+    using TapBits = typename Back::TapBits;
+    template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params& p) {
+        return Back::template tap_load<OVER>(r, x, p.back);
+    }
+    FKD_DEV static Raw tap_value(const TapBits& b) { return Back::tap_value(b); }
 #endif
 };
 
@@ -504,7 +708,7 @@ template <class Back> struct Crop {
 template <class Back, class... Ops> struct FusedRead {
     using Out = typename FoldOut<typename Back::Out, Ops...>::type;
     struct Params { typename Back::Params back; Tup<typename Ops::Params...> ops; };
-    static constexpr bool kStageable = Back::kStageable;
+    static constexpr bool kTapCursor = Back::kTapCursor;
     FKD_NAME("FusedRead<" + Back::name() + OpList<Ops...>::names() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
@@ -520,11 +724,16 @@ template <class Back, class... Ops> struct FusedRead {
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
     using Raw = typename Back::Raw;
-    FKD_DEV static Raw exec_raw(int x, int y, int z, const Params& p) { return Back::exec_raw(x, y, z, p.back); }
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return fold<Ops...>(Back::finish(r, p.back), p.ops); }
-    using RawRow = typename Back::RawRow;
-    FKD_DEV static RawRow raw_row(int y, int z, const Params& p) { return Back::raw_row(y, z, p.back); }
-    FKD_DEV static Raw raw_at(const RawRow& r, int x, const Params& p) { return Back::raw_at(r, x, p.back); }
+    static constexpr bool kTapOverread = Back::kTapOverread;
+    using TapRow = typename Back::TapRow;
+    FKD_DEV static TapRow tap_row(int x0, int y, int z, const Params& p) { return Back::tap_row(x0, y, z, p.back); }
+    FKD_DEV static bool tap_last(const TapRow& r) { return Back::tap_last(r); }
+    using TapBits = typename Back::TapBits;
+    template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params& p) {
+        return Back::template tap_load<OVER>(r, x, p.back);
+    }
+    FKD_DEV static Raw tap_value(const TapBits& b) { return Back::tap_value(b); }
 #endif
 };
 
@@ -543,7 +752,7 @@ template <int AR, class Back> struct ResizeLinear {
         Out bg;
         typename Back::Params back;
     };
-    static constexpr bool kStageable = false;
+    static constexpr bool kTapCursor = false;
     static constexpr int kAR = AR;
     using BackOp = Back;
     FKD_NAME("ResizeLinear<" + istr(AR) + "," + Back::name() + ">")
@@ -606,7 +815,7 @@ template <int N, class PlaneOp> struct BatchRead {
     using Plane = PlaneOp;
     static constexpr int kBatch = N;
     struct Params { typename PlaneOp::Params plane[N]; };
-    static constexpr bool kStageable = false;
+    static constexpr bool kTapCursor = false;
     FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
@@ -626,7 +835,7 @@ template <int N, class PlaneOp> struct BatchReadDefault {
     using Plane = PlaneOp;
     static constexpr int kBatch = N;
     struct Params { typename PlaneOp::Params plane[N]; i32 used; Out def; };
-    static constexpr bool kStageable = false;
+    static constexpr bool kTapCursor = false;
     FKD_NAME("BatchReadDefault<" + istr(N) + "," + PlaneOp::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
@@ -652,7 +861,7 @@ template <int N, class PlaneOp> struct BatchReadDefault {
 template <class T> struct ReadSet {
     using Out = T;
     struct Params { T value; u32 width, height, planes; };
-    static constexpr bool kStageable = false;
+    static constexpr bool kTapCursor = false;
     FKD_NAME("ReadSet<" + type_name<T>() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -686,7 +895,10 @@ template <class T> struct Write2D {
     // Row cursor: one address computation per row, one add per element.
     struct RowRef { T* p; };
     FKD_DEV static RowRef row(int y, int, const Params& p) { return RowRef{detail::row_ptr(p.data, p.pitch, 0, y)}; }
-    FKD_DEV static void put(const RowRef& r, int x, const T& v) { detail::store_elem(r.p + x, v); }
+    // wave-uniform row address + 32-bit byte offset of the lane: the address form that needs no per-lane 64-bit add
+    FKD_DEV static void put(const RowRef& r, int x, const T& v) {
+        detail::store_elem_at<T>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
+    }
 #endif
 };
 
@@ -711,7 +923,9 @@ template <class T> struct TensorWrite {
     }
     struct RowRef { T* p; };
     FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{detail::row_ptr(plane(p, z), p.pitch, 0, y)}; }
-    FKD_DEV static void put(const RowRef& r, int x, const T& v) { detail::store_elem(r.p + x, v); }
+    FKD_DEV static void put(const RowRef& r, int x, const T& v) {
+        detail::store_elem_at<T>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
+    }
 #endif
 };
 
@@ -760,14 +974,15 @@ template <class T> struct TensorSplit {
         return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 &&
                (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
     }
-    struct RowRef { B* p; u32 px; };
-    FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), p.width * p.height}; }
+    struct RowRef { B* p; size_t px; };
+    FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), size_t(p.width) * p.height}; }
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
-        B* w = r.p + x;
-        w[0] = chan<0>(v);
-        w[r.px] = chan<1>(v);
-        if constexpr (cn_v<T> > 2) w[2u * size_t(r.px)] = chan<2>(v);
-        if constexpr (cn_v<T> > 3) w[3u * size_t(r.px)] = chan<3>(v);
+        u32 off = u32(x) * u32(sizeof(B));   // one lane offset, four wave-uniform plane row addresses
+        asm volatile("" : "+v"(off));
+        *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p) + off) = chan<0>(v);
+        *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p + r.px) + off) = chan<1>(v);
+        if constexpr (cn_v<T> > 2) *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p + 2 * r.px) + off) = chan<2>(v);
+        if constexpr (cn_v<T> > 3) *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p + 3 * r.px) + off) = chan<3>(v);
     }
 #endif
 };
@@ -811,6 +1026,19 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     static_assert(__is_same(Value, typename W::In), "the write operation does not take the type the chain produces");
     FKD_DEV static Value compute(const typename R::Out& v, const Params& p) {
         if constexpr (sizeof...(Ops) == 0) return v; else return fold<Ops...>(v, p.ops);
+    }
+    // compute() through the operations' straight-line variants, falling back to compute() for the (rare) elements
+    // they cannot vouch for.  Same result as compute(), fewer instructions on the common path.
+    static constexpr bool kQuick = any_quick<Ops...>();
+    FKD_DEV static Value compute_checked(const typename R::Out& v, const Params& p) {
+        if constexpr (!kQuick) {
+            return compute(v, p);
+        } else {
+            bool ok = true;
+            Value r = fold_quick<Ops...>(v, p.ops, ok);
+            if (__builtin_expect(!ok, 0)) r = compute(v, p);
+            return r;
+        }
     }
 #endif
 };

@@ -91,7 +91,7 @@ int fklhip_launch_handle(const void *handle, const void *blob, size_t blob_bytes
 int fklhip_launch(const char *signature, const void *blob, size_t blob_bytes, void *stream);
 
 /* Introspection for tests and benchmarks: what the last fklhip_launch* on this thread launched.
- * kernel receives "rows" or "staged"; grid/block receive 3 values each. */
+ * kernel receives "rows", "rows_unaligned" or "gather"; grid/block receive 3 values each. */
 int fklhip_last_launch(const char **kernel, unsigned grid[3], unsigned block[3], unsigned *lds_bytes);
 
 /* Number of chain signatures compiled into the library and the i-th of them with its parameter block size. */

@@ -27,8 +27,24 @@ namespace fk {
 FK_AMD_ARITH(Add)
 FK_AMD_ARITH(Sub)
 FK_AMD_ARITH(Mul)
-FK_AMD_ARITH(Div)
 #undef FK_AMD_ARITH
+
+// Div: the device parameter block also carries the correctly rounded reciprocal of the divisor (see fkd::Div).
+template <typename I1, typename I2 = I1, typename O = I1, typename IT = BinaryType> struct Div;
+template <typename I, typename P, typename O>
+struct Div<I, P, O, BinaryType> : BinaryOperation<I, P, O, Div<I, P, O, BinaryType>> {
+    using Parent = BinaryOperation<I, P, O, Div<I, P, O, BinaryType>>;
+    FK_STATIC_STRUCT(Div, Div)
+};
+namespace amd {
+template <typename I, typename P, typename O> struct Lower<Div<I, P, O, BinaryType>> {
+    static constexpr bool available = true;
+    using type = fkd::Div<dev_t<I>, dev_t<P>, dev_t<O>>;
+    static typename type::Params params(const OperationData<Div<I, P, O, BinaryType>>& d) {
+        return type::make(to_dev(d.params));
+    }
+};
+}
 
 } // namespace fk
 #endif

@@ -106,7 +106,7 @@ def run_c4(c, device):
 def test_config1_full_size(device):
     c = wl.config1()
     got = run_c1(c, c["rects"], device)
-    assert last_launch()["kernel"] == "staged"
+    assert last_launch()["kernel"] == "gather"
     assert check_u8(got, GOLD["c1_full"], "config 1 vs reference golden"), "config 1 is expected to be bit-exact"
     assert sha(got) == DIG["c1_full"]
 
@@ -143,7 +143,7 @@ def test_config2_reduced_odd_width(device, n):
 def test_config3_full_size(device):
     c = wl.config3()
     got = run_c3(c, device)
-    assert last_launch()["kernel"] == "staged"
+    assert last_launch()["kernel"] == "gather"
     want = ol.oracle_crop_resize_norm_split(c["src"], c["rects"], c["dst"], c["sub"], c["div"])
     exact = check_float(got, want, "config 3 vs oracle")
     assert exact and sha(got) == DIG["c3_full"], "config 3 is expected to be bit-identical to the reference CPU backend"
@@ -192,7 +192,7 @@ def test_config4_full_size(device):
 def test_config5_full_size(device):
     c = wl.config5()
     got = run_c5(c, device)
-    assert last_launch()["kernel"] == "staged"
+    assert last_launch()["kernel"] == "gather"
     want = ol.oracle_nv12_rgb_resize_split(c["nv12"], c["width"], c["height"], c["dst"], c["scale"])
     assert check_float(got, want, "config 5 vs oracle") and sha(got) == DIG["c5_full"]
     # exact 2x: every output equals the colour-converted even source pixel (times 1/255)
