@@ -98,10 +98,13 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
 #define FKD_GATHER_XI 2
 #endif
 #ifndef FKD_GATHER_YI
-#define FKD_GATHER_YI 4
+#define FKD_GATHER_YI 2
+#endif
+#ifndef FKD_GATHER_BY
+#define FKD_GATHER_BY 4
 #endif
 constexpr int kGatherBX = 64;
-constexpr int kGatherBY = 4;
+constexpr int kGatherBY = FKD_GATHER_BY;
 
 struct TileGeom {
     u32 tiles_x, tiles_y, n_tiles;
@@ -129,18 +132,25 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     // consecutive workgroup ids round-robin to the 8 XCDs (the grid's x extent is a multiple of 8); XCD k gets the
     // k-th contiguous eighth of the plane's tiles so neighbouring tiles (which share source rows) share an L2.
     const int z = int(blockIdx.z);
-    const u32 per_plane = g.tiles_x * g.tiles_y;
+    // Everything the wave needs from the kernel-argument segment, fetched in one go.
+    const typename RZ::Params* rp;
+    if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
+    const TileGeom gg = detail::scalar_copy(g);
+    const typename RZ::Params q = detail::scalar_copy(*rp);
+    const typename Chain::OpParams& ops = p.ops;        // needed only after the taps are on their way
+    using WP = typename W::Plane;
+    const typename WP::Params& wpar = W::plane_params(p.write, z);
+    u32 dims[2] = {p.active_w, p.active_h};
+    asm volatile("" : "+s"(dims[0]), "+s"(dims[1]));
+    const int aw = int(dims[0]), ah = int(dims[1]);
+
+    const u32 per_plane = gg.tiles_x * gg.tiles_y;
     const u32 chunk = (per_plane + 7u) / 8u;
     const u32 tin = (blockIdx.x % 8u) * chunk + blockIdx.x / 8u;
     if (tin >= per_plane) return;
-    const int tx0 = int(tin % g.tiles_x) * TW;
+    const int tx0 = int(tin % gg.tiles_x) * TW;
     const int wy = __builtin_amdgcn_readfirstlane(int(threadIdx.y));
-    const int y0 = int(tin / g.tiles_x) * TH + wy * YI;
-
-    const typename RZ::Params* rp;
-    if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
-    const typename RZ::Params& q = *rp;
-    const int aw = int(p.active_w), ah = int(p.active_h);
+    const int y0 = int(tin / gg.tiles_x) * TH + wy * YI;
     if (y0 >= ah) return;
     int ox = 0, oy = 0;
     if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; }
@@ -151,9 +161,11 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     int x1[XI], x2[XI];
     f32 ax[XI], bx[XI];
     bool xin[XI];
+    bool lane_clamped = false;
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
-        const int x = tx0 + int(threadIdx.x) + kGatherBX * i;
+        int x = tx0 + int(threadIdx.x) + kGatherBX * i;
+        x = x < aw ? x : aw - 1;                                   // idle lanes shadow the last column
         xin[i] = true;
         if constexpr (RZ::kAR != IGNORE_AR) xin[i] = x >= q.x1 && x <= q.x2;
         const f32 sx = f32(x - ox) * q.fx;
@@ -163,20 +175,31 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
         const int xi = int(f1);
         x1[i] = xi < 0 ? 0 : (xi < sw - 1 ? xi : sw - 1);       // no-op wherever the reference is in bounds
         x2[i] = x1[i] + 1 < sw - 1 ? x1[i] + 1 : sw - 1;
+        lane_clamped = lane_clamped || x1[i] + 1 > sw - 1;
     }
+    const bool any_clamped = __builtin_amdgcn_ballot_w64(lane_clamped) != 0;
 
     // Rows, software pipelined: the taps of row y+1 are requested before row y is blended, so once the first row
     // has arrived a wave always has data to work on while its next loads are in flight.  Two tap sets alternate
     // (the loop handles two rows per trip), so no registers are copied.
-    struct RowTaps {
-        typename Back::TapBits a[XI], b[XI], c[XI], d[XI];
-        f32 ay, by;
-    };
+    // Three ways to fetch the taps of a row, chosen per wave:
+    //   kPairs    the two horizontally adjacent taps of a pixel come in one access (possible when no lane of the
+    //             wave has its right tap clamped to the last column), halving the number of gather instructions;
+    //   kSingles  one access per tap, whole dwords;
+    //   kSafe     one access per tap, never touching a byte outside the elements (channel by channel for 3- and
+    //             6-byte elements): for waves whose taps reach the last row of the image.
+    constexpr int kSafe = 0, kSingles = 1, kPairs = 2;
     const int yend = y0 + YI < ah ? y0 + YI : ah;
-    auto rows = [&](auto over) {
-        constexpr bool OVER = decltype(over)::value;
+    auto rows = [&](auto mode_tag) {
+        constexpr int MODE = decltype(mode_tag)::value;
+        struct RowTaps {
+            typename Back::TapBits a[MODE == kPairs ? 1 : XI], b[MODE == kPairs ? 1 : XI], c[MODE == kPairs ? 1 : XI], d[MODE == kPairs ? 1 : XI];
+            typename Back::PairBits ab[MODE == kPairs ? XI : 1], cd[MODE == kPairs ? XI : 1];
+            typename Back::TapRow ra, rb;
+            f32 ay, by;
+        };
         auto request = [&](int yrow, RowTaps& t) {
-            const int y = yrow < ah ? yrow : ah - 1;     // rows past the end re-read the last one; never stored
+            const int y = yrow;
             const f32 sy = f32(y - oy) * q.fy;
             const f32 f1 = __builtin_floorf(sy);
             t.ay = (f1 + 1.0f) - sy;
@@ -184,54 +207,72 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
             const int yi = __builtin_amdgcn_readfirstlane(int(f1));
             const int ya = yi < 0 ? 0 : (yi < sh - 1 ? yi : sh - 1);
             const int yb = ya + 1 < sh - 1 ? ya + 1 : sh - 1;
-            const typename Back::TapRow ra = Back::tap_row(0, ya, z, q.back);
-            const typename Back::TapRow rb = Back::tap_row(0, yb, z, q.back);
+            t.ra = Back::tap_row(0, ya, z, q.back);
+            t.rb = Back::tap_row(0, yb, z, q.back);
 #pragma unroll
             for (int i = 0; i < XI; ++i) {
-                t.a[i] = Back::template tap_load<OVER>(ra, x1[i], q.back);
-                t.b[i] = Back::template tap_load<OVER>(ra, x2[i], q.back);
-                t.c[i] = Back::template tap_load<OVER>(rb, x1[i], q.back);
-                t.d[i] = Back::template tap_load<OVER>(rb, x2[i], q.back);
+                if constexpr (MODE == kPairs) {
+                    t.ab[i] = Back::pair_load(t.ra, x1[i], q.back);
+                    t.cd[i] = Back::pair_load(t.rb, x1[i], q.back);
+                } else {
+                    t.a[i] = Back::template tap_load<MODE == kSingles>(t.ra, x1[i], q.back);
+                    t.b[i] = Back::template tap_load<MODE == kSingles>(t.ra, x2[i], q.back);
+                    t.c[i] = Back::template tap_load<MODE == kSingles>(t.rb, x1[i], q.back);
+                    t.d[i] = Back::template tap_load<MODE == kSingles>(t.rb, x2[i], q.back);
+                }
             }
         };
         auto produce = [&](int y, const RowTaps& t) {
             if (y >= yend) return;
             bool yin = true;
             if constexpr (RZ::kAR != IGNORE_AR) yin = y >= q.y1 && y <= q.y2;
-            const typename W::RowRef orow = W::row(y, z, p.write);
+            const typename WP::RowRef orow = WP::row(y, z, wpar);
 #pragma unroll
             for (int i = 0; i < XI; ++i) {
                 const int x = tx0 + int(threadIdx.x) + kGatherBX * i;
                 typename RZ::Taps tp;
                 tp.w00 = ax[i] * t.ay; tp.w10 = bx[i] * t.ay; tp.w01 = ax[i] * t.by; tp.w11 = bx[i] * t.by;
-                typename RZ::Out v = RZ::blend(Back::finish(Back::tap_value(t.a[i]), q.back), Back::finish(Back::tap_value(t.b[i]), q.back),
-                                               Back::finish(Back::tap_value(t.c[i]), q.back), Back::finish(Back::tap_value(t.d[i]), q.back), tp);
+                Raw a, b, c, d;
+                if constexpr (MODE == kPairs) {
+                    a = Back::template pair_value<0>(t.ab[i], t.ra, x1[i]); b = Back::template pair_value<1>(t.ab[i], t.ra, x1[i]);
+                    c = Back::template pair_value<0>(t.cd[i], t.rb, x1[i]); d = Back::template pair_value<1>(t.cd[i], t.rb, x1[i]);
+                } else {
+                    a = Back::tap_value(t.a[i]); b = Back::tap_value(t.b[i]);
+                    c = Back::tap_value(t.c[i]); d = Back::tap_value(t.d[i]);
+                }
+                typename RZ::Out v = RZ::blend(Back::finish(a, q.back), Back::finish(b, q.back),
+                                               Back::finish(c, q.back), Back::finish(d, q.back), tp);
                 if constexpr (RZ::kAR != IGNORE_AR) { if (!(yin && xin[i])) v = q.bg; }
-                const typename Chain::Value r = Chain::compute_checked(v, p);
-                if (x < aw) W::put(orow, x, r);
+                const typename Chain::Value r = Chain::compute_checked_ops(v, ops);
+                if (x < aw) WP::put(orow, x, r);
             }
         };
         RowTaps t0, t1;
         request(y0, t0);
 #pragma unroll 1
         for (int y = y0; y < yend; y += 2) {
-            request(y + 1, t1);
+            if (y + 1 < yend) request(y + 1, t1);      // wave uniform
             produce(y, t0);
-            request(y + 2, t0);
+            if (y + 2 < yend) request(y + 2, t0);
             produce(y + 1, t1);
         }
     };
+    // Whole-dword reads of 3- and 6-byte elements (and pair reads) touch up to 3 bytes past what they need.  Inside
+    // the image that is the next element or row; only in the image's last row it could leave the allocation.
+    bool tail = false;
     if constexpr (Back::kTapOverread) {
-        // Whole-dword reads of 3- and 6-byte elements touch up to 3 bytes past the element.  Inside the image that
-        // is the next element or row; only in the image's last row it could leave the allocation, so waves whose
-        // taps reach that row read channel by channel instead.
-        const int ylast = y0 + YI + 1 < ah - 1 ? y0 + YI + 1 : ah - 1;    // last row the pipeline may request
+        const int ylast = yend - 1;                                       // last row the wave requests
         const int yl = int(__builtin_floorf(f32(ylast - oy) * q.fy));
         const int yb = yl + 1 < sh - 1 ? yl + 1 : sh - 1;
-        if (Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back))) rows(std::false_type{});
-        else rows(std::true_type{});
+        tail = Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back));
+    }
+    if (tail) {
+        rows(std::integral_constant<int, kSafe>{});
     } else {
-        rows(std::false_type{});
+        if constexpr (Back::kTapPair) {
+            if (!any_clamped) { rows(std::integral_constant<int, kPairs>{}); return; }
+        }
+        rows(std::integral_constant<int, kSingles>{});
     }
 }
 

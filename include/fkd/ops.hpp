@@ -209,43 +209,44 @@ template <class T, int V, bool ALIGNED> FKD_DEV void store_run(T* p, const Slot<
     }
 }
 
-// One element at byte offset `off` of a (typically wave-uniform) base address: the form a gather wants, because
-// the base stays in scalar registers and the lane supplies a 32-bit offset.  The element arrives as raw dwords
-// (ElemBits) and is taken apart later, at its point of use (bits_value), so a consumer can keep many such loads in
-// flight.  The hardware takes global accesses at any byte alignment, so an element whose size is 1, 2 or a
-// multiple of 4 moves as one access.  Sizes 3 and 6 (uchar3, ushort3 ...) move as one or two whole dwords when
-// OVERREAD allows touching up to 3 bytes past the element (the caller guarantees those bytes are inside the
-// allocation); otherwise channel by channel.
+// V consecutive elements (V = 1 or 2) at byte offset `off` of a (typically wave-uniform) base address: the form a
+// gather wants, because the base stays in scalar registers and the lane supplies a 32-bit offset.  The run arrives
+// as raw dwords (RunBits) and is taken apart later, at its point of use (run_value), so a consumer can keep many
+// such loads in flight.  The hardware takes global accesses at any byte alignment, so a run of 1, 2 or a multiple
+// of 4 bytes (up to 16) moves as one access.  Runs of 3 and 6 bytes (uchar3, a uchar3 pair, ushort3) move as one or
+// two whole dwords when OVERREAD allows touching up to 3 bytes past the run (the caller guarantees those bytes are
+// inside the allocation); otherwise channel by channel.
 typedef u16 u16_a1 __attribute__((aligned(1)));
 typedef u32 u32_a1 __attribute__((aligned(1)));
 typedef u32x2_t u32x2_a1 __attribute__((aligned(1)));
 typedef u32x3_t u32x3_a1 __attribute__((aligned(1)));
 typedef u32x4_t u32x4_a1 __attribute__((aligned(1)));
-template <class T> constexpr int overread_bytes() {
-    constexpr int n = int(sizeof(T));
+template <class T, int V = 1> constexpr int overread_bytes() {
+    constexpr int n = int(sizeof(T)) * V;
     return (n == 1 || n == 2 || n % 4 == 0 || n > 16) ? 0 : (n + 3) / 4 * 4 - n;
 }
-template <class T> struct ElemBits {
+template <class T, int V = 1> struct RunBits {
     static_assert(sizeof(T) == sizeof(base_t<T>) * cn_v<T>, "elements are packed channel arrays");
-    static constexpr int kWords = (int(sizeof(T)) + 3) / 4;
+    static constexpr int kWords = (int(sizeof(T)) * V + 3) / 4;
     u32 w[kWords];
 };
-template <class T, bool OVERREAD> FKD_DEV ElemBits<T> load_bits_at(const char* base, u32 off) {
-    constexpr int n = int(sizeof(T));
-    constexpr int W = ElemBits<T>::kWords;
+template <class T, int V, bool OVERREAD> FKD_DEV RunBits<T, V> load_bits_at(const char* base, u32 off) {
+    constexpr int n = int(sizeof(T)) * V;
+    constexpr int W = RunBits<T, V>::kWords;
     // Keeps the offset a 32-bit per-lane value next to the access, so base + offset selects the scalar-base
     // addressing form instead of a hoisted 64-bit per-lane pointer.
     asm volatile("" : "+v"(off));
     const char* a = base + off;
-    ElemBits<T> e;
+    RunBits<T, V> e;
     if constexpr (n == 1) {
         e.w[0] = u32(*reinterpret_cast<const u8*>(a));
     } else if constexpr (n == 2) {
         e.w[0] = u32(*reinterpret_cast<const u16_a1*>(a));
-    } else if constexpr (n > 16 || (overread_bytes<T>() > 0 && !OVERREAD)) {
-        Slot<T> one[1];
-        one[0].v = load_elem(reinterpret_cast<const T*>(a));
-        pack_words<T, 1, W>(one, e.w);
+    } else if constexpr (n > 16 || (overread_bytes<T, V>() > 0 && !OVERREAD)) {
+        Slot<T> run[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) run[i].v = load_elem(reinterpret_cast<const T*>(a) + i);
+        pack_words<T, V, W>(run, e.w);
     } else if constexpr (W == 1) {
         e.w[0] = *reinterpret_cast<const u32_a1*>(a);
     } else if constexpr (W == 2) {
@@ -257,8 +258,8 @@ template <class T, bool OVERREAD> FKD_DEV ElemBits<T> load_bits_at(const char* b
     }
     return e;
 }
-template <class T> FKD_DEV T bits_value(const ElemBits<T>& e) {
-    constexpr int W = ElemBits<T>::kWords;
+template <int K, class T, int V> FKD_DEV T run_value(const RunBits<T, V>& e) {    // K-th element of the run
+    constexpr int W = RunBits<T, V>::kWords;
     u32 w[W];
 #pragma unroll
     for (int i = 0; i < W; ++i) w[i] = e.w[i];
@@ -266,7 +267,7 @@ template <class T> FKD_DEV T bits_value(const ElemBits<T>& e) {
 #pragma unroll
         for (int i = 0; i < W; ++i) asm("" : "+v"(w[i]));   // keep dwords whole: bytes leave through v_cvt_f32_ubyteN / v_bfe
     }
-    return unpack_one<0, T>(w);
+    return unpack_one<K, T>(w);
 }
 
 // Store counterpart of load_bits_at: element sizes 2 and multiples of 4 (up to 16) leave as one access.
@@ -292,6 +293,23 @@ template <class T> FKD_DEV void store_elem_at(char* base, u32 off, const T& v) {
             else if constexpr (W == 3) { u32x3_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; *reinterpret_cast<u32x3_a1*>(a) = q; }
             else { u32x4_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3]; *reinterpret_cast<u32x4_a1*>(a) = q; }
         }
+    }
+}
+
+// A copy of a (wave-uniform) parameter object that is pinned into scalar registers right here: all its scalar loads
+// are issued together and waited for once, instead of one load-and-wait round trip per first use further down.
+template <class T> FKD_DEV T scalar_copy(const T& src) {
+    if constexpr (sizeof(T) % 4 != 0 || sizeof(T) > 256) {
+        return src;
+    } else {
+        constexpr int N = int(sizeof(T)) / 4;
+        u32 w[N];
+        __builtin_memcpy(w, &src, sizeof(T));
+#pragma unroll
+        for (int i = 0; i < N; ++i) asm volatile("" : "+s"(w[i]));
+        T out;
+        __builtin_memcpy(&out, w, sizeof(T));
+        return out;
     }
 }
 
@@ -583,17 +601,24 @@ template <class T> struct Read2D {
     // Tap cursor for gathers: the address of element (x0, y), wave uniform when y is; tap_load adds a 32-bit byte
     // offset and returns the element's raw bits, tap_value takes them apart where they are used.  `last` marks the last row of the image, the only row in which reading a few bytes past an element
     // could leave the allocation; kTapOverread says whether tap_load<true> reads past elements at all.
-    static constexpr bool kTapOverread = detail::overread_bytes<T>() > 0;
+    static constexpr bool kTapOverread = detail::overread_bytes<T, 1>() > 0 || detail::overread_bytes<T, 2>() > 0;
     struct TapRow { const char* p; bool last; };
     FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) {
         return TapRow{reinterpret_cast<const char*>(detail::row_ptr(p.data, p.pitch, x0, y)), y >= int(p.height) - 1};
     }
     FKD_DEV static bool tap_last(const TapRow& r) { return r.last; }
-    using TapBits = detail::ElemBits<T>;
+    using TapBits = detail::RunBits<T, 1>;
     template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params&) {
-        return detail::load_bits_at<T, OVER>(r.p, u32(x) * u32(sizeof(T)));
+        return detail::load_bits_at<T, 1, OVER>(r.p, u32(x) * u32(sizeof(T)));
     }
-    FKD_DEV static Raw tap_value(const TapBits& b) { return detail::bits_value<T>(b); }
+    FKD_DEV static Raw tap_value(const TapBits& b) { return detail::run_value<0>(b); }
+    // Elements x and x+1 in one access (both must exist); may read up to 3 bytes past them like tap_load<true>.
+    static constexpr bool kTapPair = 2 * sizeof(T) <= 16;
+    using PairBits = detail::RunBits<T, 2>;
+    FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params&) {
+        return detail::load_bits_at<T, 2, true>(r.p, u32(x) * u32(sizeof(T)));
+    }
+    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow&, int) { return detail::run_value<K>(b); }
 #endif
 };
 
@@ -648,13 +673,14 @@ struct ReadNV12 {
     using Raw = Out;
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
     FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // gathers element-wise either way
-    static constexpr bool kTapOverread = false;
-    struct TapRow { const char* luma; const char* chroma; int x0; };
+    static constexpr bool kTapOverread = true;    // pair_load only; tap_load reads exact bytes
+    struct TapRow { const char* luma; const char* chroma; int x0; bool last; };
     FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) {
         const char* d = reinterpret_cast<const char*>(p.data);
-        return TapRow{d + size_t(y) * p.pitch, d + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch, x0};
+        return TapRow{d + size_t(y) * p.pitch, d + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch, x0,
+                      (y >> 1) >= int(p.height >> 1) - 1};
     }
-    FKD_DEV static bool tap_last(const TapRow&) { return false; }
+    FKD_DEV static bool tap_last(const TapRow& r) { return r.last; }
     struct TapBits { u32 y, uv; };
     template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params&) {
         u32 xs = u32(r.x0 + x), xc = xs & ~1u;
@@ -669,6 +695,33 @@ struct ReadNV12 {
         o.x = u8(b.y);
         o.y = u8(b.uv & 0xffu);
         o.z = u8(b.uv >> 8);
+        return o;
+    }
+    // Pixels x and x+1: two luma bytes in one access, and the dword at chroma pair x>>1, which holds the pair of
+    // pixel x in its low half and, when x is odd, the pair of pixel x+1 in its high half (x even: same pair).  The
+    // dword reaches one chroma pair past the one needed, hence the over-read flag on the last chroma row.
+    static constexpr bool kTapPair = true;
+    struct PairBits { u32 y, uv; };
+    FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params&) {
+        u32 xs = u32(r.x0 + x), xc = xs & ~1u;
+        asm volatile("" : "+v"(xs), "+v"(xc));
+        PairBits b;
+        b.y = u32(*reinterpret_cast<const detail::u16_a1*>(r.luma + xs));
+        b.uv = *reinterpret_cast<const detail::u32_a1*>(r.chroma + xc);
+        return b;
+    }
+    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) {
+        Out o;
+        if constexpr (K == 0) {
+            o.x = u8(b.y & 0xffu);
+            o.y = u8(b.uv & 0xffu);
+            o.z = u8((b.uv >> 8) & 0xffu);
+        } else {
+            const u32 uv = b.uv >> ((u32(r.x0 + x) & 1u) * 16u);
+            o.x = u8((b.y >> 8) & 0xffu);
+            o.y = u8(uv & 0xffu);
+            o.z = u8((uv >> 8) & 0xffu);
+        }
         return o;
     }
 #endif
@@ -700,6 +753,10 @@ template <class Back> struct Crop {
         return Back::template tap_load<OVER>(r, x, p.back);
     }
     FKD_DEV static Raw tap_value(const TapBits& b) { return Back::tap_value(b); }
+    static constexpr bool kTapPair = Back::kTapPair;
+    using PairBits = typename Back::PairBits;
+    FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
+    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) { return Back::template pair_value<K>(b, r, x); }
 #endif
 };
 
@@ -734,6 +791,10 @@ template <class Back, class... Ops> struct FusedRead {
         return Back::template tap_load<OVER>(r, x, p.back);
     }
     FKD_DEV static Raw tap_value(const TapBits& b) { return Back::tap_value(b); }
+    static constexpr bool kTapPair = Back::kTapPair;
+    using PairBits = typename Back::PairBits;
+    FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
+    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) { return Back::template pair_value<K>(b, r, x); }
 #endif
 };
 
@@ -893,6 +954,9 @@ template <class T> struct Write2D {
     }
     FKD_HD static bool rows_aligned(const Params& p) { return detail::dword_aligned(p.data) && p.pitch % 4 == 0; }
     // Row cursor: one address computation per row, one add per element.
+    // The part of the parameters one plane needs (all of them here).
+    using Plane = Write2D;
+    FKD_DEV static const Params& plane_params(const Params& p, int) { return p; }
     struct RowRef { T* p; };
     FKD_DEV static RowRef row(int y, int, const Params& p) { return RowRef{detail::row_ptr(p.data, p.pitch, 0, y)}; }
     // wave-uniform row address + 32-bit byte offset of the lane: the address form that needs no per-lane 64-bit add
@@ -921,6 +985,9 @@ template <class T> struct TensorWrite {
     FKD_HD static bool rows_aligned(const Params& p) {
         return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0;
     }
+    // The part of the parameters one plane needs (all of them here).
+    using Plane = TensorWrite;
+    FKD_DEV static const Params& plane_params(const Params& p, int) { return p; }
     struct RowRef { T* p; };
     FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{detail::row_ptr(plane(p, z), p.pitch, 0, y)}; }
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
@@ -974,6 +1041,9 @@ template <class T> struct TensorSplit {
         return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 &&
                (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
     }
+    // The part of the parameters one plane needs (all of them here).
+    using Plane = TensorSplit;
+    FKD_DEV static const Params& plane_params(const Params& p, int) { return p; }
     struct RowRef { B* p; size_t px; };
     FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), size_t(p.width) * p.height}; }
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
@@ -1001,6 +1071,8 @@ template <int N, class W> struct BatchWrite {
         for (int i = 0; i < N; ++i) if (!W::rows_aligned(p.plane[i])) return false;
         return true;
     }
+    using Plane = W;
+    FKD_DEV static const typename W::Params& plane_params(const Params& p, int z) { return p.plane[z]; }
     using RowRef = typename W::RowRef;
     FKD_DEV static RowRef row(int y, int z, const Params& p) { return W::row(y, z, p.plane[z]); }
     FKD_DEV static void put(const RowRef& r, int x, const In& v) { W::put(r, x, v); }
@@ -1030,13 +1102,17 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     // compute() through the operations' straight-line variants, falling back to compute() for the (rare) elements
     // they cannot vouch for.  Same result as compute(), fewer instructions on the common path.
     static constexpr bool kQuick = any_quick<Ops...>();
-    FKD_DEV static Value compute_checked(const typename R::Out& v, const Params& p) {
-        if constexpr (!kQuick) {
-            return compute(v, p);
+    using OpParams = Tup<typename Ops::Params...>;
+    FKD_DEV static Value compute_checked(const typename R::Out& v, const Params& p) { return compute_checked_ops(v, p.ops); }
+    FKD_DEV static Value compute_checked_ops(const typename R::Out& v, const OpParams& ops) {
+        if constexpr (sizeof...(Ops) == 0) {
+            return v;
+        } else if constexpr (!kQuick) {
+            return fold<Ops...>(v, ops);
         } else {
             bool ok = true;
-            Value r = fold_quick<Ops...>(v, p.ops, ok);
-            if (__builtin_expect(!ok, 0)) r = compute(v, p);
+            Value r = fold_quick<Ops...>(v, ops, ok);
+            if (__builtin_expect(!ok, 0)) r = fold<Ops...>(v, ops);
             return r;
         }
     }
