@@ -100,6 +100,9 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
 #ifndef FKD_GATHER_YI
 #define FKD_GATHER_YI 2
 #endif
+#ifndef FKD_GATHER_ADJ
+#define FKD_GATHER_ADJ 0
+#endif
 #ifndef FKD_GATHER_BY
 #define FKD_GATHER_BY 4
 #endif
@@ -156,6 +159,11 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; }
     const int sw = Back::width(q.back), sh = Back::height(q.back);
 
+    // Pixels of a lane: XI adjacent ones (their results leave as one wide store per plane), or 64 apart.
+    auto xof = [&](int i) {
+        if constexpr (FKD_GATHER_ADJ) return tx0 + int(threadIdx.x) * XI + i;
+        else return tx0 + int(threadIdx.x) + kGatherBX * i;
+    };
     // Horizontal part, per lane, shared by the YI rows.  float(x1) and float(x1 + 1) are taken as floor(sx) and
     // floor(sx) + 1, the same numbers (exact integers below 2^24).
     int x1[XI], x2[XI];
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     bool lane_clamped = false;
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
-        int x = tx0 + int(threadIdx.x) + kGatherBX * i;
+        int x = xof(i);
         x = x < aw ? x : aw - 1;                                   // idle lanes shadow the last column
         xin[i] = true;
         if constexpr (RZ::kAR != IGNORE_AR) xin[i] = x >= q.x1 && x <= q.x2;
@@ -227,9 +235,9 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
             bool yin = true;
             if constexpr (RZ::kAR != IGNORE_AR) yin = y >= q.y1 && y <= q.y2;
             const typename WP::RowRef orow = WP::row(y, z, wpar);
+            Slot<typename Chain::Value> res[XI];
 #pragma unroll
             for (int i = 0; i < XI; ++i) {
-                const int x = tx0 + int(threadIdx.x) + kGatherBX * i;
                 typename RZ::Taps tp;
                 tp.w00 = ax[i] * t.ay; tp.w10 = bx[i] * t.ay; tp.w01 = ax[i] * t.by; tp.w11 = bx[i] * t.by;
                 Raw a, b, c, d;
@@ -243,8 +251,18 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
                 typename RZ::Out v = RZ::blend(Back::finish(a, q.back), Back::finish(b, q.back),
                                                Back::finish(c, q.back), Back::finish(d, q.back), tp);
                 if constexpr (RZ::kAR != IGNORE_AR) { if (!(yin && xin[i])) v = q.bg; }
-                const typename Chain::Value r = Chain::compute_checked_ops(v, ops);
-                if (x < aw) WP::put(orow, x, r);
+                res[i].v = Chain::compute_checked_ops(v, ops);
+            }
+            if constexpr (FKD_GATHER_ADJ && XI > 1) {
+                if (xof(XI - 1) < aw) {
+                    WP::template put_run<XI>(orow, xof(0), res);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < XI; ++i) if (xof(i) < aw) WP::put(orow, xof(i), res[i].v);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < XI; ++i) if (xof(i) < aw) WP::put(orow, xof(i), res[i].v);
             }
         };
         RowTaps t0, t1;

@@ -33,12 +33,19 @@ template <class T> struct alignas(sizeof(T) % 4 != 0 ? 4 : alignof(T)) Slot { T 
 #if defined(FKD_DEVICE_CODE)
 namespace detail {
 
+// Every pointer this library dereferences on the device is device (global) memory.  Saying so at the access keeps
+// the accesses global_load/global_store (scalar base + lane offset addressing, vmcnt only) even where the pointer
+// value went through integer registers and the compiler can no longer infer its address space.
+#define FKD_GLOBAL __attribute__((address_space(1)))
+template <class T> FKD_DEV const FKD_GLOBAL T* gconst(const void* p) { return (const FKD_GLOBAL T*)p; }
+template <class T> FKD_DEV FKD_GLOBAL T* gmut(void* p) { return (FKD_GLOBAL T*)p; }
+
 template <class T> FKD_DEV T load_elem(const T* p) {
     T v;
     if constexpr (cn_v<T> == 1) {
-        v = *p;
+        v = *gconst<T>(p);
     } else {
-        const base_t<T>* b = reinterpret_cast<const base_t<T>*>(p);
+        const FKD_GLOBAL base_t<T>* b = gconst<base_t<T>>(p);
         chan<0>(v) = b[0];
         chan<1>(v) = b[1];
         if constexpr (cn_v<T> > 2) chan<2>(v) = b[2];
@@ -48,9 +55,9 @@ template <class T> FKD_DEV T load_elem(const T* p) {
 }
 template <class T> FKD_DEV void store_elem(T* p, const T& v) {
     if constexpr (cn_v<T> == 1) {
-        *p = v;
+        *gmut<T>(p) = v;
     } else {
-        base_t<T>* b = reinterpret_cast<base_t<T>*>(p);
+        FKD_GLOBAL base_t<T>* b = gmut<base_t<T>>(p);
         b[0] = chan<0>(v);
         b[1] = chan<1>(v);
         if constexpr (cn_v<T> > 2) b[2] = chan<2>(v);
@@ -69,17 +76,17 @@ typedef u32x4_t u32x4_a4 __attribute__((aligned(4)));
 template <int W> FKD_DEV void load_words(const void* p, u32 (&w)[W]) {
     static_assert(W >= 1 && (W <= 4 || W % 4 == 0), "runs are 1-4 dwords or whole 16-byte groups");
     if constexpr (W == 1) {
-        w[0] = *reinterpret_cast<const u32*>(p);
+        w[0] = *gconst<u32>(p);
     } else if constexpr (W == 2) {
-        const u32x2_t v = *reinterpret_cast<const u32x2_a4*>(p);
+        const u32x2_t v = *gconst<u32x2_a4>(p);
         w[0] = v.x; w[1] = v.y;
     } else if constexpr (W == 3) {
-        const u32x3_t v = *reinterpret_cast<const u32x3_a4*>(p);
+        const u32x3_t v = *gconst<u32x3_a4>(p);
         w[0] = v.x; w[1] = v.y; w[2] = v.z;
     } else {
 #pragma unroll
         for (int i = 0; i < W / 4; ++i) {
-            const u32x4_t v = reinterpret_cast<const u32x4_a4*>(p)[i];
+            const u32x4_t v = gconst<u32x4_a4>(p)[i];
             w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
         }
     }
@@ -87,18 +94,18 @@ template <int W> FKD_DEV void load_words(const void* p, u32 (&w)[W]) {
 template <int W> FKD_DEV void store_words(void* p, const u32 (&w)[W]) {
     static_assert(W >= 1 && (W <= 4 || W % 4 == 0), "runs are 1-4 dwords or whole 16-byte groups");
     if constexpr (W == 1) {
-        *reinterpret_cast<u32*>(p) = w[0];
+        *gmut<u32>(p) = w[0];
     } else if constexpr (W == 2) {
         u32x2_t v; v.x = w[0]; v.y = w[1];
-        *reinterpret_cast<u32x2_a4*>(p) = v;
+        *gmut<u32x2_a4>(p) = v;
     } else if constexpr (W == 3) {
         u32x3_t v; v.x = w[0]; v.y = w[1]; v.z = w[2];
-        *reinterpret_cast<u32x3_a4*>(p) = v;
+        *gmut<u32x3_a4>(p) = v;
     } else {
 #pragma unroll
         for (int i = 0; i < W / 4; ++i) {
             u32x4_t v; v.x = w[4 * i]; v.y = w[4 * i + 1]; v.z = w[4 * i + 2]; v.w = w[4 * i + 3];
-            reinterpret_cast<u32x4_a4*>(p)[i] = v;
+            gmut<u32x4_a4>(p)[i] = v;
         }
     }
 }
@@ -239,22 +246,22 @@ template <class T, int V, bool OVERREAD> FKD_DEV RunBits<T, V> load_bits_at(cons
     const char* a = base + off;
     RunBits<T, V> e;
     if constexpr (n == 1) {
-        e.w[0] = u32(*reinterpret_cast<const u8*>(a));
+        e.w[0] = u32(*gconst<u8>(a));
     } else if constexpr (n == 2) {
-        e.w[0] = u32(*reinterpret_cast<const u16_a1*>(a));
+        e.w[0] = u32(*gconst<u16_a1>(a));
     } else if constexpr (n > 16 || (overread_bytes<T, V>() > 0 && !OVERREAD)) {
         Slot<T> run[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) run[i].v = load_elem(reinterpret_cast<const T*>(a) + i);
         pack_words<T, V, W>(run, e.w);
     } else if constexpr (W == 1) {
-        e.w[0] = *reinterpret_cast<const u32_a1*>(a);
+        e.w[0] = *gconst<u32_a1>(a);
     } else if constexpr (W == 2) {
-        const u32x2_t v = *reinterpret_cast<const u32x2_a1*>(a); e.w[0] = v.x; e.w[1] = v.y;
+        const u32x2_t v = *gconst<u32x2_a1>(a); e.w[0] = v.x; e.w[1] = v.y;
     } else if constexpr (W == 3) {
-        const u32x3_t v = *reinterpret_cast<const u32x3_a1*>(a); e.w[0] = v.x; e.w[1] = v.y; e.w[2] = v.z;
+        const u32x3_t v = *gconst<u32x3_a1>(a); e.w[0] = v.x; e.w[1] = v.y; e.w[2] = v.z;
     } else {
-        const u32x4_t v = *reinterpret_cast<const u32x4_a1*>(a); e.w[0] = v.x; e.w[1] = v.y; e.w[2] = v.z; e.w[3] = v.w;
+        const u32x4_t v = *gconst<u32x4_a1>(a); e.w[0] = v.x; e.w[1] = v.y; e.w[2] = v.z; e.w[3] = v.w;
     }
     return e;
 }
@@ -285,14 +292,39 @@ template <class T> FKD_DEV void store_elem_at(char* base, u32 off, const T& v) {
         u32 w[W];
         if constexpr (n == 2) {
             w[0] = to_bits(chan<0>(v)) | (to_bits(chan<1>(v)) << 8);
-            *reinterpret_cast<u16_a1*>(a) = u16(w[0]);
+            *gmut<u16_a1>(a) = u16(w[0]);
         } else {
             pack_words<T, 1, W>(one, w);
-            if constexpr (W == 1) { *reinterpret_cast<u32_a1*>(a) = w[0]; }
-            else if constexpr (W == 2) { u32x2_t q; q.x = w[0]; q.y = w[1]; *reinterpret_cast<u32x2_a1*>(a) = q; }
-            else if constexpr (W == 3) { u32x3_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; *reinterpret_cast<u32x3_a1*>(a) = q; }
-            else { u32x4_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3]; *reinterpret_cast<u32x4_a1*>(a) = q; }
+            if constexpr (W == 1) { *gmut<u32_a1>(a) = w[0]; }
+            else if constexpr (W == 2) { u32x2_t q; q.x = w[0]; q.y = w[1]; *gmut<u32x2_a1>(a) = q; }
+            else if constexpr (W == 3) { u32x3_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; *gmut<u32x3_a1>(a) = q; }
+            else { u32x4_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3]; *gmut<u32x4_a1>(a) = q; }
         }
+    }
+}
+
+// V consecutive elements to byte offset `off` of a wave-uniform base, as one wide access when the run is a whole
+// number of dwords (any byte alignment), else element by element.
+template <class T, int V> FKD_DEV void store_run_at(char* base, u32 off, const Slot<T> (&v)[V]) {
+    constexpr int n = int(sizeof(T)) * V;
+    constexpr bool packed = sizeof(T) == sizeof(base_t<T>) * cn_v<T>;
+    if constexpr (packed && n % 4 == 0 && n <= 16) {
+        constexpr int W = n / 4;
+        u32 w[W];
+        pack_words<T, V, W>(v, w);
+        if constexpr (sizeof(base_t<T>) < 4) {
+#pragma unroll
+            for (int i = 0; i < W; ++i) asm("" : "+v"(w[i]));
+        }
+        asm volatile("" : "+v"(off));
+        char* a = base + off;
+        if constexpr (W == 1) { *gmut<u32_a1>(a) = w[0]; }
+        else if constexpr (W == 2) { u32x2_t q; q.x = w[0]; q.y = w[1]; *gmut<u32x2_a1>(a) = q; }
+        else if constexpr (W == 3) { u32x3_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; *gmut<u32x3_a1>(a) = q; }
+        else { u32x4_t q; q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3]; *gmut<u32x4_a1>(a) = q; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) store_elem_at<T>(base, off + u32(i) * u32(sizeof(T)), v[i].v);
     }
 }
 
@@ -660,8 +692,8 @@ struct ReadNV12 {
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) {
         Out o;
-        o.x = p.data[size_t(y) * p.pitch + x];
-        const u8* c = p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch + 2 * (x >> 1);
+        o.x = *detail::gconst<u8>(p.data + size_t(y) * p.pitch + x);
+        const FKD_GLOBAL u8* c = detail::gconst<u8>(p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch + 2 * (x >> 1));
         o.y = c[0];
         o.z = c[1];
         return o;
@@ -686,8 +718,8 @@ struct ReadNV12 {
         u32 xs = u32(r.x0 + x), xc = xs & ~1u;
         asm volatile("" : "+v"(xs), "+v"(xc));      // 32-bit lane offsets against scalar row addresses
         TapBits b;
-        b.y = u32(*reinterpret_cast<const u8*>(r.luma + xs));
-        b.uv = u32(*reinterpret_cast<const detail::u16_a1*>(r.chroma + xc));   // (U,V) pair in one access
+        b.y = u32(*detail::gconst<u8>(r.luma + xs));
+        b.uv = u32(*detail::gconst<detail::u16_a1>(r.chroma + xc));   // (U,V) pair in one access
         return b;
     }
     FKD_DEV static Raw tap_value(const TapBits& b) {
@@ -706,8 +738,8 @@ struct ReadNV12 {
         u32 xs = u32(r.x0 + x), xc = xs & ~1u;
         asm volatile("" : "+v"(xs), "+v"(xc));
         PairBits b;
-        b.y = u32(*reinterpret_cast<const detail::u16_a1*>(r.luma + xs));
-        b.uv = *reinterpret_cast<const detail::u32_a1*>(r.chroma + xc);
+        b.y = u32(*detail::gconst<detail::u16_a1>(r.luma + xs));
+        b.uv = *detail::gconst<detail::u32_a1>(r.chroma + xc);
         return b;
     }
     template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) {
@@ -963,6 +995,9 @@ template <class T> struct Write2D {
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
         detail::store_elem_at<T>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
     }
+    template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<T> (&v)[V]) {
+        detail::store_run_at<T, V>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
+    }
 #endif
 };
 
@@ -993,6 +1028,9 @@ template <class T> struct TensorWrite {
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
         detail::store_elem_at<T>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
     }
+    template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<T> (&v)[V]) {
+        detail::store_run_at<T, V>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
+    }
 #endif
 };
 
@@ -1011,10 +1049,11 @@ template <class T> struct TensorSplit {
     FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
         B* w = at(p, x, y, z);
         const size_t px = size_t(p.width) * p.height;
-        w[0] = chan<0>(v);
-        w[px] = chan<1>(v);
-        if constexpr (cn_v<T> > 2) w[2 * px] = chan<2>(v);
-        if constexpr (cn_v<T> > 3) w[3 * px] = chan<3>(v);
+        FKD_GLOBAL B* gw = detail::gmut<B>(w);
+        gw[0] = chan<0>(v);
+        gw[px] = chan<1>(v);
+        if constexpr (cn_v<T> > 2) gw[2 * px] = chan<2>(v);
+        if constexpr (cn_v<T> > 3) gw[3 * px] = chan<3>(v);
     }
     template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         B* w = at(p, x, y, z);
@@ -1049,10 +1088,30 @@ template <class T> struct TensorSplit {
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
         u32 off = u32(x) * u32(sizeof(B));   // one lane offset, four wave-uniform plane row addresses
         asm volatile("" : "+v"(off));
-        *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p) + off) = chan<0>(v);
-        *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p + r.px) + off) = chan<1>(v);
-        if constexpr (cn_v<T> > 2) *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p + 2 * r.px) + off) = chan<2>(v);
-        if constexpr (cn_v<T> > 3) *reinterpret_cast<B*>(reinterpret_cast<char*>(r.p + 3 * r.px) + off) = chan<3>(v);
+        *detail::gmut<B>(reinterpret_cast<char*>(r.p) + off) = chan<0>(v);
+        *detail::gmut<B>(reinterpret_cast<char*>(r.p + r.px) + off) = chan<1>(v);
+        if constexpr (cn_v<T> > 2) *detail::gmut<B>(reinterpret_cast<char*>(r.p + 2 * r.px) + off) = chan<2>(v);
+        if constexpr (cn_v<T> > 3) *detail::gmut<B>(reinterpret_cast<char*>(r.p + 3 * r.px) + off) = chan<3>(v);
+    }
+    template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<T> (&v)[V]) {
+        const u32 off = u32(x) * u32(sizeof(B));
+        Slot<B> c[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) c[i].v = chan<0>(v[i].v);
+        detail::store_run_at<B, V>(reinterpret_cast<char*>(r.p), off, c);
+#pragma unroll
+        for (int i = 0; i < V; ++i) c[i].v = chan<1>(v[i].v);
+        detail::store_run_at<B, V>(reinterpret_cast<char*>(r.p + r.px), off, c);
+        if constexpr (cn_v<T> > 2) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) c[i].v = chan<2>(v[i].v);
+            detail::store_run_at<B, V>(reinterpret_cast<char*>(r.p + 2 * r.px), off, c);
+        }
+        if constexpr (cn_v<T> > 3) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) c[i].v = chan<3>(v[i].v);
+            detail::store_run_at<B, V>(reinterpret_cast<char*>(r.p + 3 * r.px), off, c);
+        }
     }
 #endif
 };
@@ -1076,6 +1135,7 @@ template <int N, class W> struct BatchWrite {
     using RowRef = typename W::RowRef;
     FKD_DEV static RowRef row(int y, int z, const Params& p) { return W::row(y, z, p.plane[z]); }
     FKD_DEV static void put(const RowRef& r, int x, const In& v) { W::put(r, x, v); }
+    template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<In> (&v)[V]) { W::template put_run<V>(r, x, v); }
 #endif
 };
 
