@@ -102,3 +102,21 @@ def crop_swap_u8(src, rects, out):
 def copy_f32(src, out):
     """src/out (H,W) f32 cuda: read -> write with no compute operation."""
     _ok(cases().fklcase_copy_f32(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, _p(out), out.stride(0) * 4))
+
+
+def div_f32(src, d, out):
+    """src/out (H,W) f32 cuda: out = src / d through Read -> Div -> Write."""
+    _ok(cases().fklcase_div_f32(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, C.c_float(float(d)),
+                                _p(out), out.stride(0) * 4))
+
+
+def div_f32x3(src, d, out):
+    """src/out (H,W,3) f32 cuda, d three divisors (one per channel)."""
+    dd = _host(d, np.float32)
+    _ok(cases().fklcase_div_f32x3(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4,
+                                  dd.ctypes.data_as(C.c_void_p), _p(out), out.stride(0) * 4))
+
+
+def saturate_f32_u8(src, out):
+    """src (H,W) f32 cuda, out (H,W) u8 cuda: SaturateCast<float, uchar>."""
+    _ok(cases().fklcase_saturate_f32_u8(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, _p(out), out.stride(0)))

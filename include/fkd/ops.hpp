@@ -498,7 +498,7 @@ template <class I, class O> struct SaturateCast {
             return s;
         } else if constexpr (__is_same(S, f32) && __is_same(D, u8)) {
             // v_cvt_pk_u8_f32: round half to even, clamp to [0, 255], NaN -> 0 in one instruction.  Checked against
-            // the reference rule for all 2^32 float bit patterns (tests/test_gpu_saturate.py).
+            // the reference rule for all 2^32 float bit patterns (tests/test_gpu_exhaustive.py).
             return u8(__builtin_amdgcn_cvt_pk_u8_f32(s, 0u, 0u));
         } else if constexpr (__is_floating_point(S) && __is_integral(D)) {
             // Branch free.  Round half to even under the default rounding mode (v_rndne_f32 / v_rndne_f64), then

@@ -212,6 +212,35 @@ int fklcase_copy_f32(void* stream_, const float* in, int w, int h, int pitch, fl
         for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(i, o, stream);
     });
 }
+// Single-operation chains for the exhaustive numeric tests.
+int fklcase_div_f32(void* stream_, const float* in, int w, int h, int pitch, float d, float* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<float>(in, w, h, pitch);
+        const auto o = dev2d<float>(out, w, h, out_pitch);
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, float>::build(i.ptr()), Div<float>::build(d),
+                                          PerThreadWrite<ND::_2D, float>::build(o.ptr()));
+    });
+}
+int fklcase_div_f32x3(void* stream_, const float* in, int w, int h, int pitch, const float* d, float* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<float3>(in, w, h, pitch);
+        const auto o = dev2d<float3>(out, w, h, out_pitch);
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, float3>::build(i.ptr()),
+                                          Div<float3>::build(make_<float3>(d[0], d[1], d[2])),
+                                          PerThreadWrite<ND::_2D, float3>::build(o.ptr()));
+    });
+}
+int fklcase_saturate_f32_u8(void* stream_, const float* in, int w, int h, int pitch, uint8_t* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<float>(in, w, h, pitch);
+        const auto o = dev2d<uchar>(out, w, h, out_pitch);
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, float>::build(i.ptr()), SaturateCast<float, uchar>::build(),
+                                          PerThreadWrite<ND::_2D, uchar>::build(o.ptr()));
+    });
+}
 int fklcase_crop_swap_u8_b4(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
     return guarded([&] { crop_swap_u8<4>(stream, src, w, h, pitch, rects, out); });
 }

@@ -1,0 +1,160 @@
+"""Every fp32 bit pattern through the two device operations whose instruction sequences differ from a plain
+translation of the reference: Div (reciprocal-based five-instruction quotient for launch-constant divisors, generic
+division for everything it cannot vouch for) and SaturateCast<float, uchar> (v_cvt_pk_u8_f32).
+
+The bulk comparator runs on the GPU too (2^32 inputs per divisor): torch's own fp32 division / round-half-even.
+It is itself checked here, on samples brought back to the host, against numpy's IEEE division and against the C
+oracle's saturate_cast (which is pinned to the reference's known answers in test_oracle.py)."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from fusedkernellibrary_amd import cases, workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+CHUNK_LOG2 = 28            # 2^28 patterns per launch, 16 launches cover fp32
+SIDE = 1 << (CHUNK_LOG2 // 2)
+
+
+def _bits(f):
+    return np.float32(f).view(np.uint32)
+
+
+def _f(bits):
+    return np.uint32(bits).view(np.float32)
+
+
+def _chunk(torch, device, k):
+    """All bit patterns k*2^28 .. (k+1)*2^28 - 1 as a (SIDE, SIDE) float32 tensor."""
+    base = torch.arange(1 << CHUNK_LOG2, dtype=torch.int64, device=device) + (k << CHUNK_LOG2)
+    return base.to(torch.int32).view(torch.float32).reshape(SIDE, SIDE)
+
+
+def _same(torch, got, want):
+    """Bitwise equal, or both NaN (payloads of NaN results are not part of the contract)."""
+    gi, wi = got.view(torch.int32), want.view(torch.int32)
+    ok = (gi == wi) | (torch.isnan(got) & torch.isnan(want))
+    return bool(ok.all()), ok
+
+
+# Divisors: the normalisation constants of benchmark configuration 3, values whose mantissa is all zeros / all ones
+# (where a reciprocal is least accurate), negatives, both ends of the range the quick path accepts, and values
+# outside it (denormal, huge, tiny: these must take the generic division).
+DIVISORS = [
+    tuple(float(v) for v in wl.C3_STD),
+    (1.0, float(_f(0x3FFFFFFF)), float(_f(0x3F800001))),
+    (3.0, -7.25, 0.1),
+    (float(_f(0x2B800000)), float(_f(0x53800000)), 255.0),          # 2^-40, 2^40
+    (float(_f(0x2B7FFFFF)), float(_f(0x53800001)), float(_f(0x00000123))),   # just outside, denormal
+    (float(_f(0x7F7FFFFF)), float(_f(0x00800000)), -1.0e-3),
+]
+
+
+def test_torch_division_is_ieee_on_samples(device):
+    import torch
+    rng = np.random.RandomState(7)
+    x = rng.randint(0, 1 << 32, size=1 << 22, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    xt = torch.from_numpy(x).to(device)
+    for trio in DIVISORS:
+        for d in trio:
+            with np.errstate(all="ignore"):
+                want = x / np.float32(d)
+            got = (xt / torch.tensor(d, dtype=torch.float32, device=device)).cpu().numpy()
+            same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+            assert same.all(), (d, x[~same][:4])
+
+
+@pytest.mark.parametrize("trio", DIVISORS)
+def test_div_float3_every_bit_pattern(device, trio):
+    import torch
+    dvec = torch.tensor(trio, dtype=torch.float32, device=device)
+    out = torch.empty((SIDE, SIDE, 3), dtype=torch.float32, device=device)
+    for k in range(16):
+        x = _chunk(torch, device, k)
+        src = x.unsqueeze(-1).expand(SIDE, SIDE, 3).contiguous()
+        cases.div_f32x3(src, trio, out)
+        torch.cuda.synchronize()
+        want = src / dvec
+        ok, mask = _same(torch, out, want)
+        if not ok:
+            bad = (~mask).nonzero()[0].tolist()
+            y, xx, c = bad
+            pytest.fail(f"x bits {int(src[y, xx, c].view(torch.int32)) & 0xffffffff:#010x} / {trio[c]!r}: "
+                        f"got {float(out[y, xx, c])!r} want {float(want[y, xx, c])!r}")
+        del src, want
+
+
+def test_div_float3_mixed_channels(device):
+    """Channels of one pixel decide together whether the quick path is taken: mix ordinary values with zeros,
+    denormals, infinities and NaNs in the other channels."""
+    import torch
+    rng = np.random.RandomState(11)
+    n = 1 << 20
+    special = np.array([0x00000000, 0x80000000, 0x00000001, 0x807FFFFF, 0x7F800000, 0xFF800000, 0x7FC00000, 0x7F800001,
+                        0x21800000, 0x217FFFFF, 0x5D800000, 0x5D800001, 0x3F800000, 0xC2F6E979], np.uint32)
+    px = rng.randint(0, 1 << 32, size=(n, 3), dtype=np.uint64).astype(np.uint32)
+    pick = rng.randint(0, 4, size=(n, 3)) == 0
+    px[pick] = special[rng.randint(0, len(special), size=int(pick.sum()))]
+    src_np = px.view(np.float32).reshape(1 << 10, 1 << 10, 3)
+    src = torch.from_numpy(src_np).to(device)
+    out = torch.empty_like(src)
+    for trio in DIVISORS:
+        cases.div_f32x3(src, trio, out)
+        torch.cuda.synchronize()
+        with np.errstate(all="ignore"):
+            want = src_np / np.array(trio, np.float32)
+        got = out.cpu().numpy()
+        same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+        assert same.all(), (trio, src_np[~same][:4], got[~same][:4], want[~same][:4])
+
+
+@pytest.mark.parametrize("d", [float(wl.C3_STD[0]), 1.0, float(_f(0x3FFFFFFF)), -0.3, 1e30])
+def test_div_scalar_every_bit_pattern(device, d):
+    import torch
+    out = torch.empty((SIDE, SIDE), dtype=torch.float32, device=device)
+    dt = torch.tensor(d, dtype=torch.float32, device=device)
+    for k in range(16):
+        x = _chunk(torch, device, k)
+        cases.div_f32(x, d, out)
+        torch.cuda.synchronize()
+        ok, mask = _same(torch, out, x / dt)
+        if not ok:
+            y, xx = (~mask).nonzero()[0].tolist()
+            pytest.fail(f"x bits {int(x[y, xx].view(torch.int32)) & 0xffffffff:#010x} / {d!r}: got {float(out[y, xx])!r}")
+
+
+def _torch_saturate_u8(torch, x):
+    r = torch.round(x)                                   # half to even
+    r = torch.where(torch.isnan(x), torch.zeros_like(r), r)
+    return r.clamp(0.0, 255.0).to(torch.uint8)
+
+
+def test_torch_saturate_model_matches_oracle_on_samples(device):
+    import torch
+    lib = ol.oracle()
+    rng = np.random.RandomState(5)
+    halves = np.arange(-2, 259, dtype=np.float32)[:, None] + np.array([0.0, 0.5], np.float32)[None, :]
+    near = np.concatenate([np.nextafter(halves, np.float32(-1e9)), halves, np.nextafter(halves, np.float32(1e9))]).ravel()
+    special = np.array([0x7F800000, 0xFF800000, 0x7FC00000, 0xFFC00001, 0x7F800001, 0x00000001, 0x80000001, 0x80000000,
+                        0x437F0000, 0x437F8000, 0x437F7FFF, 0x4B000000, 0xCB000000], np.uint32).view(np.float32)
+    rnd = rng.randint(0, 1 << 32, size=1 << 16, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    small = (rng.rand(1 << 16).astype(np.float32) * 300 - 20).astype(np.float32)
+    x = np.concatenate([near.astype(np.float32), special, rnd, small])
+    want = np.array([lib.fklo_saturate_cast_u8(float(v)) for v in x], np.uint8)
+    got = _torch_saturate_u8(torch, torch.from_numpy(x).to(device)).cpu().numpy()
+    assert (got == want).all(), x[got != want][:8]
+
+
+def test_saturate_cast_f32_u8_every_bit_pattern(device):
+    import torch
+    out = torch.empty((SIDE, SIDE), dtype=torch.uint8, device=device)
+    for k in range(16):
+        x = _chunk(torch, device, k)
+        cases.saturate_f32_u8(x, out)
+        torch.cuda.synchronize()
+        want = _torch_saturate_u8(torch, x)
+        bad = out != want
+        if bool(bad.any()):
+            y, xx = bad.nonzero()[0].tolist()
+            pytest.fail(f"x bits {int(x[y, xx].view(torch.int32)) & 0xffffffff:#010x}: got {int(out[y, xx])} want {int(want[y, xx])}")
