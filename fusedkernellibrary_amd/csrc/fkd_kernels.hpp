@@ -168,7 +168,7 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     // floor(sx) + 1, the same numbers (exact integers below 2^24).
     int x1[XI], x2[XI];
     f32 ax[XI], bx[XI];
-    bool xin[XI];
+    bool xin[XI], clamped[XI];
     bool lane_clamped = false;
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
@@ -183,7 +183,8 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
         const int xi = int(f1);
         x1[i] = xi < 0 ? 0 : (xi < sw - 1 ? xi : sw - 1);       // no-op wherever the reference is in bounds
         x2[i] = x1[i] + 1 < sw - 1 ? x1[i] + 1 : sw - 1;
-        lane_clamped = lane_clamped || x1[i] + 1 > sw - 1;
+        clamped[i] = x1[i] + 1 > sw - 1;
+        lane_clamped = lane_clamped || clamped[i];
     }
     const bool any_clamped = __builtin_amdgcn_ballot_w64(lane_clamped) != 0;
 
@@ -193,16 +194,19 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     // Three ways to fetch the taps of a row, chosen per wave:
     //   kPairs    the two horizontally adjacent taps of a pixel come in one access (possible when no lane of the
     //             wave has its right tap clamped to the last column), halving the number of gather instructions;
+    //   kPairsSel the same for waves with clamped lanes: such a lane fetches the pair ending at the last column and
+    //             uses its second element for both taps;
     //   kSingles  one access per tap, whole dwords;
     //   kSafe     one access per tap, never touching a byte outside the elements (channel by channel for 3- and
     //             6-byte elements): for waves whose taps reach the last row of the image.
-    constexpr int kSafe = 0, kSingles = 1, kPairs = 2;
+    constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3;
     const int yend = y0 + YI < ah ? y0 + YI : ah;
     auto rows = [&](auto mode_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
+        constexpr bool PAIRED = MODE == kPairs || MODE == kPairsSel;
         struct RowTaps {
-            typename Back::TapBits a[MODE == kPairs ? 1 : XI], b[MODE == kPairs ? 1 : XI], c[MODE == kPairs ? 1 : XI], d[MODE == kPairs ? 1 : XI];
-            typename Back::PairBits ab[MODE == kPairs ? XI : 1], cd[MODE == kPairs ? XI : 1];
+            typename Back::TapBits a[PAIRED ? 1 : XI], b[PAIRED ? 1 : XI], c[PAIRED ? 1 : XI], d[PAIRED ? 1 : XI];
+            typename Back::PairBits ab[PAIRED ? XI : 1], cd[PAIRED ? XI : 1];
             typename Back::TapRow ra, rb;
             f32 ay, by;
         };
@@ -219,9 +223,10 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
             t.rb = Back::tap_row(0, yb, z, q.back);
 #pragma unroll
             for (int i = 0; i < XI; ++i) {
-                if constexpr (MODE == kPairs) {
-                    t.ab[i] = Back::pair_load(t.ra, x1[i], q.back);
-                    t.cd[i] = Back::pair_load(t.rb, x1[i], q.back);
+                if constexpr (PAIRED) {
+                    const int xl = MODE == kPairsSel ? x1[i] - int(clamped[i]) : x1[i];
+                    t.ab[i] = Back::pair_load(t.ra, xl, q.back);
+                    t.cd[i] = Back::pair_load(t.rb, xl, q.back);
                 } else {
                     t.a[i] = Back::template tap_load<MODE == kSingles>(t.ra, x1[i], q.back);
                     t.b[i] = Back::template tap_load<MODE == kSingles>(t.ra, x2[i], q.back);
@@ -241,9 +246,11 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
                 typename RZ::Taps tp;
                 tp.w00 = ax[i] * t.ay; tp.w10 = bx[i] * t.ay; tp.w01 = ax[i] * t.by; tp.w11 = bx[i] * t.by;
                 Raw a, b, c, d;
-                if constexpr (MODE == kPairs) {
-                    a = Back::template pair_value<0>(t.ab[i], t.ra, x1[i]); b = Back::template pair_value<1>(t.ab[i], t.ra, x1[i]);
-                    c = Back::template pair_value<0>(t.cd[i], t.rb, x1[i]); d = Back::template pair_value<1>(t.cd[i], t.rb, x1[i]);
+                if constexpr (PAIRED) {
+                    const int xl = MODE == kPairsSel ? x1[i] - int(clamped[i]) : x1[i];
+                    Back::pair_values(t.ab[i], t.ra, xl, a, b);
+                    Back::pair_values(t.cd[i], t.rb, xl, c, d);
+                    if constexpr (MODE == kPairsSel) { if (clamped[i]) { a = b; c = d; } }
                 } else {
                     a = Back::tap_value(t.a[i]); b = Back::tap_value(t.b[i]);
                     c = Back::tap_value(t.c[i]); d = Back::tap_value(t.d[i]);
@@ -289,6 +296,7 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     } else {
         if constexpr (Back::kTapPair) {
             if (!any_clamped) { rows(std::integral_constant<int, kPairs>{}); return; }
+            if (sw >= 2) { rows(std::integral_constant<int, kPairsSel>{}); return; }
         }
         rows(std::integral_constant<int, kSingles>{});
     }

@@ -277,6 +277,57 @@ template <int K, class T, int V> FKD_DEV T run_value(const RunBits<T, V>& e) {  
     return unpack_one<K, T>(w);
 }
 
+// Two consecutive elements for a gather, fetched as ONE dword-aligned window.  A vector-L1 access that starts on a
+// dword boundary costs the same whether it is 4 or 16 bytes wide, while a wide access at a byte address costs about
+// twice as much; so for elements whose size is not a multiple of 4 the window starts at the dword boundary at or
+// below the first element (at most 3 bytes early: same dword, so same page, as a byte that is needed) and the two
+// elements are shifted into place with v_alignbyte_b32 where they are used.  The window may end up to 6 bytes past
+// the second element; the caller guarantees those bytes are inside the allocation.
+template <class T> struct PairWindow {
+    static_assert(sizeof(T) == sizeof(base_t<T>) * cn_v<T>, "elements are packed channel arrays");
+    static constexpr int kBytes = 2 * int(sizeof(T));
+    static constexpr bool kShift = sizeof(T) % 4 != 0;
+    static constexpr int kOut = (kBytes + 3) / 4;                          // dwords holding the aligned pair
+    static constexpr int kWords = kShift ? (kBytes + 3 + 3) / 4 : kOut;    // dwords fetched
+    static constexpr bool kSupported = kWords <= 4;
+    u32 w[kWords];
+    u32 shift;      // bytes between the window start and the first element
+};
+template <class T> FKD_DEV PairWindow<T> load_pair_window(const char* row, u32 off) {
+    using PW = PairWindow<T>;
+    PW p;
+    const char* base = row;
+    if constexpr (PW::kShift) {
+        const u32 lo = u32(reinterpret_cast<uintptr_t>(row)) & 3u;     // wave uniform
+        base = row - lo;
+        off += lo;
+        p.shift = off & 3u;
+        off &= ~3u;
+    } else {
+        p.shift = 0;
+    }
+    asm volatile("" : "+v"(off));
+    const char* a = base + off;
+    constexpr int W = PW::kWords;
+    if constexpr (W == 1) { p.w[0] = *gconst<u32_a1>(a); }
+    else if constexpr (W == 2) { const u32x2_t v = *gconst<u32x2_a4>(a); p.w[0] = v.x; p.w[1] = v.y; }
+    else if constexpr (W == 3) { const u32x3_t v = *gconst<u32x3_a4>(a); p.w[0] = v.x; p.w[1] = v.y; p.w[2] = v.z; }
+    else { const u32x4_t v = *gconst<u32x4_a4>(a); p.w[0] = v.x; p.w[1] = v.y; p.w[2] = v.z; p.w[3] = v.w; }
+    return p;
+}
+template <class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& first, T& second) {
+    using PW = PairWindow<T>;
+    u32 v[PW::kOut];
+#pragma unroll
+    for (int i = 0; i < PW::kOut; ++i) {
+        if constexpr (PW::kShift) v[i] = __builtin_amdgcn_alignbyte(p.w[i + 1 < PW::kWords ? i + 1 : i], p.w[i], p.shift);
+        else v[i] = p.w[i];
+        if constexpr (sizeof(base_t<T>) < 4) asm("" : "+v"(v[i]));   // keep dwords whole: v_cvt_f32_ubyteN / v_bfe
+    }
+    first = unpack_one<0, T>(v);
+    second = unpack_one<1, T>(v);
+}
+
 // Store counterpart of load_bits_at: element sizes 2 and multiples of 4 (up to 16) leave as one access.
 template <class T> FKD_DEV void store_elem_at(char* base, u32 off, const T& v) {
     constexpr int n = int(sizeof(T));
@@ -631,12 +682,16 @@ template <class T> struct Read2D {
     using Raw = T;
     FKD_DEV static T finish(const Raw& r, const Params&) { return r; }
     // Tap cursor for gathers: the address of element (x0, y), wave uniform when y is; tap_load adds a 32-bit byte
-    // offset and returns the element's raw bits, tap_value takes them apart where they are used.  `last` marks the last row of the image, the only row in which reading a few bytes past an element
-    // could leave the allocation; kTapOverread says whether tap_load<true> reads past elements at all.
-    static constexpr bool kTapOverread = detail::overread_bytes<T, 1>() > 0 || detail::overread_bytes<T, 2>() > 0;
+    // offset and returns the element's raw bits, tap_value takes them apart where they are used.  `last` marks
+    // rows so close to the end of the image that reading a few bytes past an element could leave the allocation
+    // (the last row, for any image wider than two pixels); kTapOverread says whether tap_load<true> or pair_load
+    // read past elements at all.
+    static constexpr bool kTapOverread = detail::overread_bytes<T, 1>() > 0 || detail::PairWindow<T>::kShift;
     struct TapRow { const char* p; bool last; };
     FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) {
-        return TapRow{reinterpret_cast<const char*>(detail::row_ptr(p.data, p.pitch, x0, y)), y >= int(p.height) - 1};
+        // bytes of the image after this row's start that an over-reading access could lean on
+        const bool last = size_t(int(p.height) - 1 - y) * p.pitch < 8;
+        return TapRow{reinterpret_cast<const char*>(detail::row_ptr(p.data, p.pitch, x0, y)), last};
     }
     FKD_DEV static bool tap_last(const TapRow& r) { return r.last; }
     using TapBits = detail::RunBits<T, 1>;
@@ -644,13 +699,15 @@ template <class T> struct Read2D {
         return detail::load_bits_at<T, 1, OVER>(r.p, u32(x) * u32(sizeof(T)));
     }
     FKD_DEV static Raw tap_value(const TapBits& b) { return detail::run_value<0>(b); }
-    // Elements x and x+1 in one access (both must exist); may read up to 3 bytes past them like tap_load<true>.
-    static constexpr bool kTapPair = 2 * sizeof(T) <= 16;
-    using PairBits = detail::RunBits<T, 2>;
+    // Elements x and x+1 in one access (both must exist); may read up to 6 bytes past them.
+    static constexpr bool kTapPair = detail::PairWindow<T>::kSupported;
+    using PairBits = detail::PairWindow<T>;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params&) {
-        return detail::load_bits_at<T, 2, true>(r.p, u32(x) * u32(sizeof(T)));
+        return detail::load_pair_window<T>(r.p, u32(x) * u32(sizeof(T)));
     }
-    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow&, int) { return detail::run_value<K>(b); }
+    FKD_DEV static void pair_values(const PairBits& b, const TapRow&, int, Raw& first, Raw& second) {
+        detail::pair_window_values<T>(b, first, second);
+    }
 #endif
 };
 
@@ -742,19 +799,14 @@ struct ReadNV12 {
         b.uv = *detail::gconst<detail::u32_a1>(r.chroma + xc);
         return b;
     }
-    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) {
-        Out o;
-        if constexpr (K == 0) {
-            o.x = u8(b.y & 0xffu);
-            o.y = u8(b.uv & 0xffu);
-            o.z = u8((b.uv >> 8) & 0xffu);
-        } else {
-            const u32 uv = b.uv >> ((u32(r.x0 + x) & 1u) * 16u);
-            o.x = u8((b.y >> 8) & 0xffu);
-            o.y = u8(uv & 0xffu);
-            o.z = u8((uv >> 8) & 0xffu);
-        }
-        return o;
+    FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) {
+        first.x = u8(b.y & 0xffu);
+        first.y = u8(b.uv & 0xffu);
+        first.z = u8((b.uv >> 8) & 0xffu);
+        const u32 uv = b.uv >> ((u32(r.x0 + x) & 1u) * 16u);
+        second.x = u8((b.y >> 8) & 0xffu);
+        second.y = u8(uv & 0xffu);
+        second.z = u8((uv >> 8) & 0xffu);
     }
 #endif
 };
@@ -788,7 +840,7 @@ template <class Back> struct Crop {
     static constexpr bool kTapPair = Back::kTapPair;
     using PairBits = typename Back::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
-    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) { return Back::template pair_value<K>(b, r, x); }
+    FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
 #endif
 };
 
@@ -826,7 +878,7 @@ template <class Back, class... Ops> struct FusedRead {
     static constexpr bool kTapPair = Back::kTapPair;
     using PairBits = typename Back::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
-    template <int K> FKD_DEV static Raw pair_value(const PairBits& b, const TapRow& r, int x) { return Back::template pair_value<K>(b, r, x); }
+    FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
 #endif
 };
 
