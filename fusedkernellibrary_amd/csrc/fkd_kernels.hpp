@@ -69,25 +69,39 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
     if (x0 + V <= aw) {
         // All loads first, unconditionally (rows past the end re-read the last row, which is in bounds), so every
         // lane has ROWS independent wide loads in flight before the first use; only the stores are predicated.
-        Slot<typename R::Out> in[ROWS][V];
+        Slot<typename R::Out> in[ROWS * V];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
             const int y = ybase + r < ah ? ybase + r : ah - 1;
-            R::template exec_row<V, ALIGNED>(x0, y, z, p.read, in[r]);
+            Slot<typename R::Out> row[V];
+            R::template exec_row<V, ALIGNED>(x0, y, z, p.read, row);
+#pragma unroll
+            for (int i = 0; i < V; ++i) in[r * V + i].v = row[i].v;
         }
+        // all ROWS*V elements go through the chain together, operation by operation
+        Slot<typename Chain::Value> out[ROWS * V];
+        if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<ROWS * V>(in, out, (const FKD_CONSTANT void*)__builtin_amdgcn_kernarg_segment_ptr());
+        else Chain::template compute_run<ROWS * V>(in, out, p.ops);
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
             const int y = ybase + r;
-            Slot<typename Chain::Value> out[V];
+            Slot<typename Chain::Value> row[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) out[i].v = Chain::compute_checked(in[r][i].v, p);
-            if (y < ah) W::template exec_row<V, ALIGNED>(x0, y, z, out, p.write);
+            for (int i = 0; i < V; ++i) row[i].v = out[r * V + i].v;
+            if (y < ah) W::template exec_row<V, ALIGNED>(x0, y, z, row, p.write);
         }
     } else {
         for (int r = 0; r < ROWS; ++r) {
             const int y = ybase + r;
             if (y >= ah) break;
-            for (int x = x0; x < aw; ++x) W::exec(x, y, z, Chain::compute_checked(R::exec(x, y, z, p.read), p), p.write);
+            for (int x = x0; x < aw; ++x) {
+                Slot<typename R::Out> in[1];
+                Slot<typename Chain::Value> out[1];
+                in[0].v = R::exec(x, y, z, p.read);
+                if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<1>(in, out, (const FKD_CONSTANT void*)__builtin_amdgcn_kernarg_segment_ptr());
+                else Chain::template compute_run<1>(in, out, p.ops);
+                W::exec(x, y, z, out[0].v, p.write);
+            }
         }
     }
 }

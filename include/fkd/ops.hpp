@@ -642,6 +642,85 @@ FKD_DEV auto fold_quick(const V& v, const Tup<typename Op::Params, typename Rest
     if constexpr (sizeof...(Rest) == 0) return step();
     else return fold_quick<Rest...>(step(), p.tail, ok);
 }
+
+// The fold over a run of N elements, operation by operation: every element goes through operation k before any
+// goes through operation k+1.  A long chain then needs each operation's parameters (scalar registers) only once and
+// only briefly, instead of all parameters of the chain at the same time for every element.
+template <bool QUICK, int N, class V> FKD_DEV void fold_run(const Slot<V> (&in)[N], Slot<V> (&out)[N], const Tup<>&, bool&) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i].v = in[i].v;
+}
+template <bool QUICK, class Op, class... Rest, int N, class V, class O>
+FKD_DEV void fold_run(const Slot<V> (&in)[N], Slot<O> (&out)[N], const Tup<typename Op::Params, typename Rest::Params...>& p, bool& ok) {
+    static_assert(__is_same(V, typename Op::In), "operation input type does not match the value it receives");
+    auto step = [&](const V& v) {
+        if constexpr (QUICK && has_quick<Op>()) return Op::exec_quick(v, p.head, ok); else return Op::exec(v, p.head);
+    };
+    if constexpr (sizeof...(Rest) == 0) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) out[i].v = step(in[i].v);
+    } else {
+        Slot<typename Op::Out> mid[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) mid[i].v = step(in[i].v);
+        fold_run<QUICK, Rest...>(mid, out, p.tail, ok);
+    }
+}
+
+// fold_run for long chains, reading the parameters from the kernel-argument segment where they are used.  Left to
+// itself the compiler fetches every kernel argument at the top of the kernel; a chain of 100 operations then holds
+// 100+ scalar registers at once and spills them into vector-register lanes (one v_readlane per use).  Here the
+// pointer into the segment is made opaque every kGroup operations, so only one group's parameters are live.
+#define FKD_CONSTANT __attribute__((address_space(4)))
+constexpr int kParamGroup = 16;
+template <class B> FKD_DEV void pin_base(B& b) {
+    if constexpr (sizeof(B) == 4) { asm volatile("" : "+v"(b)); }
+    else if constexpr (sizeof(B) < 4) { u32 w = detail::to_bits(b); asm volatile("" : "+v"(w)); b = __builtin_bit_cast(B, decltype(detail::to_bits(b))(w)); }
+    else { unsigned long long w = __builtin_bit_cast(unsigned long long, b); asm volatile("" : "+v"(w)); b = __builtin_bit_cast(B, w); }
+}
+template <class V> FKD_DEV void pin_value(V& v) {
+    pin_base(chan<0>(v));
+    if constexpr (cn_v<V> > 1) pin_base(chan<1>(v));
+    if constexpr (cn_v<V> > 2) pin_base(chan<2>(v));
+    if constexpr (cn_v<V> > 3) pin_base(chan<3>(v));
+}
+template <bool QUICK, int IDX, int N, class V> FKD_DEV void fold_run_k(const Slot<V> (&in)[N], Slot<V> (&out)[N], const FKD_CONSTANT Tup<>*, bool&) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i].v = in[i].v;
+}
+template <bool QUICK, int IDX, class Op, class... Rest, int N, class V, class O>
+FKD_DEV void fold_run_k(const Slot<V> (&in)[N], Slot<O> (&out)[N],
+                        const FKD_CONSTANT Tup<typename Op::Params, typename Rest::Params...>* pk, bool& ok) {
+    static_assert(__is_same(V, typename Op::In), "operation input type does not match the value it receives");
+    if constexpr (IDX % kParamGroup == 0) {
+        // Every element finishes the previous group before the next group's parameters are touched: the values
+        // pass through ordered opaque points, and so does the parameter pointer, which is then declared wave
+        // uniform again so the reads stay scalar loads.
+        if constexpr (IDX > 0) {
+#pragma unroll
+            for (int i = 0; i < N; ++i) pin_value(const_cast<Slot<V>&>(in[i]).v);
+        }
+        unsigned long long a = reinterpret_cast<unsigned long long>(pk);
+        asm volatile("" : "+s"(a));
+        const u32 lo = __builtin_amdgcn_readfirstlane(u32(a)), hi = __builtin_amdgcn_readfirstlane(u32(a >> 32));
+        pk = reinterpret_cast<decltype(pk)>((unsigned long long)lo | ((unsigned long long)hi << 32));
+    }
+    typename Op::Params head;
+    if constexpr (!__is_empty(typename Op::Params))
+        __builtin_memcpy(&head, __builtin_assume_aligned((const void*)&pk->head, 4), sizeof(head));   // dword aligned: scalar loads
+    auto step = [&](const V& v) {
+        if constexpr (QUICK && has_quick<Op>()) return Op::exec_quick(v, head, ok); else return Op::exec(v, head);
+    };
+    if constexpr (sizeof...(Rest) == 0) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) out[i].v = step(in[i].v);
+    } else {
+        Slot<typename Op::Out> mid[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) mid[i].v = step(in[i].v);
+        fold_run_k<QUICK, IDX + 1, Rest...>(mid, out, &pk->tail, ok);
+    }
+}
 #endif
 
 // A run of compute operations packaged as one (host side: FusedOperation of compute IOps).
@@ -1216,6 +1295,26 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     static constexpr bool kQuick = any_quick<Ops...>();
     using OpParams = Tup<typename Ops::Params...>;
     FKD_DEV static Value compute_checked(const typename R::Out& v, const Params& p) { return compute_checked_ops(v, p.ops); }
+    // N elements at once, operation-major (see fold_run); same results as compute() element by element.
+    template <int N> FKD_DEV static void compute_run(const Slot<typename R::Out> (&in)[N], Slot<Value> (&out)[N], const OpParams& ops) {
+        bool ok = true;
+        fold_run<kQuick, Ops...>(in, out, ops, ok);
+        if constexpr (kQuick) {
+            if (__builtin_expect(!ok, 0)) fold_run<false, Ops...>(in, out, ops, ok);
+        }
+    }
+    // The same for chains with many parameters; `kernarg` is the kernel-argument segment, holding a Params at offset 0.
+    static constexpr bool kLongChain = sizeof(Tup<typename Ops::Params...>) > 128;
+    template <int N> FKD_DEV static void compute_run_kernarg(const Slot<typename R::Out> (&in)[N], Slot<Value> (&out)[N],
+                                                             const FKD_CONSTANT void* kernarg) {
+        const auto* ops = reinterpret_cast<const FKD_CONSTANT OpParams*>(
+            reinterpret_cast<const FKD_CONSTANT char*>(kernarg) + __builtin_offsetof(Params, ops));
+        bool ok = true;
+        fold_run_k<kQuick, 0, Ops...>(in, out, ops, ok);
+        if constexpr (kQuick) {
+            if (__builtin_expect(!ok, 0)) fold_run_k<false, 0, Ops...>(in, out, ops, ok);
+        }
+    }
     FKD_DEV static Value compute_checked_ops(const typename R::Out& v, const OpParams& ops) {
         if constexpr (sizeof...(Ops) == 0) {
             return v;
