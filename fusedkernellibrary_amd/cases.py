@@ -120,3 +120,21 @@ def div_f32x3(src, d, out):
 def saturate_f32_u8(src, out):
     """src (H,W) f32 cuda, out (H,W) u8 cuda: SaturateCast<float, uchar>."""
     _ok(cases().fklcase_saturate_f32_u8(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, _p(out), out.stride(0)))
+
+
+def crop_resize_default_norm_split(src, rects, dst, used, default, sub, div, out):
+    """Configuration-3 chain on 8 crops with BatchRead<CONDITIONAL_WITH_DEFAULT>: planes >= used yield `default`."""
+    assert len(rects) == 8
+    r, d, s, v = _host(rects, np.int32), _host(default, np.float32), _host(sub, np.float32), _host(div, np.float32)
+    _ok(cases().fklcase_crop_resize_default_norm_split_b8(
+        _stream(), _p(src), src.shape[1], src.shape[0], src.stride(0), r.ctypes.data_as(C.c_void_p), int(dst[0]), int(dst[1]),
+        int(used), d.ctypes.data_as(C.c_void_p), s.ctypes.data_as(C.c_void_p), v.ctypes.data_as(C.c_void_p), _p(out)))
+
+
+def batch_default_cast_mul(srcs, active, default, mul, out):
+    """4 (H,W,3) u8 cuda images, planes >= active yield `default` (3 bytes); out (4,H,W,3) f32 cuda."""
+    assert len(srcs) == 4
+    sp = (C.c_void_p * 4)(*[s.data_ptr() for s in srcs])
+    d, m = _host(default, np.uint8), _host(mul, np.float32)
+    _ok(cases().fklcase_batch_default_cast_mul_b4(_stream(), sp, srcs[0].shape[1], srcs[0].shape[0], srcs[0].stride(0), int(active),
+                                                  d.ctypes.data_as(C.c_void_p), m.ctypes.data_as(C.c_void_p), _p(out)))

@@ -45,6 +45,14 @@ template <int N, int AR, class Back> struct ResizeRoot<BatchRead<N, ResizeLinear
     using Resize = ResizeLinear<AR, Back>;
 };
 
+template <int N, int AR, class Back> struct ResizeRoot<BatchReadDefault<N, ResizeLinear<AR, Back>>> {
+    static constexpr bool value = true;
+    static constexpr bool batched = true;
+    using Resize = ResizeLinear<AR, Back>;
+};
+template <class R> struct HasDefaultPlanes { static constexpr bool value = false; };
+template <int N, class PlaneOp> struct HasDefaultPlanes<BatchReadDefault<N, PlaneOp>> { static constexpr bool value = true; };
+
 template <class Chain> constexpr bool is_gather_chain() {
     if constexpr (ResizeRoot<typename Chain::Read>::value)
         return ResizeRoot<typename Chain::Read>::Resize::BackOp::kTapCursor;
@@ -169,6 +177,23 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
     const int wy = __builtin_amdgcn_readfirstlane(int(threadIdx.y));
     const int y0 = int(tin / gg.tiles_x) * TH + wy * YI;
     if (y0 >= ah) return;
+    if constexpr (HasDefaultPlanes<typename Chain::Read>::value) {
+        // BatchRead<CONDITIONAL_WITH_DEFAULT>: planes at or beyond `used` read nothing; every element is the default
+        // value, which still goes through the chain's compute operations and the write.
+        if (z >= p.read.used) {
+            const typename RZ::Out def = p.read.def;
+            const typename Chain::Value r = Chain::compute_checked_ops(def, ops);
+            for (int y = y0; y < (y0 + YI < ah ? y0 + YI : ah); ++y) {
+                const typename WP::RowRef orow = WP::row(y, z, wpar);
+#pragma unroll
+                for (int i = 0; i < XI; ++i) {
+                    const int x = tx0 + int(threadIdx.x) + kGatherBX * i;
+                    if (x < aw) WP::put(orow, x, r);
+                }
+            }
+            return;
+        }
+    }
     int ox = 0, oy = 0;
     if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; }
     const int sw = Back::width(q.back), sh = Back::height(q.back);

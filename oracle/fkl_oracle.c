@@ -316,6 +316,31 @@ static int write_value(const fklo_write *w, int x, int y, int z, const fklo_val 
  * active threads of the (fused) read; BatchRead picks plane z (batch_operations.h:205-212) and
  * activeThreads = (max W, max H, BATCH) (batch_operations.h:401-424). Planes whose own geometry is smaller
  * than the maximum are rejected here: the reference runs them unchecked, which reads outside the crop. */
+/* BatchRead<CONDITIONAL_WITH_DEFAULT>::exec, FK/core/execution_model/operation_model/batch_operations.h:262-273:
+ * planes at or beyond usedPlanes return params.default_value, whose type is the plane operation's output type
+ * (float_<cn> after a resize, the tap type after fused tap operations, else the element type). */
+static void read_default(const fklo_read *r, fklo_val *out) {
+    int cn = r->kind == FKLO_READ_NV12 ? 3 : r->cn;
+    int elem = r->kind == FKLO_READ_NV12 ? FKLO_U8 : r->elem;
+    if (r->n_tap_ops > 0 || r->has_resize) {
+        /* find the type the read yields by running the tap operations on a dummy element */
+        fklo_val probe;
+        memset(&probe, 0, sizeof(probe));
+        probe.elem = elem;
+        probe.cn = cn;
+        for (int i = 0; i < r->n_tap_ops; ++i) apply_op(&r->tap_ops[i], &probe);
+        elem = r->has_resize ? FKLO_F32 : probe.elem;
+        cn = probe.cn;
+    }
+    memset(out, 0, sizeof(*out));
+    out->elem = elem;
+    out->cn = cn;
+    for (int c = 0; c < cn; ++c) {
+        if (elem == FKLO_F32) out->f[c] = r->def[c];
+        else out->u[c] = (uint8_t)r->def[c];
+    }
+}
+
 int fklo_execute(int32_t n_planes, const fklo_read *reads,
                  int32_t n_ops, const fklo_op *ops,
                  int32_t n_writes, const fklo_write *writes) {
@@ -342,7 +367,9 @@ int fklo_execute(int32_t n_planes, const fklo_read *reads,
         for (int y = 0; y < act_h; ++y) {
             for (int x = 0; x < act_w; ++x) {
                 fklo_val v;
-                int rc = r->has_resize ? read_resized(r, &rp, x, y, &v) : read_tap(r, x, y, &v);
+                int rc = FKLO_OK;
+                if (r->use_default) read_default(r, &v);
+                else rc = r->has_resize ? read_resized(r, &rp, x, y, &v) : read_tap(r, x, y, &v);
                 if (rc) return rc;
                 for (int i = 0; i < n_ops; ++i) {
                     if ((rc = apply_op(&ops[i], &v))) return rc;

@@ -82,6 +82,8 @@ typedef struct {
     float bg[4];             /* letterbox background (PRESERVE_AR) */
     int32_t n_tap_ops;       /* ops fused INTO the read: run on every source tap */
     const fklo_op *tap_ops;
+    int32_t use_default;     /* BatchRead<CONDITIONAL_WITH_DEFAULT>, plane index >= usedPlanes: every element of */
+    float def[4];            /* this plane is def, typed like the read's output, and nothing is read             */
 } fklo_read;
 
 typedef struct {

@@ -83,6 +83,45 @@ int crop_resize_norm_split(const uint8_t* src, int w, int h, int pitch, const in
     return 0;
 }
 
+// Horizontal fusion with fewer live planes than the compiled batch (BatchRead<CONDITIONAL_WITH_DEFAULT>): planes
+// >= used_planes produce default_value instead of reading.  Same chain as configuration 3 otherwise.
+template <size_t B>
+int crop_resize_default_norm_split(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                                   int used_planes, const float* def, const float* sub, const float* div, float* out) {
+    CpuStream stream;
+    const auto in = wrap2d<uchar3>(src, w, h, pitch);
+    Tensor<float> o(out, uint(dw), uint(dh), uint(B), 3, MemType::Host, 0);
+    const auto crops = rects_from<B>(rects);
+    std::array<Size, B> sizes{};
+    for (auto& s : sizes) s = Size(dw, dh);
+    executeOperations<CpuDPP>(stream,
+        PerThreadRead<ND::_2D, uchar3>::build(in.ptr())
+            .then(Crop<>::build(crops))
+            .then(Resize<InterpolationType::INTER_LINEAR>::build(used_planes, make_<float3>(def[0], def[1], def[2]), sizes)),
+        ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, float3, float3>::build(),
+        Sub<float3>::build(make_<float3>(sub[0], sub[1], sub[2])),
+        Div<float3>::build(make_<float3>(div[0], div[1], div[2])),
+        TensorSplit<float3>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
+// The executor overload for an array of images with active batch and default value:
+// executeOperations(std::array<Ptr2D<I>,B>, activeBatch, defaultValue, Tensor<O>, stream, ops...).
+template <size_t B>
+int batch_default_cast_mul(const uint8_t* const* srcs, int w, int h, int pitch, int active, const uint8_t* def,
+                           const float* mul, float* out) {
+    CpuStream stream;
+    std::array<Ptr2D<uchar3>, B> ins{};
+    for (size_t i = 0; i < B; ++i) ins[i] = wrap2d<uchar3>(srcs[i], w, h, pitch);
+    Tensor<float3> o(reinterpret_cast<float3*>(out), uint(w), uint(h), uint(B), 1, MemType::Host, 0);
+    executeOperations<CpuDPP>(ins, active, uchar3{def[0], def[1], def[2]}, o, stream,
+        Cast<uchar3, float3>::build(),
+        Mul<float3>::build(make_<float3>(mul[0], mul[1], mul[2])));
+    stream.sync();
+    return 0;
+}
+
 // Benchmark configuration 4: B independent uchar3 images, per-image Mul and Add fused into each plane's
 // read, SaturateCast, B separate outputs in one launch.
 template <size_t B>
@@ -166,6 +205,15 @@ int fklref_crop_resize_norm_split_b8(const uint8_t* src, int w, int h, int pitch
 int fklref_crop_resize_norm_split_b64(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw,
                                       int dh, const float* sub, const float* div, float* out) {
     return crop_resize_norm_split<64>(src, w, h, pitch, rects, dw, dh, sub, div, out);
+}
+
+int fklref_crop_resize_default_norm_split_b8(const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                                             int used_planes, const float* def, const float* sub, const float* div, float* out) {
+    return crop_resize_default_norm_split<8>(src, w, h, pitch, rects, dw, dh, used_planes, def, sub, div, out);
+}
+int fklref_batch_default_cast_mul_b4(const uint8_t* const* srcs, int w, int h, int pitch, int active, const uint8_t* def,
+                                     const float* mul, float* out) {
+    return batch_default_cast_mul<4>(srcs, w, h, pitch, active, def, mul, out);
 }
 
 int fklref_batch_muladd_sat_b4(const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,

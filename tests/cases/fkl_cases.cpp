@@ -212,6 +212,43 @@ int fklcase_copy_f32(void* stream_, const float* in, int w, int h, int pitch, fl
         for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(i, o, stream);
     });
 }
+// Horizontal fusion with fewer live planes than the compiled batch (BatchRead<CONDITIONAL_WITH_DEFAULT>).
+int fklcase_crop_resize_default_norm_split_b8(void* stream_, const uint8_t* src, int w, int h, int pitch, const int32_t* rects,
+                                              int dw, int dh, int used_planes, const float* def, const float* sub,
+                                              const float* div, float* out) {
+    return guarded([&] {
+        constexpr size_t B = 8;
+        Stream stream(stream_);
+        const auto in = dev2d<uchar3>(src, w, h, pitch);
+        Tensor<float> o(out, uint(dw), uint(dh), uint(B), 3, MemType::Device, 0);
+        const auto crops = rects_from<B>(rects);
+        std::array<Size, B> sizes{};
+        for (auto& s : sizes) s = Size(dw, dh);
+        for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
+            PerThreadRead<ND::_2D, uchar3>::build(in.ptr())
+                .then(Crop<>::build(crops))
+                .then(Resize<InterpolationType::INTER_LINEAR>::build(used_planes, make_<float3>(def[0], def[1], def[2]), sizes)),
+            ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, float3, float3>::build(),
+            Sub<float3>::build(make_<float3>(sub[0], sub[1], sub[2])),
+            Div<float3>::build(make_<float3>(div[0], div[1], div[2])),
+            TensorSplit<float3>::build(o.ptr()));
+    });
+}
+// executeOperations(std::array<Ptr2D<I>,B>, activeBatch, defaultValue, Tensor<O>, stream, ops...)
+int fklcase_batch_default_cast_mul_b4(void* stream_, const uint8_t* const* srcs, int w, int h, int pitch, int active,
+                                      const uint8_t* def, const float* mul, float* out) {
+    return guarded([&] {
+        constexpr size_t B = 4;
+        Stream stream(stream_);
+        std::array<Ptr2D<uchar3>, B> ins{};
+        for (size_t i = 0; i < B; ++i) ins[i] = dev2d<uchar3>(srcs[i], w, h, pitch);
+        Tensor<float3> o(reinterpret_cast<float3*>(out), uint(w), uint(h), uint(B), 1, MemType::Device, 0);
+        executeOperations<TransformDPP<>>(ins, active, uchar3{def[0], def[1], def[2]}, o, stream,
+            Cast<uchar3, float3>::build(),
+            Mul<float3>::build(make_<float3>(mul[0], mul[1], mul[2])));
+    });
+}
+
 // Single-operation chains for the exhaustive numeric tests.
 int fklcase_div_f32(void* stream_, const float* in, int w, int h, int pitch, float d, float* out, int out_pitch) {
     return guarded([&] {

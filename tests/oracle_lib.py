@@ -34,6 +34,7 @@ class Read(C.Structure):
         ("has_resize", C.c_int32), ("dst_w", C.c_int32), ("dst_h", C.c_int32),
         ("ar", C.c_int32), ("bg", C.c_float * 4),
         ("n_tap_ops", C.c_int32), ("tap_ops", C.POINTER(Op)),
+        ("use_default", C.c_int32), ("def_", C.c_float * 4),
     ]
 
 
@@ -222,6 +223,38 @@ def oracle_crop_resize_norm_split(src, rects, dst, sub, div):
     return out
 
 
+def _defaulted(r: Read, default) -> Read:
+    r.use_default = 1
+    for i, v in enumerate(default):
+        r.def_[i] = float(v)
+    return r
+
+
+def oracle_crop_resize_default_norm_split(src, rects, dst, used, default, sub, div):
+    """Configuration-3 chain with BatchRead<CONDITIONAL_WITH_DEFAULT>: planes >= used yield `default` (float3)."""
+    dw, dh = dst
+    b = len(rects)
+    out = np.zeros((b, 3, dh, dw), np.float32)
+    reads = [read_2d(src, 3, crop=rects[i], resize=dst, ar=IGNORE_AR) for i in range(b)]
+    for i in range(used, b):
+        _defaulted(reads[i], default)
+    execute(reads, [op(REORDER, idx=(2, 1, 0, 0)), op(SUB, sub), op(DIV, div)],
+            [write(TENSOR_SPLIT, out, 3, dw, dh, b, 3)])
+    return out
+
+
+def oracle_batch_default_cast_mul(srcs, active, default, mul):
+    """B uchar3 images, planes >= active yield `default` (uchar3); Cast to float3, Mul; Tensor<float3> B x H x W x 3."""
+    b = len(srcs)
+    h, w = srcs[0].shape[:2]
+    out = np.zeros((b, h, w, 3), np.float32)
+    reads = [read_2d(srcs[i], 3) for i in range(b)]
+    for i in range(active, b):
+        _defaulted(reads[i], default)
+    execute(reads, [op(CAST_F32), op(MUL, mul)], [write(TENSOR_WRITE, out, 3, w, h, b, 1)])
+    return out
+
+
 def oracle_batch_muladd_sat(srcs, mul, add):
     b = len(srcs)
     h, w = srcs[0].shape[:2]
@@ -284,6 +317,29 @@ def ref_crop_resize_norm_split(src, rects, dst, sub, div):
     out = np.zeros((b, 3, dh, dw), np.float32)
     rc = getattr(ref(), fn)(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], _i32p(rects), dw, dh,
                             _f32p(sub), _f32p(div), C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
+def ref_crop_resize_default_norm_split(src, rects, dst, used, default, sub, div):
+    assert len(rects) == 8
+    dw, dh = dst
+    out = np.zeros((8, 3, dh, dw), np.float32)
+    rc = ref().fklref_crop_resize_default_norm_split_b8(
+        C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], _i32p(rects), dw, dh, int(used),
+        _f32p(default), _f32p(sub), _f32p(div), C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
+def ref_batch_default_cast_mul(srcs, active, default, mul):
+    assert len(srcs) == 4
+    h, w = srcs[0].shape[:2]
+    out = np.zeros((4, h, w, 3), np.float32)
+    sp = (C.c_void_p * 4)(*[_ptr(s) for s in srcs])
+    d = np.ascontiguousarray(default, np.uint8)
+    rc = ref().fklref_batch_default_cast_mul_b4(sp, w, h, srcs[0].strides[0], int(active), C.c_void_p(_ptr(d)), _f32p(mul),
+                                                C.c_void_p(_ptr(out)))
     assert rc == 0
     return out
 

@@ -309,3 +309,33 @@ def test_divergent_plane_sizes_are_rejected():
     with pytest.raises(RuntimeError):
         ol.execute([ol.read_2d(src, 3, crop=(0, 0, 8, 8)), ol.read_2d(src, 3, crop=(0, 0, 6, 8))], [],
                    [ol.write(ol.TENSOR_WRITE, out, 3, 8, 8, 2, 1)])
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="reference CPU backend not built (needs the reference tree)")
+def test_default_planes_match_reference_backend():
+    """BatchRead<CONDITIONAL_WITH_DEFAULT> (batch_operations.h:221-281): planes >= usedPlanes yield the default value."""
+    rng = np.random.RandomState(3)
+    src = rng.randint(0, 256, (120, 200, 3)).astype(np.uint8)
+    rects = np.array([[0, 0, 50, 40], [10, 10, 100, 80], [150, 80, 50, 40], [5, 5, 20, 100], [0, 0, 200, 120], [100, 60, 3, 2],
+                      [20, 30, 64, 64], [1, 2, 77, 33]], np.int32)
+    mean, std = (123.675, 116.28, 103.53), (58.395, 57.12, 57.375)
+    for used in (0, 3, 8):
+        a = ol.oracle_crop_resize_default_norm_split(src, rects, (32, 24), used, (1.5, -2.0, 300.0), mean, std)
+        b = ol.ref_crop_resize_default_norm_split(src, rects, (32, 24), used, (1.5, -2.0, 300.0), mean, std)
+        assert a.tobytes() == b.tobytes()
+    srcs = [rng.randint(0, 256, (30, 41, 3)).astype(np.uint8) for _ in range(4)]
+    for active in (0, 2, 4):
+        a = ol.oracle_batch_default_cast_mul(srcs, active, (7, 200, 33), (0.5, 2.0, 1.25))
+        b = ol.ref_batch_default_cast_mul(srcs, active, (7, 200, 33), (0.5, 2.0, 1.25))
+        assert a.tobytes() == b.tobytes()
+
+
+def test_default_planes_closed_form():
+    """A default plane holds compute(default) everywhere, whatever the source: checked without the reference."""
+    src = np.full((40, 50, 3), 9, np.uint8)
+    rects = np.array([[0, 0, 10, 10]] * 8, np.int32)
+    out = ol.oracle_crop_resize_default_norm_split(src, rects, (6, 5), 2, (10.0, 20.0, 40.0), (1.0, 2.0, 3.0), (2.0, 4.0, 8.0))
+    # BGR->RGB swaps the default too: (40, 20, 10), then (x - sub) / div
+    assert np.all(out[2:, 0] == np.float32((40.0 - 1.0) / 2.0)) and np.all(out[2:, 1] == np.float32((20.0 - 2.0) / 4.0))
+    assert np.all(out[2:, 2] == np.float32((10.0 - 3.0) / 8.0))
+    assert np.all(out[:2, 0] == np.float32((9.0 - 1.0) / 2.0))
