@@ -138,3 +138,22 @@ def batch_default_cast_mul(srcs, active, default, mul, out):
     d, m = _host(default, np.uint8), _host(mul, np.float32)
     _ok(cases().fklcase_batch_default_cast_mul_b4(_stream(), sp, srcs[0].shape[1], srcs[0].shape[0], srcs[0].stride(0), int(active),
                                                   d.ctypes.data_as(C.c_void_p), m.ctypes.data_as(C.c_void_p), _p(out)))
+
+
+def set_and_loop_f32(n, init, add, iterations):
+    """setTo(init) on a library-owned 1-D float array, StaticLoop<Add<float>, iterations>(add), download: (n,) f32."""
+    out = np.empty(n, np.float32)
+    _ok(cases().fklcase_set_and_loop_f32(_stream(), int(n), C.c_float(float(init)), C.c_float(float(add)), int(iterations),
+                                         out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+def set_to_shapes(w, h, planes, v3, vf):
+    """setTo on a pitched (h,w) uchar3 image and a (planes,h,w) float tensor; returns (image rows incl. pitch, pitch, tensor)."""
+    img = np.zeros(h * (w * 3 + 1024), np.uint8)
+    pitch = C.c_int(0)
+    ten = np.empty((planes, h, w), np.float32)
+    v = _host(v3, np.uint8)
+    _ok(cases().fklcase_set_to_shapes(_stream(), int(w), int(h), int(planes), v.ctypes.data_as(C.c_void_p), C.c_float(float(vf)),
+                                      img.ctypes.data_as(C.c_void_p), C.byref(pitch), ten.ctypes.data_as(C.c_void_p)))
+    return img[: pitch.value * h].reshape(h, pitch.value), pitch.value, ten

@@ -507,6 +507,21 @@ template <class I, class P, class O> struct Div {
 #endif
 };
 
+// StaticLoop<Operation, ITERATIONS>: Operation applied ITERATIONS times with the same parameters.
+// FK/algorithms/basic_ops/static_loop.h:21-44.
+template <class Op, int N> struct StaticLoop {
+    using In = typename Op::In; using Out = typename Op::Out;
+    using Params = typename Op::Params;
+    static_assert(N >= 1 && __is_same(In, Out), "the looped operation maps a type onto itself");
+    FKD_NAME("StaticLoop<" + Op::name() + "," + istr(N) + ">")
+    FKD_DEV static Out exec(const In& a, const Params& p) {
+        Out v = Op::exec(a, p);
+#pragma unroll
+        for (int i = 1; i < N; ++i) v = Op::exec(v, p);
+        return v;
+    }
+};
+
 // Cast<I,O>: per-channel static_cast.  FK/algorithms/basic_ops/cast.h:22-33.
 template <class I, class O> struct Cast {
     using In = I; using Out = O; using Params = Empty;

@@ -4,5 +4,6 @@
 #include <fused_kernel/algorithms/basic_ops/cast.h>
 #include <fused_kernel/algorithms/basic_ops/memory_operations.h>
 #include <fused_kernel/algorithms/basic_ops/set.h>
+#include <fused_kernel/algorithms/basic_ops/static_loop.h>
 #include <fused_kernel/algorithms/basic_ops/vector_ops.h>
 #endif

@@ -2,6 +2,7 @@
 // Interface counterpart: FK/algorithms/basic_ops/set.h:29-80.
 #ifndef FK_AMD_SET_H
 #define FK_AMD_SET_H
+#include <fused_kernel/core/data/ptr_nd.h>
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
 namespace fk {
 template <typename T> struct ReadSetParams {
@@ -19,6 +20,12 @@ template <typename T> struct ReadSet : ReadOperation<T, ReadSetParams<T>, T, TF:
     static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) { return opData.params.size; }
     using Parent::build;
     static constexpr InstantiableType build(const T& value, const ActiveThreads& activeThreads) { return {{{value, activeThreads}}}; }
+    template <ND D> static constexpr InstantiableType build(const T& value, const PtrDims<D>& dims) {
+        static_assert(D == ND::_1D || D == ND::_2D || D == ND::_3D || D == ND::T3D, "Unsupported ND type for ReadSet build.");
+        if constexpr (D == ND::_1D) return build(value, ActiveThreads(dims.width, 1, 1));
+        else if constexpr (D == ND::_2D) return build(value, ActiveThreads(dims.width, dims.height, 1));
+        else return build(value, ActiveThreads(dims.width, dims.height, dims.planes));
+    }
 };
 namespace amd {
 template <typename T> struct Lower<ReadSet<T>> {

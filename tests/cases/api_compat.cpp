@@ -146,3 +146,26 @@ void batch_and_video() {
                                       TensorSplit<float3>::build(planar));
     stream.sync();
 }
+
+// ---- setTo, StaticLoop and the activeBatch/defaultValue overloads, as the reference's benchmarks spell them ------
+// (benchmarks/numinstructions/benchmark_numinstructions_x_operation.h:40-75, executors.h:80-100)
+#include <fused_kernel/algorithms/basic_ops/static_loop.h>
+#include <fused_kernel/core/data/ptr_utils.h>
+constexpr auto singleOp = fk::Add<float>::build(1.f);
+constexpr auto allInstr = fk::StaticLoop<typename decltype(singleOp)::Operation, 50>::build(1.f);
+static_assert(std::is_same_v<std::decay_t<decltype(allInstr)>, fk::Binary<fk::StaticLoop<fk::Add<float>, 50>>>);
+void set_loop_and_conditional_batch() {
+    using namespace fk;
+    Stream stream;
+    Ptr1D<float> in(1024), out(1024);
+    setTo(1.f, in, stream);
+    setTo(0.f, out, stream);
+    executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_1D, float>::build(in), allInstr,
+                                      PerThreadWrite<ND::_1D, float>::build(out));
+    Ptr2D<uchar> img(60, 120);
+    setTo(uchar(10), img, stream);
+    std::array<Ptr2D<uchar3>, 4> ins{Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32), Ptr2D<uchar3>(64, 32)};
+    Tensor<float3> t(64, 32, 4);
+    executeOperations<TransformDPP<>>(ins, 2, uchar3{1, 2, 3}, t, stream, Cast<uchar3, float3>::build());
+    stream.sync();
+}

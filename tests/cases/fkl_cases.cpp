@@ -7,6 +7,8 @@
 #include <fused_kernel/algorithms/basic_ops/memory_operations.h>
 #include <fused_kernel/algorithms/basic_ops/arithmetic.h>
 #include <fused_kernel/algorithms/basic_ops/cast.h>
+#include <fused_kernel/algorithms/basic_ops/static_loop.h>
+#include <fused_kernel/core/data/ptr_utils.h>
 #include <fused_kernel/algorithms/image_processing/crop.h>
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
@@ -146,6 +148,21 @@ void crop_swap_u8(void* stream_, const uint8_t* src, int w, int h, int pitch, co
 
 } // namespace
 
+// setTo + StaticLoop, spelled like the reference's instruction-count benchmark
+// (benchmarks/numinstructions/benchmark_numinstructions_x_operation.h:40-75): library-owned 1-D device arrays are
+// filled with setTo, run through StaticLoop<Add<float>, N> and downloaded into `host_out`.
+template <int N> void set_and_loop(Stream& stream, int n, float init, float add, float* host_out) {
+    Ptr1D<float> in(uint(n), 0, MemType::DeviceAndPinned), out(uint(n), 0, MemType::DeviceAndPinned);
+    setTo(init, in, stream);
+    setTo(0.f, out, stream);
+    constexpr auto singleOp = Add<float>::build(1.f);
+    const auto loop = StaticLoop<typename decltype(singleOp)::Operation, N>::build(add);
+    executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_1D, float>::build(in), loop, PerThreadWrite<ND::_1D, float>::build(out));
+    out.download(stream);
+    stream.sync();
+    std::memcpy(host_out, out.ptrPinned().data, size_t(n) * sizeof(float));
+}
+
 extern "C" {
 
 const char* fklcase_last_error(void) { return g_error; }
@@ -246,6 +263,36 @@ int fklcase_batch_default_cast_mul_b4(void* stream_, const uint8_t* const* srcs,
         executeOperations<TransformDPP<>>(ins, active, uchar3{def[0], def[1], def[2]}, o, stream,
             Cast<uchar3, float3>::build(),
             Mul<float3>::build(make_<float3>(mul[0], mul[1], mul[2])));
+    });
+}
+
+int fklcase_set_and_loop_f32(void* stream_, int n, float init, float add, int iterations, float* host_out) {
+    return guarded([&] {
+        Stream stream(stream_);
+        switch (iterations) {
+        case 1: set_and_loop<1>(stream, n, init, add, host_out); break;
+        case 6: set_and_loop<6>(stream, n, init, add, host_out); break;
+        case 50: set_and_loop<50>(stream, n, init, add, host_out); break;
+        default: throw std::runtime_error("fklcase_set_and_loop_f32: iterations must be 1, 6 or 50");
+        }
+    });
+}
+// setTo on a pitched 2-D uchar3 image and on a float tensor; results downloaded into host buffers.
+int fklcase_set_to_shapes(void* stream_, int w, int h, int planes, const uint8_t* v3, float vf, uint8_t* host_img, int* host_pitch,
+                          float* host_tensor) {
+    return guarded([&] {
+        Stream stream(stream_);
+        Ptr2D<uchar3> img(uint(w), uint(h), 0, MemType::DeviceAndPinned);
+        Tensor<float> t(uint(w), uint(h), uint(planes), 1, MemType::DeviceAndPinned);
+        setTo(uchar3{v3[0], v3[1], v3[2]}, img, stream);
+        setTo(vf, t, stream);
+        img.download(stream);
+        t.download(stream);
+        stream.sync();
+        const auto mirror = img.ptrPinned();    // tightly packed, unlike the pitched device image
+        *host_pitch = int(mirror.dims.pitch);
+        std::memcpy(host_img, mirror.data, size_t(mirror.dims.pitch) * size_t(h));
+        std::memcpy(host_tensor, t.ptrPinned().data, size_t(w) * size_t(h) * size_t(planes) * sizeof(float));
     });
 }
 
