@@ -157,3 +157,21 @@ def set_to_shapes(w, h, planes, v3, vf):
     _ok(cases().fklcase_set_to_shapes(_stream(), int(w), int(h), int(planes), v.ctypes.data_as(C.c_void_p), C.c_float(float(vf)),
                                       img.ctypes.data_as(C.c_void_p), C.byref(pitch), ten.ctypes.data_as(C.c_void_p)))
     return img[: pitch.value * h].reshape(h, pitch.value), pitch.value, ten
+
+
+def uncompiled_pointwise_f32(src, out):
+    """(H,W) f32 cuda: ((x*1.5 - 0.25) / 3) + 7 -- a chain that is not in the ahead-of-time list."""
+    _ok(cases().fklcase_uncompiled_pointwise_f32(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, _p(out), out.stride(0) * 4))
+
+
+def uncompiled_gray_resize(src, rect, dst, mul, out):
+    """(H,W) u8 cuda -> crop -> bilinear (dst = (w,h)) -> * mul -> out (dh,dw) f32 cuda."""
+    r = _host(rect, np.int32)
+    _ok(cases().fklcase_uncompiled_gray_resize(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0), r.ctypes.data_as(C.c_void_p),
+                                               int(dst[0]), int(dst[1]), C.c_float(float(mul)), _p(out), out.stride(0) * 4))
+
+
+def uncompiled_float4_resize(src, dst, out):
+    """(H,W,4) f32 cuda -> bilinear -> out (dh,dw,4) f32 cuda."""
+    _ok(cases().fklcase_uncompiled_float4_resize(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, int(dst[0]), int(dst[1]),
+                                                 _p(out), out.stride(0) * 4))

@@ -3,7 +3,7 @@
 #pragma once
 
 #define FKD_DEVICE_CODE 1
-#include "fkd_kernels.hpp"
+#include "fkd_launch.hpp"
 #include "registry.hpp"
 #include <fklhip.h>
 
@@ -12,7 +12,7 @@
 
 namespace fklhip {
 
-template <class Chain> int aot_launch(const void* blob, size_t bytes, void* stream, fkd::LaunchInfo* info) {
+template <class Chain> int aot_launch(const void*, const void* blob, size_t bytes, void* stream, fkd::LaunchInfo* info) {
     using Params = typename Chain::Params;
     if (!blob) return FKLHIP_EINVAL;
     if (bytes != sizeof(Params)) return FKLHIP_EBLOB_SIZE;

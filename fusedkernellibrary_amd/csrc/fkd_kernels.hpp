@@ -22,14 +22,16 @@
 // launch geometry FK/core/execution_model/executors.h:242-351.
 #pragma once
 
-#include <hip/hip_runtime.h>
-
-#include <type_traits>
+#if !defined(__HIPCC_RTC__)
+#include <hip/hip_runtime.h>   // the run-time compiler provides the HIP device API without any header
+#endif
 
 #include <fkd/launch_info.hpp>
 #include <fkd/ops.hpp>
 
 namespace fkd {
+
+template <int I> struct IntTag { static constexpr int value = I; };
 
 // ---- chain classification ---------------------------------------------------------------------------
 
@@ -66,7 +68,7 @@ constexpr int kRowsBX = 64;   // lanes along x: one wave per row segment
 constexpr int kRowsBY = 4;    // waves per workgroup
 
 template <class Chain, int V, int ROWS, bool ALIGNED>
-__global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain::Params p) {
+__device__ __forceinline__ void rows_body(const typename Chain::Params& p) {
     using R = typename Chain::Read;
     using W = typename Chain::Write;
     const int z = blockIdx.z;
@@ -114,6 +116,30 @@ __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain
     }
 }
 
+template <class Chain, int V, int ROWS, bool ALIGNED>
+__global__ __launch_bounds__(kRowsBX * kRowsBY) void k_rows(const typename Chain::Params p) {
+    rows_body<Chain, V, ROWS, ALIGNED>(p);
+}
+
+// Whether the rows of plane z of the read and of the write all start on dword boundaries, decided on the device
+// (wave uniform, a handful of scalar instructions).  Kernels compiled at run time use this instead of the
+// launcher's host-side check, because their launcher does not know the chain's type.
+template <class Op, class P> FKD_DEV bool read_plane_aligned(const P& p, int z) {
+    if constexpr (requires { Op::plane_rows_aligned(p, z, 0); }) return Op::plane_rows_aligned(p, z, 0);
+    else return Op::rows_aligned(p, 0);
+}
+template <class Op, class P> FKD_DEV bool write_plane_aligned(const P& p, int z) {
+    if constexpr (requires { Op::plane_rows_aligned(p, z); }) return Op::plane_rows_aligned(p, z);
+    else return Op::rows_aligned(p);
+}
+template <class Chain, int V, int ROWS>
+__device__ __forceinline__ void rows_auto_body(const typename Chain::Params& p) {
+    const int z = blockIdx.z;
+    const bool aligned = read_plane_aligned<typename Chain::Read>(p.read, z) && write_plane_aligned<typename Chain::Write>(p.write, z);
+    if (aligned) rows_body<Chain, V, ROWS, true>(p);
+    else rows_body<Chain, V, ROWS, false>(p);
+}
+
 // ---- gather bilinear kernel ----------------------------------------------------------------------------
 
 #ifndef FKD_GATHER_XI
@@ -144,7 +170,7 @@ struct TileGeom {
 // All loads of a lane are issued before the first use and are unconditional (coordinates are clamped into the
 // source); only stores are predicated.
 template <class Chain, int XI, int YI>
-__global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename Chain::Params p, const TileGeom g) {
+__device__ __forceinline__ void gather_body(const typename Chain::Params& p, const TileGeom& g) {
     using Root = ResizeRoot<typename Chain::Read>;
     using RZ = typename Root::Resize;
     using Back = typename RZ::BackOp;
@@ -331,17 +357,22 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
         tail = Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back));
     }
     if (tail) {
-        rows(std::integral_constant<int, kSafe>{});
+        rows(IntTag<kSafe>{});
     } else {
         if constexpr (Back::kTapPair) {
-            if (!any_clamped) { rows(std::integral_constant<int, kPairs>{}); return; }
-            if (sw >= 2) { rows(std::integral_constant<int, kPairsSel>{}); return; }
+            if (!any_clamped) { rows(IntTag<kPairs>{}); return; }
+            if (sw >= 2) { rows(IntTag<kPairsSel>{}); return; }
         }
-        rows(std::integral_constant<int, kSingles>{});
+        rows(IntTag<kSingles>{});
     }
 }
 
-// ---- host-side launchers -------------------------------------------------------------------------------
+template <class Chain, int XI, int YI>
+__global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename Chain::Params p, const TileGeom g) {
+    gather_body<Chain, XI, YI>(p, g);
+}
+
+// ---- per-chain constants shared by the ahead-of-time and the run-time launchers ---------------------------
 
 template <class Chain> struct RowsConfig {
     // Four elements per thread wherever the chain reads rows; a bilinear read without a tap cursor keeps one
@@ -353,45 +384,22 @@ template <class Chain> struct RowsConfig {
     static constexpr int ROWS = ResizeRoot<typename Chain::Read>::value ? 1 : FKD_ROWS;
 };
 
-inline const char* aligned_name(bool aligned) { return aligned ? "rows" : "rows_unaligned"; }
-
-template <class Chain>
-hipError_t launch_rows(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
-    constexpr int V = RowsConfig<Chain>::V, ROWS = RowsConfig<Chain>::ROWS;
-    const unsigned gx = (p.active_w + kRowsBX * V - 1) / (kRowsBX * V);
-    const unsigned gy = (p.active_h + kRowsBY * ROWS - 1) / (kRowsBY * ROWS);
-    const dim3 grid(gx, gy, p.active_z), block(kRowsBX, kRowsBY, 1);
-    // Wide (dwordx3/x4) accesses need every row start dword aligned; checked here, once per launch, on the host.
-    const bool aligned = Chain::Read::rows_aligned(p.read, 0) && Chain::Write::rows_aligned(p.write);
-    if (info) *info = LaunchInfo{aligned_name(aligned), {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
-    if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
-    if (grid.y > 65535u || grid.z > 65535u) return hipErrorInvalidConfiguration;
-    if (aligned) hipLaunchKernelGGL((k_rows<Chain, V, ROWS, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((k_rows<Chain, V, ROWS, false>), grid, block, 0, stream, p);
-    return hipGetLastError();
+// The one kernel of a chain compiled at run time, and what its launcher needs to know about it.  A launcher that
+// only has the parameter block as bytes reads the active grid from its first three words.
+struct JitMeta {
+    u32 gather;          // 1: gather kernel geometry, 0: rows kernel geometry
+    u32 params_bytes;    // sizeof(Chain::Params)
+    u32 v, rows;         // rows kernel: elements per thread along x, rows per thread
+    u32 xi, yi, by;      // gather kernel: pixels per lane along x, rows per wave, waves per workgroup
+    u32 reserved;
+};
+template <class Chain> constexpr JitMeta jit_meta() {
+    return JitMeta{is_gather_chain<Chain>() ? 1u : 0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V),
+                   u32(RowsConfig<Chain>::ROWS), u32(FKD_GATHER_XI), u32(FKD_GATHER_YI), u32(kGatherBY), 0u};
 }
-
-template <class Chain>
-hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
-    constexpr int XI = FKD_GATHER_XI, YI = FKD_GATHER_YI;
-    constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
-    TileGeom g;
-    g.tiles_x = (p.active_w + TW - 1) / TW;
-    g.tiles_y = (p.active_h + TH - 1) / TH;
-    g.n_tiles = g.tiles_x * g.tiles_y * p.active_z;
-    const unsigned chunk = (g.tiles_x * g.tiles_y + 7u) / 8u;
-    const dim3 grid(chunk * 8u, 1, p.active_z), block(kGatherBX, kGatherBY, 1);
-    if (info) *info = LaunchInfo{"gather", {grid.x, 1, grid.z}, {block.x, block.y, 1}, 0};
-    if (g.n_tiles == 0) return hipSuccess;
-    if (grid.z > 65535u) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((k_gather<Chain, XI, YI>), grid, block, 0, stream, p, g);
-    return hipGetLastError();
-}
-
-template <class Chain>
-hipError_t launch_chain(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
-    if constexpr (is_gather_chain<Chain>()) return launch_gather<Chain>(p, stream, info);
-    else return launch_rows<Chain>(p, stream, info);
+template <class Chain> __device__ __forceinline__ void jit_body(const typename Chain::Params& p, const TileGeom& g) {
+    if constexpr (is_gather_chain<Chain>()) gather_body<Chain, FKD_GATHER_XI, FKD_GATHER_YI>(p, g);
+    else rows_auto_body<Chain, RowsConfig<Chain>::V, RowsConfig<Chain>::ROWS>(p);
 }
 
 } // namespace fkd

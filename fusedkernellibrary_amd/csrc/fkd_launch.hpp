@@ -1,0 +1,52 @@
+// fkd_launch.hpp -- host-side launchers of the ahead-of-time compiled kernels (grid geometry, host-side alignment
+// check, hipLaunchKernelGGL).  Launch geometry being replaced: FK/core/execution_model/executors.h:242-351.
+#pragma once
+
+#include "fkd_kernels.hpp"
+
+namespace fkd {
+
+// ---- host-side launchers -------------------------------------------------------------------------------
+
+inline const char* aligned_name(bool aligned) { return aligned ? "rows" : "rows_unaligned"; }
+
+template <class Chain>
+hipError_t launch_rows(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
+    constexpr int V = RowsConfig<Chain>::V, ROWS = RowsConfig<Chain>::ROWS;
+    const unsigned gx = (p.active_w + kRowsBX * V - 1) / (kRowsBX * V);
+    const unsigned gy = (p.active_h + kRowsBY * ROWS - 1) / (kRowsBY * ROWS);
+    const dim3 grid(gx, gy, p.active_z), block(kRowsBX, kRowsBY, 1);
+    // Wide (dwordx3/x4) accesses need every row start dword aligned; checked here, once per launch, on the host.
+    const bool aligned = Chain::Read::rows_aligned(p.read, 0) && Chain::Write::rows_aligned(p.write);
+    if (info) *info = LaunchInfo{aligned_name(aligned), {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
+    if (grid.y > 65535u || grid.z > 65535u) return hipErrorInvalidConfiguration;
+    if (aligned) hipLaunchKernelGGL((k_rows<Chain, V, ROWS, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((k_rows<Chain, V, ROWS, false>), grid, block, 0, stream, p);
+    return hipGetLastError();
+}
+
+template <class Chain>
+hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
+    constexpr int XI = FKD_GATHER_XI, YI = FKD_GATHER_YI;
+    constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
+    TileGeom g;
+    g.tiles_x = (p.active_w + TW - 1) / TW;
+    g.tiles_y = (p.active_h + TH - 1) / TH;
+    g.n_tiles = g.tiles_x * g.tiles_y * p.active_z;
+    const unsigned chunk = (g.tiles_x * g.tiles_y + 7u) / 8u;
+    const dim3 grid(chunk * 8u, 1, p.active_z), block(kGatherBX, kGatherBY, 1);
+    if (info) *info = LaunchInfo{"gather", {grid.x, 1, grid.z}, {block.x, block.y, 1}, 0};
+    if (g.n_tiles == 0) return hipSuccess;
+    if (grid.z > 65535u) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_gather<Chain, XI, YI>), grid, block, 0, stream, p, g);
+    return hipGetLastError();
+}
+
+template <class Chain>
+hipError_t launch_chain(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
+    if constexpr (is_gather_chain<Chain>()) return launch_gather<Chain>(p, stream, info);
+    else return launch_rows<Chain>(p, stream, info);
+}
+
+} // namespace fkd

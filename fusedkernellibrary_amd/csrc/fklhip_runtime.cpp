@@ -31,12 +31,12 @@ thread_local fkd::LaunchInfo g_last = {"", {0, 0, 0}, {0, 0, 0}, 0};
 
 } // namespace
 
-void register_chain(const char* signature, size_t blob_bytes, LaunchFn fn) {
+void register_chain(const char* signature, size_t blob_bytes, LaunchFn fn, const void* ctx) {
     Table& t = table();
     std::lock_guard<std::mutex> lock(t.mu);
     if (t.index.count(signature)) return;
     t.index.emplace(signature, t.entries.size());
-    t.entries.push_back(Entry{signature, blob_bytes, fn});
+    t.entries.push_back(Entry{signature, blob_bytes, fn, ctx});
 }
 
 } // namespace fklhip
@@ -51,7 +51,8 @@ const char* fklhip_error_string(int code) {
     switch (code) {
     case FKLHIP_OK: return "success";
     case FKLHIP_EUNKNOWN_SIGNATURE:
-        return "no kernel was compiled for this chain signature (add it to aot_signatures.txt and rebuild libfklhip.so)";
+        return "no kernel was compiled for this chain signature (add it to aot_signatures.txt and rebuild libfklhip.so)"
+               " and it could not be compiled at run time (fklhip_jit_log has the compiler's messages)";
     case FKLHIP_EBLOB_SIZE: return "parameter block size does not match the chain signature";
     case FKLHIP_EINVAL: return "invalid argument";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
@@ -124,10 +125,24 @@ int fklhip_event_elapsed_ms(float* ms, void* start, void* stop) {
 int fklhip_lookup(const char* signature, const void** handle) {
     if (!signature || !handle) return FKLHIP_EINVAL;
     Table& t = table();
-    std::lock_guard<std::mutex> lock(t.mu);
-    const auto it = t.index.find(signature);
-    if (it == t.index.end()) { *handle = nullptr; return FKLHIP_EUNKNOWN_SIGNATURE; }
+    std::unique_lock<std::mutex> lock(t.mu);
+    auto it = t.index.find(signature);
+    if (it == t.index.end()) {
+        // Not compiled ahead of time: compile it now (once per process), outside the table lock.
+        lock.unlock();
+        const int rc = jit_compile_and_register(signature);
+        lock.lock();
+        if (rc != FKLHIP_OK) { *handle = nullptr; return rc; }
+        it = t.index.find(signature);
+        if (it == t.index.end()) { *handle = nullptr; return FKLHIP_EUNKNOWN_SIGNATURE; }
+    }
     *handle = reinterpret_cast<const void*>(it->second + 1);   // index + 1: entries never move out of the table
+    return FKLHIP_OK;
+}
+
+int fklhip_jit_log(const char** log) {
+    if (!log) return FKLHIP_EINVAL;
+    *log = jit_last_log();
     return FKLHIP_OK;
 }
 
@@ -140,7 +155,7 @@ int fklhip_launch_handle(const void* handle, const void* blob, size_t blob_bytes
         if (idx == 0 || idx > t.entries.size()) return FKLHIP_EINVAL;
         e = t.entries[idx - 1];
     }
-    return e.launch(blob, blob_bytes, stream, &g_last);
+    return e.launch(e.ctx, blob, blob_bytes, stream, &g_last);
 }
 
 int fklhip_launch(const char* signature, const void* blob, size_t blob_bytes, void* stream) {

@@ -1065,6 +1065,7 @@ template <int N, class PlaneOp> struct BatchRead {
         for (int i = 0; i < N; ++i) if (!PlaneOp::rows_aligned(p.plane[i], xoff)) return false;
         return true;
     }
+    FKD_HD static bool plane_rows_aligned(const Params& p, int z, int xoff) { return PlaneOp::rows_aligned(p.plane[z], xoff); }
 #endif
 };
 
@@ -1092,6 +1093,9 @@ template <int N, class PlaneOp> struct BatchReadDefault {
     FKD_HD static bool rows_aligned(const Params& p, int xoff) {
         for (int i = 0; i < N && i < p.used; ++i) if (!PlaneOp::rows_aligned(p.plane[i], xoff)) return false;
         return true;
+    }
+    FKD_HD static bool plane_rows_aligned(const Params& p, int z, int xoff) {
+        return z >= p.used || PlaneOp::rows_aligned(p.plane[z], xoff);
     }
 #endif
 };
@@ -1276,6 +1280,7 @@ template <int N, class W> struct BatchWrite {
         for (int i = 0; i < N; ++i) if (!W::rows_aligned(p.plane[i])) return false;
         return true;
     }
+    FKD_HD static bool plane_rows_aligned(const Params& p, int z) { return W::rows_aligned(p.plane[z]); }
     using Plane = W;
     FKD_DEV static const typename W::Params& plane_params(const Params& p, int z) { return p.plane[z]; }
     using RowRef = typename W::RowRef;

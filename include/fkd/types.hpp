@@ -5,7 +5,21 @@
 // fenced by FKD_DEVICE_CODE (defined by the HIP translation units); host-only naming helpers by FKD_HOST_NAMES.
 #pragma once
 
+#if defined(__HIPCC_RTC__)
+// Run-time compilation has no C library headers: name the fixed-width types through the compiler's own macros.
+typedef __UINT8_TYPE__ uint8_t;
+typedef __INT8_TYPE__ int8_t;
+typedef __UINT16_TYPE__ uint16_t;
+typedef __INT16_TYPE__ int16_t;
+typedef __UINT32_TYPE__ uint32_t;
+typedef __INT32_TYPE__ int32_t;
+typedef __UINTPTR_TYPE__ uintptr_t;
+typedef __PTRDIFF_TYPE__ ptrdiff_t;
+typedef __SIZE_TYPE__ size_t;
+#else
+#include <stddef.h>
 #include <stdint.h>
+#endif
 
 #if defined(FKD_DEVICE_CODE)
 #define FKD_DEV __device__ __forceinline__

@@ -90,8 +90,16 @@ int fklhip_lookup(const char *signature, const void **handle);
 int fklhip_launch_handle(const void *handle, const void *blob, size_t blob_bytes, void *stream);
 int fklhip_launch(const char *signature, const void *blob, size_t blob_bytes, void *stream);
 
+/* A signature that was not compiled ahead of time is compiled when fklhip_lookup / fklhip_launch first see it
+ * (device headers are embedded in the library; about a second per new signature, once per process; switched off by
+ * the environment variable FKLHIP_JIT=0).  This is the library's stand-in for nvcc compiling the user's translation
+ * unit, FK/core/execution_model/executors.h:316-351 being instantiated for whatever chain the user wrote.  When the
+ * lookup fails, fklhip_jit_log returns the device compiler's messages for the last attempt on this thread (valid
+ * until the next lookup on the thread). */
+int fklhip_jit_log(const char **log);
+
 /* Introspection for tests and benchmarks: what the last fklhip_launch* on this thread launched.
- * kernel receives "rows", "rows_unaligned" or "gather"; grid/block receive 3 values each. */
+ * kernel receives "rows", "rows_unaligned", "gather", or "rows_jit" / "gather_jit" for chains compiled at run time; grid/block receive 3 values each. */
 int fklhip_last_launch(const char **kernel, unsigned grid[3], unsigned block[3], unsigned *lds_bytes);
 
 /* Number of chain signatures compiled into the library and the i-th of them with its parameter block size. */

@@ -296,6 +296,42 @@ int fklcase_set_to_shapes(void* stream_, int w, int h, int planes, const uint8_t
     });
 }
 
+// Chains that are NOT in the ahead-of-time list: the library compiles them when it first sees them.
+int fklcase_uncompiled_pointwise_f32(void* stream_, const float* in, int w, int h, int pitch, float* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<float>(in, w, h, pitch);
+        const auto o = dev2d<float>(out, w, h, out_pitch);
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, float>::build(i.ptr()), Mul<float>::build(1.5f),
+                                          Sub<float>::build(0.25f), Div<float>::build(3.f), Add<float>::build(7.f),
+                                          PerThreadWrite<ND::_2D, float>::build(o.ptr()));
+    });
+}
+// one-channel uchar image -> crop -> bilinear resize -> Mul -> float image
+int fklcase_uncompiled_gray_resize(void* stream_, const uint8_t* in, int w, int h, int pitch, const int32_t* rect, int dw, int dh,
+                                   float mul, float* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<uchar>(in, w, h, pitch);
+        const auto o = dev2d<float>(out, dw, dh, out_pitch);
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, uchar>::build(i.ptr()),
+                                          Crop<>::build(Rect(rect[0], rect[1], rect[2], rect[3])),
+                                          Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)), Mul<float>::build(mul),
+                                          PerThreadWrite<ND::_2D, float>::build(o.ptr()));
+    });
+}
+// float4 image -> bilinear resize -> float4 image (16-byte elements: one access per tap)
+int fklcase_uncompiled_float4_resize(void* stream_, const float* in, int w, int h, int pitch, int dw, int dh, float* out, int out_pitch) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto i = dev2d<float4>(in, w, h, pitch);
+        const auto o = dev2d<float4>(out, dw, dh, out_pitch);
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, float4>::build(i.ptr()),
+                                          Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
+                                          PerThreadWrite<ND::_2D, float4>::build(o.ptr()));
+    });
+}
+
 // Single-operation chains for the exhaustive numeric tests.
 int fklcase_div_f32(void* stream_, const float* in, int w, int h, int pitch, float d, float* out, int out_pitch) {
     return guarded([&] {
