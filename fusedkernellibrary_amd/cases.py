@@ -175,3 +175,14 @@ def uncompiled_float4_resize(src, dst, out):
     """(H,W,4) f32 cuda -> bilinear -> out (dh,dw,4) f32 cuda."""
     _ok(cases().fklcase_uncompiled_float4_resize(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, int(dst[0]), int(dst[1]),
                                                  _p(out), out.stride(0) * 4))
+
+
+def warp(src, matrix, perspective, dst, out):
+    """src (H,W,3) u8 or (H,W) f32 cuda; matrix 2x3 (affine) or 3x3 (perspective); out (dh,dw,3) / (dh,dw) f32 cuda."""
+    m = np.zeros(9, np.float32)
+    m[: (9 if perspective else 6)] = np.asarray(matrix, np.float32).ravel()
+    is_u8 = src.element_size() == 1
+    fn = cases().fklcase_warp_u8x3 if is_u8 else cases().fklcase_warp_f32
+    esz = 1 if is_u8 else 4
+    _ok(fn(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * esz, m.ctypes.data_as(C.c_void_p), int(bool(perspective)),
+           int(dst[0]), int(dst[1]), _p(out), out.stride(0) * 4))

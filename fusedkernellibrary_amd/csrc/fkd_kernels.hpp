@@ -55,6 +55,13 @@ template <int N, int AR, class Back> struct ResizeRoot<BatchReadDefault<N, Resiz
 template <class R> struct HasDefaultPlanes { static constexpr bool value = false; };
 template <int N, class PlaneOp> struct HasDefaultPlanes<BatchReadDefault<N, PlaneOp>> { static constexpr bool value = true; };
 
+// Reads whose taps are scattered gathers (warps): the rows kernel then keeps one element per thread.
+template <class R> constexpr bool is_scattered_read() {
+    if constexpr (requires { R::kGatherRead; }) return R::kGatherRead;
+    else if constexpr (requires { typename R::Plane; }) return is_scattered_read<typename R::Plane>();
+    else return false;
+}
+
 template <class Chain> constexpr bool is_gather_chain() {
     if constexpr (ResizeRoot<typename Chain::Read>::value)
         return ResizeRoot<typename Chain::Read>::Resize::BackOp::kTapCursor;
@@ -377,11 +384,12 @@ __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename
 template <class Chain> struct RowsConfig {
     // Four elements per thread wherever the chain reads rows; a bilinear read without a tap cursor keeps one
     // element per thread (its taps are gathers, wider threads would only spread them further apart).
-    static constexpr int V = ResizeRoot<typename Chain::Read>::value ? 1 : 4;
+    static constexpr bool kScattered = ResizeRoot<typename Chain::Read>::value || is_scattered_read<typename Chain::Read>();
+    static constexpr int V = kScattered ? 1 : 4;
 #ifndef FKD_ROWS
 #define FKD_ROWS 4
 #endif
-    static constexpr int ROWS = ResizeRoot<typename Chain::Read>::value ? 1 : FKD_ROWS;
+    static constexpr int ROWS = kScattered ? 1 : FKD_ROWS;
 };
 
 // The one kernel of a chain compiled at run time, and what its launcher needs to know about it.  A launcher that

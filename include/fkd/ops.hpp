@@ -1047,6 +1047,68 @@ template <int AR, class Back> struct ResizeLinear {
 #endif
 };
 
+// Warping<Affine|Perspective, Back>: FK/algorithms/image_processing/warping.h:42-96.  Destination pixel (x, y) maps
+// to source coordinate m * (x, y, 1) (row sums left to right, perspective divide as a multiplication by the
+// reciprocal, as the reference writes it); outside [0,w) x [0,h) the result is 0, inside it is the bilinear
+// interpolation of interpolation.h:70-104 at that coordinate (floor, +1 taps clamped, weights from the unclamped
+// +1 coordinates).
+template <int WT, class Back> struct Warp {
+    using Src = typename Back::Out;
+    using Out = vec_t<f32, cn_v<Src>>;
+    struct Params {
+        f32 m[9];
+        i32 dst_w, dst_h;
+        typename Back::Params back;
+    };
+    static constexpr bool kTapCursor = false;
+    static constexpr bool kGatherRead = true;     // taps are scattered: one element per thread
+    FKD_NAME("Warp<" + istr(WT) + "," + Back::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return p.dst_w; }
+    FKD_DEV static int height(const Params& p) { return p.dst_h; }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        const f32 fx = f32(x), fy = f32(y);
+        f32 sx = (p.m[0] * fx + p.m[1] * fy) + p.m[2];
+        f32 sy = (p.m[3] * fx + p.m[4] * fy) + p.m[5];
+        if constexpr (WT == 1) {
+            const f32 coeff = 1.0f / ((p.m[6] * fx + p.m[7] * fy) + p.m[8]);
+            sx = coeff * sx;
+            sy = coeff * sy;
+        }
+        const int sw = Back::width(p.back), sh = Back::height(p.back);
+        Out o;
+        if (sx >= 0.f && sx < f32(sw) && sy >= 0.f && sy < f32(sh)) {
+            const f32 f1x = __builtin_floorf(sx), f1y = __builtin_floorf(sy);
+            const int x1 = int(f1x), y1 = int(f1y);
+            const int x2 = x1 + 1, y2 = y1 + 1;
+            const int x2r = x2 < sw - 1 ? x2 : sw - 1, y2r = y2 < sh - 1 ? y2 : sh - 1;
+            const f32 ax = f32(x2) - sx, bx = sx - f32(x1), ay = f32(y2) - sy, by = sy - f32(y1);
+            const f32 w00 = ax * ay, w10 = bx * ay, w01 = ax * by, w11 = bx * by;
+            const Src a = Back::exec(x1, y1, z, p.back), b = Back::exec(x2r, y1, z, p.back);
+            const Src c = Back::exec(x1, y2r, z, p.back), d = Back::exec(x2r, y2r, z, p.back);
+            auto one = [&](auto pa, auto pb, auto pc, auto pd) {
+                return ((f32(pa) * w00 + f32(pb) * w10) + f32(pc) * w01) + f32(pd) * w11;
+            };
+            chan<0>(o) = one(chan<0>(a), chan<0>(b), chan<0>(c), chan<0>(d));
+            if constexpr (cn_v<Src> > 1) chan<1>(o) = one(chan<1>(a), chan<1>(b), chan<1>(c), chan<1>(d));
+            if constexpr (cn_v<Src> > 2) chan<2>(o) = one(chan<2>(a), chan<2>(b), chan<2>(c), chan<2>(d));
+            if constexpr (cn_v<Src> > 3) chan<3>(o) = one(chan<3>(a), chan<3>(b), chan<3>(c), chan<3>(d));
+        } else {
+            chan<0>(o) = 0.f;
+            if constexpr (cn_v<Src> > 1) chan<1>(o) = 0.f;
+            if constexpr (cn_v<Src> > 2) chan<2>(o) = 0.f;
+            if constexpr (cn_v<Src> > 3) chan<3>(o) = 0.f;
+        }
+        return o;
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+    }
+    FKD_HD static bool rows_aligned(const Params&, int) { return true; }
+#endif
+};
+
 // BatchRead<PROCESS_ALL, N, Op>: FK/core/execution_model/operation_model/batch_operations.h:164-219.  Plane z
 // uses its own parameter set; z is the workgroup's grid-z index, so the selection is wave uniform.
 template <int N, class PlaneOp> struct BatchRead {

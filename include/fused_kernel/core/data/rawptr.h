@@ -93,5 +93,32 @@ template <> struct PtrAccessor<ND::_3D> {
     }
 };
 
+// Small arrays with compile-time extents held by value (transform matrices and the like).
+// Interface counterpart: FK/core/data/rawptr.h:105-185.
+template <int W> struct StaticPtrDims1D { static constexpr uint width{W}; };
+template <int W, int H> struct StaticPtrDims2D { static constexpr uint width{W}; static constexpr uint height{H}; };
+template <int W, int H, int P> struct StaticPtrDims3D {
+    static constexpr uint width{W}; static constexpr uint height{H}; static constexpr uint planes{P};
+};
+template <typename Dims, typename T> struct StaticRawPtr;
+template <typename T, int W> struct StaticRawPtr<StaticPtrDims1D<W>, T> {
+    using type = T;
+    T data[W];
+    static constexpr StaticPtrDims1D<W> dims{};
+    static constexpr ND NDim{ND::_1D};
+};
+template <typename T, int W, int H> struct StaticRawPtr<StaticPtrDims2D<W, H>, T> {
+    using type = T;
+    T data[H][W];
+    static constexpr StaticPtrDims2D<W, H> dims{};
+    static constexpr ND NDim{ND::_2D};
+};
+template <typename T, int W, int H, int P> struct StaticRawPtr<StaticPtrDims3D<W, H, P>, T> {
+    using type = T;
+    T data[P][H][W];
+    static constexpr StaticPtrDims3D<W, H, P> dims{};
+    static constexpr ND NDim{ND::_3D};
+};
+
 } // namespace fk
 #endif

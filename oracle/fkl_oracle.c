@@ -316,6 +316,44 @@ static int write_value(const fklo_write *w, int x, int y, int z, const fklo_val 
  * active threads of the (fused) read; BatchRead picks plane z (batch_operations.h:205-212) and
  * activeThreads = (max W, max H, BATCH) (batch_operations.h:401-424). Planes whose own geometry is smaller
  * than the maximum are rejected here: the reference runs them unchecked, which reads outside the crop. */
+/* Warping<WT, BackIOp>::exec and WarpingCoords<WT>::exec, FK/algorithms/image_processing/warping.h:42-96: the
+ * destination pixel maps to m * (x, y, 1); inside the source the value is InterpolateComplete<INTER_LINEAR> at
+ * that coordinate (interpolation.h:70-104), outside it is 0. */
+static int read_warped(const fklo_read *r, int x, int y, fklo_val *out) {
+    const float *m = r->warp_m;
+    float sx = (m[0] * (float)x + m[1] * (float)y) + m[2];
+    float sy = (m[3] * (float)x + m[4] * (float)y) + m[5];
+    if (r->warp == 2) {
+        const float coeff = 1.0f / ((m[6] * (float)x + m[7] * (float)y) + m[8]);
+        sx = coeff * sx;
+        sy = coeff * sy;
+    }
+    int sw, sh;
+    read_extent(r, &sw, &sh);
+    out->elem = FKLO_F32;
+    out->cn = r->kind == FKLO_READ_NV12 ? 3 : r->cn;
+    if (!(sx >= 0.f && sx < (float)sw && sy >= 0.f && sy < (float)sh)) {
+        for (int c = 0; c < out->cn; ++c) out->f[c] = 0.f;
+        return FKLO_OK;
+    }
+    const int x1 = (int)floorf(sx), y1 = (int)floorf(sy);
+    const int x2 = x1 + 1, y2 = y1 + 1;
+    const int x2r = x2 < sw - 1 ? x2 : sw - 1;
+    const int y2r = y2 < sh - 1 ? y2 : sh - 1;
+    fklo_val t00, t10, t01, t11;
+    int rc;
+    if ((rc = read_tap(r, x1, y1, &t00))) return rc;
+    if ((rc = read_tap(r, x2r, y1, &t10))) return rc;
+    if ((rc = read_tap(r, x1, y2r, &t01))) return rc;
+    if ((rc = read_tap(r, x2r, y2r, &t11))) return rc;
+    out->cn = t00.cn;
+    for (int c = 0; c < t00.cn; ++c) {
+        out->f[c] = fklo_bilinear(chan_as_float(&t00, c), chan_as_float(&t10, c),
+                                  chan_as_float(&t01, c), chan_as_float(&t11, c), sx, sy);
+    }
+    return FKLO_OK;
+}
+
 /* BatchRead<CONDITIONAL_WITH_DEFAULT>::exec, FK/core/execution_model/operation_model/batch_operations.h:262-273:
  * planes at or beyond usedPlanes return params.default_value, whose type is the plane operation's output type
  * (float_<cn> after a resize, the tap type after fused tap operations, else the element type). */
@@ -349,7 +387,8 @@ int fklo_execute(int32_t n_planes, const fklo_read *reads,
     int act_w = 0, act_h = 0;
     for (int z = 0; z < n_planes; ++z) {
         int w, h;
-        if (reads[z].has_resize) { w = reads[z].dst_w; h = reads[z].dst_h; }
+        if (reads[z].has_resize && reads[z].warp) return FKLO_EINVAL;
+        if (reads[z].has_resize || reads[z].warp) { w = reads[z].dst_w; h = reads[z].dst_h; }
         else read_extent(&reads[z], &w, &h);
         if (z == 0) { act_w = w; act_h = h; }
         else if (w != act_w || h != act_h) return FKLO_EGEOM;
@@ -369,6 +408,7 @@ int fklo_execute(int32_t n_planes, const fklo_read *reads,
                 fklo_val v;
                 int rc = FKLO_OK;
                 if (r->use_default) read_default(r, &v);
+                else if (r->warp) rc = read_warped(r, x, y, &v);
                 else rc = r->has_resize ? read_resized(r, &rp, x, y, &v) : read_tap(r, x, y, &v);
                 if (rc) return rc;
                 for (int i = 0; i < n_ops; ++i) {

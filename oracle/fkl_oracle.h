@@ -84,6 +84,8 @@ typedef struct {
     const fklo_op *tap_ops;
     int32_t use_default;     /* BatchRead<CONDITIONAL_WITH_DEFAULT>, plane index >= usedPlanes: every element of */
     float def[4];            /* this plane is def, typed like the read's output, and nothing is read             */
+    int32_t warp;            /* 0 none, 1 Warping<Affine>, 2 Warping<Perspective>; output grid dst_w x dst_h,     */
+    float warp_m[9];         /* row-major transform (affine uses the first two rows); excludes has_resize         */
 } fklo_read;
 
 typedef struct {

@@ -14,6 +14,7 @@
 #include <fused_kernel/algorithms/image_processing/crop.h>
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
+#include <fused_kernel/algorithms/image_processing/warping.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
@@ -122,6 +123,23 @@ int batch_default_cast_mul(const uint8_t* const* srcs, int w, int h, int pitch, 
     return 0;
 }
 
+// Warping<Affine|Perspective> of a uchar3 image into a float3 image (matrix row-major, 6 or 9 values).
+template <WarpType WT>
+int warp_u8x3(const uint8_t* src, int w, int h, int pitch, const float* m, int dw, int dh, float* out) {
+    CpuStream stream;
+    const auto in = wrap2d<uchar3>(src, w, h, pitch);
+    Ptr2D<float3> o(reinterpret_cast<float3*>(out), uint(dw), uint(dh), uint(dw) * uint(sizeof(float3)), MemType::Host, 0);
+    WarpingParameters<WT> params{};
+    constexpr int rows = WT == WarpType::Affine ? 2 : 3;
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < 3; ++c) params.transformMatrix.data[r][c] = m[r * 3 + c];
+    params.dstSize = Size(dw, dh);
+    executeOperations<CpuDPP>(stream, PerThreadRead<ND::_2D, uchar3>::build(in.ptr()).then(Warping<WT>::build(params)),
+                              PerThreadWrite<ND::_2D, float3>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
 // Benchmark configuration 4: B independent uchar3 images, per-image Mul and Add fused into each plane's
 // read, SaturateCast, B separate outputs in one launch.
 template <size_t B>
@@ -214,6 +232,11 @@ int fklref_crop_resize_default_norm_split_b8(const uint8_t* src, int w, int h, i
 int fklref_batch_default_cast_mul_b4(const uint8_t* const* srcs, int w, int h, int pitch, int active, const uint8_t* def,
                                      const float* mul, float* out) {
     return batch_default_cast_mul<4>(srcs, w, h, pitch, active, def, mul, out);
+}
+
+int fklref_warp_u8x3(const uint8_t* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh, float* out) {
+    return perspective ? warp_u8x3<WarpType::Perspective>(src, w, h, pitch, m, dw, dh, out)
+                       : warp_u8x3<WarpType::Affine>(src, w, h, pitch, m, dw, dh, out);
 }
 
 int fklref_batch_muladd_sat_b4(const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,

@@ -169,3 +169,13 @@ void set_loop_and_conditional_batch() {
     executeOperations<TransformDPP<>>(ins, 2, uchar3{1, 2, 3}, t, stream, Cast<uchar3, float3>::build());
     stream.sync();
 }
+
+// ---- Warping, as the reference's own test spells it (tests/algorithm/test_warp.h:20-33) -------------------------
+#include <fused_kernel/algorithms/image_processing/warping.h>
+constexpr auto warpReadIOp = fk::PerThreadRead<fk::ND::_2D, uchar3>::build(
+    fk::RawPtr<fk::ND::_2D, uchar3>{nullptr, {128, 128, 128 * sizeof(uchar3)}});
+constexpr auto warpIOp = fk::Warping<fk::WarpType::Perspective>::build(fk::WarpingParameters<fk::WarpType::Perspective>{});
+constexpr auto warpFusedIOp = warpReadIOp.then(warpIOp);
+static_assert(std::is_same_v<std::decay_t<decltype(warpFusedIOp)>,
+                             fk::ReadBack<fk::Warping<fk::WarpType::Perspective, fk::Read<fk::PerThreadRead<fk::ND::_2D, uchar3>>>>>,
+              "Unexpected type for fusedIOp");

@@ -12,6 +12,7 @@
 #include <fused_kernel/algorithms/image_processing/crop.h>
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
+#include <fused_kernel/algorithms/image_processing/warping.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
@@ -161,6 +162,21 @@ template <int N> void set_and_loop(Stream& stream, int n, float init, float add,
     out.download(stream);
     stream.sync();
     std::memcpy(host_out, out.ptrPinned().data, size_t(n) * sizeof(float));
+}
+
+// Warping<Affine|Perspective> of an image of T into a float image with the same channel count (row-major matrix).
+template <WarpType WT, typename T, typename O>
+void warp_image(void* stream_, const void* src, int w, int h, int pitch, const float* m, int dw, int dh, void* out, int out_pitch) {
+    Stream stream(stream_);
+    const auto in = dev2d<T>(src, w, h, pitch);
+    const auto o = dev2d<O>(out, dw, dh, out_pitch);
+    WarpingParameters<WT> params{};
+    constexpr int rows = WT == WarpType::Affine ? 2 : 3;
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < 3; ++c) params.transformMatrix.data[r][c] = m[r * 3 + c];
+    params.dstSize = Size(dw, dh);
+    executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, T>::build(in.ptr()).then(Warping<WT>::build(params)),
+                                      PerThreadWrite<ND::_2D, O>::build(o.ptr()));
 }
 
 extern "C" {
@@ -329,6 +345,21 @@ int fklcase_uncompiled_float4_resize(void* stream_, const float* in, int w, int 
         executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, float4>::build(i.ptr()),
                                           Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
                                           PerThreadWrite<ND::_2D, float4>::build(o.ptr()));
+    });
+}
+
+int fklcase_warp_u8x3(void* stream, const uint8_t* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh,
+                      float* out, int out_pitch) {
+    return guarded([&] {
+        if (perspective) warp_image<WarpType::Perspective, uchar3, float3>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
+        else warp_image<WarpType::Affine, uchar3, float3>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
+    });
+}
+int fklcase_warp_f32(void* stream, const float* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh,
+                     float* out, int out_pitch) {
+    return guarded([&] {
+        if (perspective) warp_image<WarpType::Perspective, float, float>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
+        else warp_image<WarpType::Affine, float, float>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
     });
 }
 

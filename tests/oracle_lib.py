@@ -35,6 +35,7 @@ class Read(C.Structure):
         ("ar", C.c_int32), ("bg", C.c_float * 4),
         ("n_tap_ops", C.c_int32), ("tap_ops", C.POINTER(Op)),
         ("use_default", C.c_int32), ("def_", C.c_float * 4),
+        ("warp", C.c_int32), ("warp_m", C.c_float * 9),
     ]
 
 
@@ -252,6 +253,32 @@ def oracle_batch_default_cast_mul(srcs, active, default, mul):
     for i in range(active, b):
         _defaulted(reads[i], default)
     execute(reads, [op(CAST_F32), op(MUL, mul)], [write(TENSOR_WRITE, out, 3, w, h, b, 1)])
+    return out
+
+
+def oracle_warp(src, cn, matrix, dst, perspective):
+    """Warping<Affine|Perspective> of an (H,W[,cn]) u8/f32 image into a (dh,dw[,cn]) float image."""
+    dw, dh = dst
+    out = np.zeros((dh, dw, cn) if cn > 1 else (dh, dw), np.float32)
+    r = read_2d(src, cn)
+    r.warp = 2 if perspective else 1
+    r.dst_w, r.dst_h = dw, dh
+    m = np.zeros(9, np.float32)
+    m[: (9 if perspective else 6)] = np.asarray(matrix, np.float32).ravel()
+    for i in range(9):
+        r.warp_m[i] = float(m[i])
+    execute([r], [], [write(WRITE_2D, out, cn, dw, dh)])
+    return out
+
+
+def ref_warp_u8x3(src, matrix, dst, perspective):
+    dw, dh = dst
+    out = np.zeros((dh, dw, 3), np.float32)
+    m = np.zeros(9, np.float32)
+    m[: (9 if perspective else 6)] = np.asarray(matrix, np.float32).ravel()
+    rc = ref().fklref_warp_u8x3(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], _f32p(m), int(bool(perspective)),
+                                dw, dh, C.c_void_p(_ptr(out)))
+    assert rc == 0
     return out
 
 

@@ -339,3 +339,29 @@ def test_default_planes_closed_form():
     assert np.all(out[2:, 0] == np.float32((40.0 - 1.0) / 2.0)) and np.all(out[2:, 1] == np.float32((20.0 - 2.0) / 4.0))
     assert np.all(out[2:, 2] == np.float32((10.0 - 3.0) / 8.0))
     assert np.all(out[:2, 0] == np.float32((9.0 - 1.0) / 2.0))
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="reference CPU backend not built (needs the reference tree)")
+def test_warp_matches_reference_backend():
+    """Warping<Affine|Perspective> (warping.h:42-96) on a uchar3 image."""
+    import math
+    rng = np.random.RandomState(5)
+    src = rng.randint(0, 256, (90, 131, 3)).astype(np.uint8)
+    th = math.radians(17)
+    affine = [[1.3 * math.cos(th), -1.3 * math.sin(th), 20.5], [1.3 * math.sin(th), 1.3 * math.cos(th), -7.25]]
+    persp = [[1.1, 0.05, -3.0], [0.02, 0.9, 4.0], [0.0008, -0.0005, 1.0]]
+    for matrix, p, dst in ((affine, False, (100, 70)), (persp, True, (160, 120)), ([[1, 0, 0], [0, 1, 0]], False, (131, 90))):
+        a = ol.oracle_warp(src, 3, matrix, dst, p)
+        b = ol.ref_warp_u8x3(src, matrix, dst, p)
+        assert a.tobytes() == b.tobytes()
+
+
+def test_warp_closed_forms():
+    """Identity warp returns float(source); an integer shift returns the shifted source and zeros outside."""
+    rng = np.random.RandomState(8)
+    src = rng.randint(0, 256, (20, 30, 3)).astype(np.uint8)
+    out = ol.oracle_warp(src, 3, [[1, 0, 0], [0, 1, 0]], (30, 20), False)
+    assert (out == src.astype(np.float32)).all()
+    out = ol.oracle_warp(src, 3, [[1, 0, 4], [0, 1, -2]], (30, 20), False)   # dst (x,y) reads src (x+4, y-2)
+    assert (out[2:, :26] == src[:18, 4:].astype(np.float32)).all()
+    assert (out[:2] == 0).all() and (out[:, 26:] == 0).all()
