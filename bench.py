@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5 (c3 is always run)")
+    ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
 
@@ -86,7 +86,7 @@ def main():
     fkl.lib()   # raises if the HIP library is missing: there is no fallback
     dev = torch.device("cuda:0")
     timer = Timer(torch, fkl, cases)
-    only = set(filter(None, args.only.split(","))) or {"c1", "c2", "c3", "c4", "c5"}
+    only = set(filter(None, args.only.split(","))) or {"c1", "c2", "c3", "c4", "c5", "ext"}
     results = {}
 
     def record(name, out_px, alg_bytes, fn, steps, warmup):
@@ -148,6 +148,22 @@ def main():
         record("c4", 100 * 1920 * 1080, 2 * 100 * 1920 * 1080 * 3, lambda: cases.batch_muladd_sat(srcs, mul, add, outs),
                max(10, args.steps // 10), max(2, args.warmup // 10))
         del srcs, outs
+
+    if "ext" in only:
+        # rows beyond the five benchmark configurations: warp, conditional batch, fill
+        import math
+        rng = np.random.RandomState(7)
+        img = torch.from_numpy(rng.randint(0, 256, (1080, 1920, 3)).astype(np.uint8)).to(dev)
+        th = math.radians(7.0)
+        affine = [[math.cos(th), -math.sin(th), 40.0], [math.sin(th), math.cos(th), -60.0]]
+        wo = torch.zeros((1080, 1920, 3), dtype=torch.float32, device=dev)
+        record("warp_affine_1080p_u8x3", 1920 * 1080, 1920 * 1080 * (3 + 12), lambda: cases.warp(img, affine, False, (1920, 1080), wo),
+               args.steps, args.warmup)
+        rects8 = c3["rects"][:8]
+        o8 = torch.zeros((8, 3, 224, 224), dtype=torch.float32, device=dev)
+        record("c3_b8_default_planes_5_of_8", 8 * 224 * 224, 8 * 3 * 224 * 224 * 4,
+               lambda: cases.crop_resize_default_norm_split(src3, rects8, (224, 224), 5, (0.0, 0.0, 0.0), c3["sub"], c3["div"], o8),
+               args.steps, args.warmup)
 
     # ---- CPU baseline: the same chain on this machine's host cores, one thread, bounded sample --------------------
     cpu = None

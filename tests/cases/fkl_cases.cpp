@@ -175,8 +175,9 @@ void warp_image(void* stream_, const void* src, int w, int h, int pitch, const f
     for (int r = 0; r < rows; ++r)
         for (int c = 0; c < 3; ++c) params.transformMatrix.data[r][c] = m[r * 3 + c];
     params.dstSize = Size(dw, dh);
-    executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, T>::build(in.ptr()).then(Warping<WT>::build(params)),
-                                      PerThreadWrite<ND::_2D, O>::build(o.ptr()));
+    for (int rep = 0; rep < g_reps; ++rep)
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, T>::build(in.ptr()).then(Warping<WT>::build(params)),
+                                          PerThreadWrite<ND::_2D, O>::build(o.ptr()));
 }
 
 extern "C" {
