@@ -186,3 +186,10 @@ def warp(src, matrix, perspective, dst, out):
     esz = 1 if is_u8 else 4
     _ok(fn(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * esz, m.ctypes.data_as(C.c_void_p), int(bool(perspective)),
            int(dst[0]), int(dst[1]), _p(out), out.stride(0) * 4))
+
+
+def deinterlace(src, mode, out):
+    """src (H,W,3) u8 or (H,W) f32 cuda; mode 1 BLEND, 2 INTER_LINEAR keeping even lines, 3 keeping odd; out f32 same shape."""
+    is_u8 = src.element_size() == 1
+    fn = cases().fklcase_deinterlace_u8x3 if is_u8 else cases().fklcase_deinterlace_f32
+    _ok(fn(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * (1 if is_u8 else 4), int(mode), _p(out), out.stride(0) * 4))

@@ -1047,6 +1047,55 @@ template <int AR, class Back> struct ResizeLinear {
 #endif
 };
 
+// Deinterlace<BLEND|INTER_LINEAR, Back>: FK/algorithms/image_processing/deinterlace.h:24-121.  BLEND (DT 0): line y > 0
+// is (current + above + 1) * 0.5f, line 0 is current * 1.f.  INTER_LINEAR (DT 1): with use_even the odd lines
+// except the last, otherwise the even lines except the first, are (above + below + 1) * 0.5f; all other lines are
+// current * 1.f.  Sums follow the C++ promotions of the element type (uchar + uchar + 1 is an int).
+template <int DT, class Back> struct Deinterlace {
+    using Src = typename Back::Out;
+    using Out = vec_t<f32, cn_v<Src>>;
+    struct Params { i32 use_even; typename Back::Params back; };
+    static constexpr bool kTapCursor = false;
+    FKD_NAME("Deinterlace<" + istr(DT) + "," + Back::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
+    FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
+    // which lines take part for output line y: first, second, and whether they are averaged
+    FKD_DEV static void lines(int y, const Params& p, int& ya, int& yb, bool& average) {
+        const int h = Back::height(p.back);
+        if constexpr (DT == 0) {
+            average = y > 0;
+            ya = y; yb = y > 0 ? y - 1 : y;
+        } else {
+            const bool even = (y & 1) == 0;
+            average = p.use_even ? (!even && y != h - 1) : (even && y != 0);
+            ya = average ? y - 1 : y; yb = average ? y + 1 : y;
+            // The reference assumes an even number of lines; with an odd one and use_even == false its last line
+            // would read one line past the image.  Here that read takes the last line instead.
+            yb = yb < h ? yb : h - 1;
+        }
+    }
+    FKD_DEV static Out mix(const Src& a, const Src& b, bool average) {
+        return map2<Out>(a, b, [&](auto x, auto y) { return average ? (x + y + 1) * 0.5f : x * 1.f; });
+    }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        int ya, yb; bool average;
+        lines(y, p, ya, yb, average);
+        return mix(Back::exec(x, ya, z, p.back), Back::exec(x, yb, z, p.back), average);
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        int ya, yb; bool average;
+        lines(y, p, ya, yb, average);
+        Slot<Src> ra[V], rb[V];
+        Back::template exec_row<V, A>(x, ya, z, p.back, ra);
+        Back::template exec_row<V, A>(x, yb, z, p.back, rb);
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i].v = mix(ra[i].v, rb[i].v, average);
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
+#endif
+};
+
 // Warping<Affine|Perspective, Back>: FK/algorithms/image_processing/warping.h:42-96.  Destination pixel (x, y) maps
 // to source coordinate m * (x, y, 1) (row sums left to right, perspective divide as a multiplication by the
 // reciprocal, as the reference writes it); outside [0,w) x [0,h) the result is 0, inside it is the bilinear

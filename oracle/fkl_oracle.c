@@ -354,6 +354,43 @@ static int read_warped(const fklo_read *r, int x, int y, fklo_val *out) {
     return FKLO_OK;
 }
 
+/* Deinterlace<DType, BackIOp>::exec, FK/algorithms/image_processing/deinterlace.h:44-103.  Sums of uchar channels are
+ * ints (C++ promotion), of float channels floats; the result is float_<cn>. */
+static int read_deinterlaced(const fklo_read *r, int x, int y, fklo_val *out) {
+    int sw, sh;
+    read_extent(r, &sw, &sh);
+    int average, ya, yb;
+    if (r->deinterlace == 1) {
+        average = y > 0;
+        ya = y; yb = y - 1;                 /* current, above */
+    } else {
+        const int even = (y & 1) == 0;
+        average = r->deinterlace == 2 ? (!even && y != sh - 1) : (even && y != 0);
+        ya = y - 1; yb = y + 1;             /* above, below */
+        /* the reference assumes an even line count; for an odd one, keeping odd lines, its last line would read
+         * past the image: that read is defined here (and in the device code) as the last line */
+        if (yb > sh - 1) yb = sh - 1;
+    }
+    fklo_val a, b;
+    int rc;
+    if (!average) {
+        if ((rc = read_tap(r, x, y, &a))) return rc;
+        out->elem = FKLO_F32;
+        out->cn = a.cn;
+        for (int c = 0; c < a.cn; ++c) out->f[c] = chan_as_float(&a, c) * 1.f;
+        return FKLO_OK;
+    }
+    if ((rc = read_tap(r, x, ya, &a))) return rc;
+    if ((rc = read_tap(r, x, yb, &b))) return rc;
+    out->elem = FKLO_F32;
+    out->cn = a.cn;
+    for (int c = 0; c < a.cn; ++c) {
+        if (a.elem == FKLO_U8) out->f[c] = (float)((int)a.u[c] + (int)b.u[c] + 1) * 0.5f;
+        else out->f[c] = ((a.f[c] + b.f[c]) + 1.f) * 0.5f;
+    }
+    return FKLO_OK;
+}
+
 /* BatchRead<CONDITIONAL_WITH_DEFAULT>::exec, FK/core/execution_model/operation_model/batch_operations.h:262-273:
  * planes at or beyond usedPlanes return params.default_value, whose type is the plane operation's output type
  * (float_<cn> after a resize, the tap type after fused tap operations, else the element type). */
@@ -409,6 +446,7 @@ int fklo_execute(int32_t n_planes, const fklo_read *reads,
                 int rc = FKLO_OK;
                 if (r->use_default) read_default(r, &v);
                 else if (r->warp) rc = read_warped(r, x, y, &v);
+                else if (r->deinterlace) rc = read_deinterlaced(r, x, y, &v);
                 else rc = r->has_resize ? read_resized(r, &rp, x, y, &v) : read_tap(r, x, y, &v);
                 if (rc) return rc;
                 for (int i = 0; i < n_ops; ++i) {

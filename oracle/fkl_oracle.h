@@ -86,6 +86,7 @@ typedef struct {
     float def[4];            /* this plane is def, typed like the read's output, and nothing is read             */
     int32_t warp;            /* 0 none, 1 Warping<Affine>, 2 Warping<Perspective>; output grid dst_w x dst_h,     */
     float warp_m[9];         /* row-major transform (affine uses the first two rows); excludes has_resize         */
+    int32_t deinterlace;     /* 0 none, 1 Deinterlace<BLEND>, 2 <INTER_LINEAR> keeping even lines, 3 keeping odd   */
 } fklo_read;
 
 typedef struct {

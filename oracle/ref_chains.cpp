@@ -15,6 +15,7 @@
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
 #include <fused_kernel/algorithms/image_processing/warping.h>
+#include <fused_kernel/algorithms/image_processing/deinterlace.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
@@ -237,6 +238,20 @@ int fklref_batch_default_cast_mul_b4(const uint8_t* const* srcs, int w, int h, i
 int fklref_warp_u8x3(const uint8_t* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh, float* out) {
     return perspective ? warp_u8x3<WarpType::Perspective>(src, w, h, pitch, m, dw, dh, out)
                        : warp_u8x3<WarpType::Affine>(src, w, h, pitch, m, dw, dh, out);
+}
+
+// Deinterlace of a uchar3 image into a float3 image: mode 1 BLEND, 2 INTER_LINEAR keeping even lines, 3 keeping odd.
+int fklref_deinterlace_u8x3(const uint8_t* src, int w, int h, int pitch, int mode, float* out) {
+    CpuStream stream;
+    const auto in = wrap2d<uchar3>(src, w, h, pitch);
+    Ptr2D<float3> o(reinterpret_cast<float3*>(out), uint(w), uint(h), uint(w) * uint(sizeof(float3)), MemType::Host, 0);
+    const auto read = PerThreadRead<ND::_2D, uchar3>::build(in.ptr());
+    const auto write = PerThreadWrite<ND::_2D, float3>::build(o.ptr());
+    if (mode == 1) executeOperations<CpuDPP>(stream, read.then(Deinterlace<DeinterlaceType::BLEND>::build()), write);
+    else executeOperations<CpuDPP>(stream, read.then(Deinterlace<DeinterlaceType::INTER_LINEAR>::build(
+                                               DeinterlaceParameters<DeinterlaceType::INTER_LINEAR>{mode == 2})), write);
+    stream.sync();
+    return 0;
 }
 
 int fklref_batch_muladd_sat_b4(const uint8_t* const* srcs, int w, int h, int pitch, const float* mul,

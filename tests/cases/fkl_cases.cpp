@@ -13,6 +13,7 @@
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
 #include <fused_kernel/algorithms/image_processing/warping.h>
+#include <fused_kernel/algorithms/image_processing/deinterlace.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
@@ -178,6 +179,20 @@ void warp_image(void* stream_, const void* src, int w, int h, int pitch, const f
     for (int rep = 0; rep < g_reps; ++rep)
         executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, T>::build(in.ptr()).then(Warping<WT>::build(params)),
                                           PerThreadWrite<ND::_2D, O>::build(o.ptr()));
+}
+
+// Deinterlace: mode 1 BLEND, 2 INTER_LINEAR keeping even lines, 3 keeping odd lines.
+template <typename T, typename O> void deinterlace_image(void* stream_, const void* src, int w, int h, int pitch, int mode, void* out, int out_pitch) {
+    Stream stream(stream_);
+    const auto in = dev2d<T>(src, w, h, pitch);
+    const auto o = dev2d<O>(out, w, h, out_pitch);
+    const auto read = PerThreadRead<ND::_2D, T>::build(in.ptr());
+    const auto write = PerThreadWrite<ND::_2D, O>::build(o.ptr());
+    for (int rep = 0; rep < g_reps; ++rep) {
+        if (mode == 1) executeOperations<TransformDPP<>>(stream, read.then(Deinterlace<DeinterlaceType::BLEND>::build()), write);
+        else executeOperations<TransformDPP<>>(stream, read.then(Deinterlace<DeinterlaceType::INTER_LINEAR>::build(
+                                                          DeinterlaceParameters<DeinterlaceType::INTER_LINEAR>{mode == 2})), write);
+    }
 }
 
 extern "C" {
@@ -362,6 +377,13 @@ int fklcase_warp_f32(void* stream, const float* src, int w, int h, int pitch, co
         if (perspective) warp_image<WarpType::Perspective, float, float>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
         else warp_image<WarpType::Affine, float, float>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
     });
+}
+
+int fklcase_deinterlace_u8x3(void* stream, const uint8_t* src, int w, int h, int pitch, int mode, float* out, int out_pitch) {
+    return guarded([&] { deinterlace_image<uchar3, float3>(stream, src, w, h, pitch, mode, out, out_pitch); });
+}
+int fklcase_deinterlace_f32(void* stream, const float* src, int w, int h, int pitch, int mode, float* out, int out_pitch) {
+    return guarded([&] { deinterlace_image<float, float>(stream, src, w, h, pitch, mode, out, out_pitch); });
 }
 
 // Single-operation chains for the exhaustive numeric tests.

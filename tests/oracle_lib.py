@@ -36,6 +36,7 @@ class Read(C.Structure):
         ("n_tap_ops", C.c_int32), ("tap_ops", C.POINTER(Op)),
         ("use_default", C.c_int32), ("def_", C.c_float * 4),
         ("warp", C.c_int32), ("warp_m", C.c_float * 9),
+        ("deinterlace", C.c_int32),
     ]
 
 
@@ -278,6 +279,27 @@ def ref_warp_u8x3(src, matrix, dst, perspective):
     m[: (9 if perspective else 6)] = np.asarray(matrix, np.float32).ravel()
     rc = ref().fklref_warp_u8x3(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], _f32p(m), int(bool(perspective)),
                                 dw, dh, C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
+DEINTERLACE_BLEND, DEINTERLACE_LINEAR_EVEN, DEINTERLACE_LINEAR_ODD = 1, 2, 3
+
+
+def oracle_deinterlace(src, cn, mode):
+    """Deinterlace of an (H,W[,cn]) u8/f32 image into a float image of the same shape."""
+    h, w = src.shape[:2]
+    out = np.zeros((h, w, cn) if cn > 1 else (h, w), np.float32)
+    r = read_2d(src, cn)
+    r.deinterlace = mode
+    execute([r], [], [write(WRITE_2D, out, cn, w, h)])
+    return out
+
+
+def ref_deinterlace_u8x3(src, mode):
+    h, w = src.shape[:2]
+    out = np.zeros((h, w, 3), np.float32)
+    rc = ref().fklref_deinterlace_u8x3(C.c_void_p(_ptr(src)), w, h, src.strides[0], int(mode), C.c_void_p(_ptr(out)))
     assert rc == 0
     return out
 

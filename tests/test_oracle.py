@@ -365,3 +365,25 @@ def test_warp_closed_forms():
     out = ol.oracle_warp(src, 3, [[1, 0, 4], [0, 1, -2]], (30, 20), False)   # dst (x,y) reads src (x+4, y-2)
     assert (out[2:, :26] == src[:18, 4:].astype(np.float32)).all()
     assert (out[:2] == 0).all() and (out[:, 26:] == 0).all()
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="reference CPU backend not built (needs the reference tree)")
+def test_deinterlace_matches_reference_backend():
+    rng = np.random.RandomState(5)
+    for shape in ((12, 17, 3), (11, 9, 3), (1, 4, 3), (2, 3, 3)):
+        src = rng.randint(0, 256, shape).astype(np.uint8)
+        for mode in (ol.DEINTERLACE_BLEND, ol.DEINTERLACE_LINEAR_EVEN, ol.DEINTERLACE_LINEAR_ODD):
+            if mode == ol.DEINTERLACE_LINEAR_ODD and shape[0] % 2:
+                continue   # outside the reference's domain: its last line would read past the image
+            assert ol.oracle_deinterlace(src, 3, mode).tobytes() == ol.ref_deinterlace_u8x3(src, mode).tobytes()
+
+
+def test_deinterlace_closed_forms():
+    """Rows r*10: BLEND gives ((r + r-1)*10 + 1)/2; INTER_LINEAR keeps one field and averages the neighbours of the other."""
+    src = np.repeat((np.arange(6, dtype=np.uint8) * 10)[:, None], 4, axis=1)
+    b = ol.oracle_deinterlace(src, 1, ol.DEINTERLACE_BLEND)
+    assert (b[0] == 0).all() and all((b[r] == ((2 * r - 1) * 10 + 1) * 0.5).all() for r in range(1, 6))
+    e = ol.oracle_deinterlace(src, 1, ol.DEINTERLACE_LINEAR_EVEN)
+    assert all((e[r] == r * 10).all() for r in (0, 2, 4, 5)) and all((e[r] == (2 * r * 10 + 1) * 0.5).all() for r in (1, 3))
+    o = ol.oracle_deinterlace(src, 1, ol.DEINTERLACE_LINEAR_ODD)
+    assert all((o[r] == r * 10).all() for r in (0, 1, 3, 5)) and all((o[r] == (2 * r * 10 + 1) * 0.5).all() for r in (2, 4))
