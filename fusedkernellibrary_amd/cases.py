@@ -193,3 +193,42 @@ def deinterlace(src, mode, out):
     is_u8 = src.element_size() == 1
     fn = cases().fklcase_deinterlace_u8x3 if is_u8 else cases().fklcase_deinterlace_f32
     _ok(fn(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * (1 if is_u8 else 4), int(mode), _p(out), out.stride(0) * 4))
+
+
+# ---- pixel formats and colour conversions (tests/cases/color_chains.h) ------------------------------------
+# pf / cd / cr / cp are the enumerator values of fk::PixelFormat, ColorDepth, ColorRange and ColorPrimitives.
+
+def _pitch(t):
+    return t.stride(0) * t.element_size()
+
+
+def yuv_to_rgb(pf, cr, cp, frame, width, height, out):
+    """frame: 2-D u8/i16 cuda tensor holding a width x height frame in pixel format pf; out (H,W,3) f32 cuda."""
+    _ok(cases().fklcase_yuv_to_rgb(_stream(), int(pf), int(cr), int(cp), _p(frame), int(width), int(height), _pitch(frame), _p(out), _pitch(out)))
+
+
+def rgb_to_yuv(pf, cr, cp, rgb, frame):
+    """rgb (H,W,3) u8/i16 cuda; frame: 2-D cuda tensor the chain stores the pixel-format frame into."""
+    _ok(cases().fklcase_rgb_to_yuv(_stream(), int(pf), int(cr), int(cp), _p(rgb), rgb.shape[1], rgb.shape[0], _pitch(rgb), _p(frame), _pitch(frame)))
+
+
+def yuv_resize(pf, frame, width, height, dst, scale, out):
+    """ReadYUV -> ConvertYUVToRGB -> bilinear resize to dst = (w, h) -> * scale; out (dh,dw,3) f32 cuda."""
+    _ok(cases().fklcase_yuv_resize(_stream(), int(pf), _p(frame), int(width), int(height), _pitch(frame), int(dst[0]), int(dst[1]),
+                                   C.c_float(float(scale)), _p(out), _pitch(out)))
+
+
+def convert_depth(cd, cr, cp, to_rgb, src, out):
+    """src (H,W,3) u8/i16/f32 cuda pixels of depth cd -> ConvertYUVToRGB or ConvertRGBToYUV -> out (H,W,3) f32 cuda."""
+    _ok(cases().fklcase_convert_depth(_stream(), int(cd), int(cr), int(cp), int(bool(to_rgb)), _p(src), src.shape[1], src.shape[0], _pitch(src),
+                                      _p(out), _pitch(out)))
+
+
+def convert_code(which, src, out):
+    """ColorConversion<code> number `which` of the list in tests/cases/color_chains.h."""
+    _ok(cases().fklcase_convert_code(_stream(), int(which), _p(src), src.shape[1], src.shape[0], _pitch(src), _p(out), _pitch(out)))
+
+
+def normalize(which, src, out):
+    """NormalizePixel<uchar3, p8bit> (which = 0) or <ushort3, p10bit> (which = 1); out (H,W,3) f32 cuda."""
+    _ok(cases().fklcase_normalize(_stream(), int(which), _p(src), src.shape[1], src.shape[0], _pitch(src), _p(out), _pitch(out)))

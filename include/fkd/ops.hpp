@@ -600,23 +600,145 @@ template <class I, class O> struct SaturateCast {
     }
 };
 
-// ConvertYUVToRGB<p8bit, Full, bt709>: FK/algorithms/image_processing/color_conversion.h:150-174 with the
-// constexpr matrix of FK/algorithms/image_processing/itu_color.h:185-265 (all binary32) and
-// MxVFloat3<UnaryType>, FK/algorithms/basic_ops/algebraic.h:42-56: per row three products, (a+b)+c; no clamp.
-struct YUV2RGB709Full8 {
-    using In = Vec<u8, 3>; using Out = Vec<f32, 3>; using Params = Empty;
-    FKD_NAME("YUV2RGB709Full8")
+// Codes of the colour vocabulary: the enumerator values of fk::ColorDepth, fk::ColorRange and fk::ColorPrimitives
+// (FK/algorithms/image_processing/itu_color.h:26-29).
+enum : int { CD_P8 = 0, CD_P10 = 1, CD_P12 = 2, CD_FN8 = 3, CD_FN10 = 4, CD_FN12 = 5 };
+enum : int { CR_LIMITED = 0, CR_FULL = 1 };
+enum : int { CP_BT601 = 0, CP_BT709 = 1, CP_BT2020 = 2 };
+
+// Per-depth constants: sample type, largest value, the luma/chroma offsets and the limited-range spans.
+// FK/algorithms/image_processing/itu_color.h:103-183; the normalised-float depths divide the integer constants by the
+// integer depth's largest value, in binary32.
+template <int CD> struct DepthConsts;
+template <> struct DepthConsts<CD_P8>  { using base = u8;  static constexpr f32 max_v = 255.f,  luma = 16.f,  chroma = 128.f,  limit_y = 219.f,  limit_c = 224.f; };
+template <> struct DepthConsts<CD_P10> { using base = u16; static constexpr f32 max_v = 1023.f, luma = 64.f,  chroma = 512.f,  limit_y = 876.f,  limit_c = 896.f; };
+template <> struct DepthConsts<CD_P12> { using base = u16; static constexpr f32 max_v = 4095.f, luma = 256.f, chroma = 2048.f, limit_y = 3504.f, limit_c = 3584.f; };
+template <> struct DepthConsts<CD_FN8> {
+    using base = f32;
+    static constexpr f32 max_v = 1.f, luma = 16.f / 255.f, chroma = 128.f / 255.f, limit_y = 219.f / 255.f, limit_c = 224.f / 255.f;
+};
+template <> struct DepthConsts<CD_FN10> {
+    using base = f32;
+    static constexpr f32 max_v = 1.f, luma = 64.f / 1023.f, chroma = 512.f / 1023.f, limit_y = 876.f / 1023.f, limit_c = 896.f / 1023.f;
+};
+template <> struct DepthConsts<CD_FN12> {
+    using base = f32;
+    static constexpr f32 max_v = 1.f, luma = 256.f / 4095.f, chroma = 2048.f / 4095.f, limit_y = 3504.f / 4095.f, limit_c = 3584.f / 4095.f;
+};
+
+// computeMatrix<CR, CP, dir, CD>, FK/algorithms/image_processing/itu_color.h:185-265: the ITU matrix from the luma
+// weights Kr, Kb of the primaries (itu_color.h:150-158), then the limited-range scaling of the luma and chroma
+// columns (to RGB) or rows (to YCbCr).  All binary32, in the reference's expression order, evaluated at compile time.
+struct ColorMatrix { f32 m[9]; };
+template <int CD, int CR, int CP, bool TO_RGB> constexpr ColorMatrix color_matrix() {
+    static_assert(CP >= 0 && CP <= 2 && (CR == CR_LIMITED || CR == CR_FULL), "unknown colour primaries or range");
+    constexpr f32 Kr = CP == CP_BT601 ? 0.299f : (CP == CP_BT709 ? 0.2126f : 0.2627f);
+    constexpr f32 Kb = CP == CP_BT601 ? 0.114f : (CP == CP_BT709 ? 0.0722f : 0.0593f);
+    constexpr f32 Kg = 1.0f - Kr - Kb;
+    using D = DepthConsts<CD>;
+    ColorMatrix c{};
+    f32 (&m)[9] = c.m;
+    if constexpr (TO_RGB) {
+        m[0] = 1.0f; m[1] = 0.0f;                            m[2] = 2.0f * (1.0f - Kr);
+        m[3] = 1.0f; m[4] = -2.0f * Kb * (1.0f - Kb) / Kg;   m[5] = -2.0f * Kr * (1.0f - Kr) / Kg;
+        m[6] = 1.0f; m[7] = 2.0f * (1.0f - Kb);              m[8] = 0.0f;
+        if constexpr (CR == CR_LIMITED) {
+            constexpr f32 scale_y = D::max_v / D::limit_y, scale_c = D::max_v / D::limit_c;
+            for (int r = 0; r < 3; ++r) { m[3 * r] *= scale_y; m[3 * r + 1] *= scale_c; m[3 * r + 2] *= scale_c; }
+        }
+    } else {
+        m[0] = Kr;                          m[1] = Kg;                          m[2] = Kb;
+        m[3] = -Kr / (2.0f * (1.0f - Kb));  m[4] = -Kg / (2.0f * (1.0f - Kb));  m[5] = 0.5f;
+        m[6] = 0.5f;                        m[7] = -Kg / (2.0f * (1.0f - Kr));  m[8] = -Kb / (2.0f * (1.0f - Kr));
+        if constexpr (CR == CR_LIMITED) {
+            constexpr f32 scale_y = D::limit_y / D::max_v, scale_c = D::limit_c / D::max_v;
+            for (int i = 0; i < 3; ++i) { m[i] *= scale_y; m[3 + i] *= scale_c; m[6 + i] *= scale_c; }
+        }
+    }
+    return c;
+}
+// MxVFloat3<UnaryType>, FK/algorithms/basic_ops/algebraic.h:42-56: per row three products, (a + b) + c.
+FKD_DEV Vec<f32, 3> color_mxv(const ColorMatrix& c, f32 a, f32 b, f32 d) {
+    Vec<f32, 3> o;
+    o.x = (a * c.m[0] + b * c.m[1]) + d * c.m[2];
+    o.y = (a * c.m[3] + b * c.m[4]) + d * c.m[5];
+    o.z = (a * c.m[6] + b * c.m[7]) + d * c.m[8];
+    return o;
+}
+
+// ConvertYUVToRGB<CD, CR, CP>: FK/algorithms/image_processing/color_conversion.h:150-174.  (Y, Cb, Cr) minus the
+// depth's offsets (luma only for limited range) times the matrix; no clamp.
+template <int CD, int CR, int CP> struct YUV2RGB {
+    using In = Vec<typename DepthConsts<CD>::base, 3>; using Out = Vec<f32, 3>; using Params = Empty;
+    FKD_NAME("YUV2RGB<" + istr(CD) + "," + istr(CR) + "," + istr(CP) + ">")
     FKD_DEV static Out exec(const In& a, const Params&) {
-        constexpr f32 Kr = 0.2126f, Kb = 0.0722f;
-        constexpr f32 Kg = 1.0f - Kr - Kb;
-        constexpr f32 m00 = 1.0f, m01 = 0.0f, m02 = 2.0f * (1.0f - Kr);
-        constexpr f32 m10 = 1.0f, m11 = -2.0f * Kb * (1.0f - Kb) / Kg, m12 = -2.0f * Kr * (1.0f - Kr) / Kg;
-        constexpr f32 m20 = 1.0f, m21 = 2.0f * (1.0f - Kb), m22 = 0.0f;
-        const f32 y = f32(a.x), u = f32(a.y) - 128.0f, v = f32(a.z) - 128.0f;
+        using D = DepthConsts<CD>;
+        constexpr ColorMatrix c = color_matrix<CD, CR, CP, true>();
+        const f32 y = CR == CR_LIMITED ? f32(a.x) - D::luma : f32(a.x);
+        return color_mxv(c, y, f32(a.y) - D::chroma, f32(a.z) - D::chroma);
+    }
+};
+
+// ConvertRGBToYUV<CD, CR, CP>: FK/algorithms/image_processing/color_conversion.h:176-201.  Matrix times (R, G, B),
+// then the depth's offsets are added (luma only for limited range); no rounding, no clamp.
+template <int CD, int CR, int CP> struct RGB2YUV {
+    using In = Vec<typename DepthConsts<CD>::base, 3>; using Out = Vec<f32, 3>; using Params = Empty;
+    FKD_NAME("RGB2YUV<" + istr(CD) + "," + istr(CR) + "," + istr(CP) + ">")
+    FKD_DEV static Out exec(const In& a, const Params&) {
+        using D = DepthConsts<CD>;
+        constexpr ColorMatrix c = color_matrix<CD, CR, CP, false>();
+        Out o = color_mxv(c, f32(a.x), f32(a.y), f32(a.z));
+        if constexpr (CR == CR_LIMITED) o.x = o.x + D::luma;
+        o.y = o.y + D::chroma;
+        o.z = o.z + D::chroma;
+        return o;
+    }
+};
+
+// RGB2Gray<I, O, CCIR_601>: FK/algorithms/image_processing/color_conversion.h:49-80.  (R*0.299f + G*0.587f) + B*0.114f in
+// binary32, rounded to the nearest integer (ties to even) for EVERY output type: the reference tests is_unsigned,
+// then is_signed, and float is a signed type, so its float branch is never taken and a float output holds the
+// rounded value too.  Integer outputs then convert like a C cast of the rounded value.  A fourth input channel is
+// ignored.
+template <class I, class O> struct RGB2Gray {
+    static_assert(cn_v<I> >= 3 && cn_v<O> == 1, "three or four channels in, one out");
+    using In = I; using Out = O; using Params = Empty;
+    FKD_NAME("RGB2Gray<" + type_name<I>() + "," + type_name<O>() + ">")
+    FKD_DEV static O exec(const I& a, const Params&) {
+        const f32 l = (f32(a.x) * 0.299f + f32(a.y) * 0.587f) + f32(a.z) * 0.114f;
+        if constexpr (__is_same(O, f32) || __is_same(O, f64)) return O(__builtin_rintf(l));
+        else if constexpr (O(-1) < O(0)) return O(int(__builtin_rintf(l)));
+        else return O(u32(__builtin_rintf(l)));
+    }
+};
+
+// AddLast<I, O> with a run-time value and AddOpaqueAlpha<I, CD> (value = largest of the depth):
+// FK/algorithms/basic_ops/vector_ops.h:94-118, FK/algorithms/image_processing/color_conversion.h:81-93.
+template <class I> struct AddLast {
+    static_assert(cn_v<I> <= 3, "at most three channels in");
+    using In = I; using Out = vec_t<base_t<I>, cn_v<I> + 1>;
+    struct Params { base_t<I> last; };
+    FKD_NAME("AddLast<" + type_name<I>() + ">")
+    FKD_DEV static Out exec(const I& a, const Params& p) {
         Out o;
-        o.x = (y * m00 + u * m01) + v * m02;
-        o.y = (y * m10 + u * m11) + v * m12;
-        o.z = (y * m20 + u * m21) + v * m22;
+        chan<0>(o) = chan<0>(a);
+        if constexpr (cn_v<I> > 1) chan<1>(o) = chan<1>(a);
+        if constexpr (cn_v<I> > 2) chan<2>(o) = chan<2>(a);
+        chan<cn_v<I>>(o) = p.last;
+        return o;
+    }
+};
+
+// Discard<I, O>: the first cn<O> channels of the input.  FK/algorithms/basic_ops/vector_ops.h:22-41.
+template <class I, class O> struct Discard {
+    static_assert(cn_v<I> > cn_v<O> && __is_same(base_t<I>, base_t<O>), "fewer channels out, same sample type");
+    using In = I; using Out = O; using Params = Empty;
+    FKD_NAME("Discard<" + type_name<I>() + "," + type_name<O>() + ">")
+    FKD_DEV static O exec(const I& a, const Params&) {
+        O o;
+        chan<0>(o) = chan<0>(a);
+        if constexpr (cn_v<O> > 1) chan<1>(o) = chan<1>(a);
+        if constexpr (cn_v<O> > 2) chan<2>(o) = chan<2>(a);
         return o;
     }
 };
@@ -831,13 +953,14 @@ template <class T> struct Read3D {
 #endif
 };
 
-// ReadYUV<NV12>: FK/algorithms/image_processing/color_conversion.h:219-238.  Y from the luma plane, (U,V) from
-// element x>>1 of chroma row y>>1; chroma base = data + pitch*height.
-struct ReadNV12 {
+// ReadYUV<NV12> and ReadYUV<NV21>: FK/algorithms/image_processing/color_conversion.h:219-253.  Y from the luma
+// plane, the chroma pair from element x>>1 of chroma row y>>1; chroma base = data + pitch*height.  NV12 stores the
+// pair as (U,V), NV21 as (V,U) (template argument VU); the value is (Y,U,V) either way.
+template <bool VU> struct ReadNV {
     using Out = Vec<u8, 3>;
     using Params = RawNV12;
     static constexpr bool kTapCursor = true;
-    FKD_NAME("ReadNV12")
+    FKD_NAME(VU ? "ReadNV21" : "ReadNV12")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
@@ -845,8 +968,8 @@ struct ReadNV12 {
         Out o;
         o.x = *detail::gconst<u8>(p.data + size_t(y) * p.pitch + x);
         const FKD_GLOBAL u8* c = detail::gconst<u8>(p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch + 2 * (x >> 1));
-        o.y = c[0];
-        o.z = c[1];
+        o.y = c[VU ? 1 : 0];
+        o.z = c[VU ? 0 : 1];
         return o;
     }
     template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
@@ -876,8 +999,8 @@ struct ReadNV12 {
     FKD_DEV static Raw tap_value(const TapBits& b) {
         Out o;
         o.x = u8(b.y);
-        o.y = u8(b.uv & 0xffu);
-        o.z = u8(b.uv >> 8);
+        o.y = u8(VU ? b.uv >> 8 : b.uv & 0xffu);
+        o.z = u8(VU ? b.uv & 0xffu : b.uv >> 8);
         return o;
     }
     // Pixels x and x+1: two luma bytes in one access, and the dword at chroma pair x>>1, which holds the pair of
@@ -895,13 +1018,75 @@ struct ReadNV12 {
     }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) {
         first.x = u8(b.y & 0xffu);
-        first.y = u8(b.uv & 0xffu);
-        first.z = u8((b.uv >> 8) & 0xffu);
+        first.y = u8((b.uv >> (VU ? 8 : 0)) & 0xffu);
+        first.z = u8((b.uv >> (VU ? 0 : 8)) & 0xffu);
         const u32 uv = b.uv >> ((u32(r.x0 + x) & 1u) * 16u);
         second.x = u8((b.y >> 8) & 0xffu);
-        second.y = u8(uv & 0xffu);
-        second.z = u8((uv >> 8) & 0xffu);
+        second.y = u8((uv >> (VU ? 8 : 0)) & 0xffu);
+        second.z = u8((uv >> (VU ? 0 : 8)) & 0xffu);
     }
+#endif
+};
+using ReadNV12 = ReadNV<false>;
+using ReadNV21 = ReadNV<true>;
+
+// Pixel-format codes: the enumerator values of fk::PixelFormat (FK/algorithms/image_processing/itu_color.h:51).
+enum : int { PF_NV12 = 0, PF_NV21 = 1, PF_P010 = 3, PF_P210 = 6, PF_Y210 = 8, PF_UYVY = 10 };
+template <int PF> struct PixelLayout {
+    static_assert(PF == PF_NV12 || PF == PF_NV21 || PF == PF_P010 || PF == PF_P210 || PF == PF_Y210 || PF == PF_UYVY,
+                  "pixel format without a reader/writer in the reference (YV12, P016, P216, Y216) or whose reader does not compile there (Y416)");
+    static constexpr bool kSemiPlanar = PF == PF_NV12 || PF == PF_NV21 || PF == PF_P010 || PF == PF_P210;
+    static constexpr bool k420 = PF == PF_NV12 || PF == PF_NV21 || PF == PF_P010;
+    static constexpr bool kWide = PF == PF_P010 || PF == PF_P210 || PF == PF_Y210;     // 16-bit samples
+    static constexpr bool kSwapUV = PF == PF_NV21;
+};
+template <int PF> struct PixelBase { using type = u8; };
+template <> struct PixelBase<PF_P010> { using type = u16; };
+template <> struct PixelBase<PF_P210> { using type = u16; };
+template <> struct PixelBase<PF_Y210> { using type = u16; };
+
+// ReadYUV<P010 | P210 | Y210 | UYVY>: FK/algorithms/image_processing/color_conversion.h:219-268.  Semi-planar formats
+// (P010 4:2:0, P210 4:2:2): Y at (x, y) of the luma plane, the (U,V) pair at element x>>1 of chroma row y>>1 (4:2:0) or
+// y (4:2:2), chroma base = data + pitch*height.  Packed 4:2:2: the four-sample group x>>1 of row y holds U Y0 V Y1
+// (UYVY) or Y0 U Y1 V (Y210); even pixels take the first luma sample, odd ones the second.
+template <int PF> struct ReadYUV {
+    using L = PixelLayout<PF>;
+    using B = typename PixelBase<PF>::type;
+    using Out = Vec<B, 3>;
+    using Params = RawYUV;
+    static constexpr bool kTapCursor = false;
+    FKD_NAME("ReadYUV<" + istr(PF) + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return int(p.width); }
+    FKD_DEV static int height(const Params& p) { return int(p.height); }
+    FKD_DEV static Out exec(int x, int y, int, const Params& p) {
+        Out o;
+        if constexpr (L::kSemiPlanar) {
+            o.x = *detail::gconst<B>(p.data + size_t(y) * p.pitch + size_t(x) * sizeof(B));
+            const int cy = L::k420 ? y >> 1 : y;
+            const FKD_GLOBAL B* c = detail::gconst<B>(p.data + size_t(p.pitch) * p.height + size_t(cy) * p.pitch + size_t(x >> 1) * 2 * sizeof(B));
+            o.y = c[L::kSwapUV ? 1 : 0];
+            o.z = c[L::kSwapUV ? 0 : 1];
+        } else {
+            const FKD_GLOBAL B* g = detail::gconst<B>(p.data + size_t(y) * p.pitch + size_t(x >> 1) * 4 * sizeof(B));
+            const B s0 = g[0], s1 = g[1], s2 = g[2], s3 = g[3];
+            const bool even = (x & 1) == 0;
+            if constexpr (PF == PF_UYVY) { o.x = even ? s1 : s3; o.y = s0; o.z = s2; }
+            else { o.x = even ? s0 : s2; o.y = s1; o.z = s3; }
+        }
+        return o;
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+    }
+    FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // element-wise either way
+    // No tap cursor: a bilinear resize over this read takes its taps through exec().  The names below only let the
+    // wrappers that forward a cursor (Crop, FusedRead) be formed around this read.
+    using Raw = Out;
+    FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
+    struct TapRow {}; struct TapBits {}; struct PairBits {};
+    static constexpr bool kTapOverread = false, kTapPair = false;
 #endif
 };
 
@@ -1374,6 +1559,65 @@ template <class T> struct TensorSplit {
             detail::store_run_at<B, V>(reinterpret_cast<char*>(r.p + 3 * r.px), off, c);
         }
     }
+#endif
+};
+
+// WriteYUV<NV12 | NV21 | P010 | P210 | Y210 | UYVY>: FK/algorithms/image_processing/color_conversion.h:298-389.  The value
+// is (Y, U, V).  Semi-planar formats store Y at (x, y) and the chroma pair of a 2x2 (4:2:0) or 2x1 (4:2:2) block from
+// ONE pixel of the block: the top-left one for NV12, P010 and P210 (the reference stores from even x / even y only).
+// For NV21 the reference lets every pixel of the block store its own pair to the same place, so its result is the
+// block's last pixel in z, y, x order on the CPU backend and whichever thread comes last on a GPU; here it is always
+// the block's last pixel (odd x or the last column, odd y or the last row).  Packed 4:2:2 stores U, Y0, V from the
+// even pixel of a pair and Y1 from the odd one (UYVY: U Y0 V Y1; Y210: Y0 U Y1 V).
+template <int PF> struct WriteYUV {
+    using L = PixelLayout<PF>;
+    using B = typename PixelBase<PF>::type;
+    using In = Vec<B, 3>;
+    using Params = RawYUVOut;
+    FKD_NAME("WriteYUV<" + istr(PF) + ">")
+#if defined(FKD_DEVICE_CODE)
+    struct RowRef { char* row; char* crow; bool chroma_row; int last_x; };
+    FKD_DEV static RowRef row(int y, int, const Params& p) {
+        RowRef r;
+        char* d = reinterpret_cast<char*>(p.data);
+        r.row = d + size_t(y) * p.pitch;
+        r.crow = d + size_t(p.pitch) * p.height + size_t(L::k420 ? y >> 1 : y) * p.pitch;
+        if constexpr (!L::k420) r.chroma_row = true;
+        else if constexpr (L::kSwapUV) r.chroma_row = (y & 1) != 0 || y == int(p.height) - 1;
+        else r.chroma_row = (y & 1) == 0;
+        r.last_x = int(p.width) - 1;
+        return r;
+    }
+    FKD_DEV static void put(const RowRef& r, int x, const In& v) {
+        if constexpr (L::kSemiPlanar) {
+            *detail::gmut<B>(r.row + size_t(x) * sizeof(B)) = v.x;
+            const bool mine = L::kSwapUV ? ((x & 1) != 0 || x == r.last_x) : (x & 1) == 0;
+            if (r.chroma_row && mine) {
+                FKD_GLOBAL B* c = detail::gmut<B>(r.crow + size_t(x >> 1) * 2 * sizeof(B));
+                c[0] = L::kSwapUV ? v.z : v.y;
+                c[1] = L::kSwapUV ? v.y : v.z;
+            }
+        } else {
+            FKD_GLOBAL B* g = detail::gmut<B>(r.row + size_t(x >> 1) * 4 * sizeof(B));
+            if ((x & 1) == 0) {
+                if constexpr (PF == PF_UYVY) { g[0] = v.y; g[1] = v.x; g[2] = v.z; }
+                else { g[0] = v.x; g[1] = v.y; g[3] = v.z; }
+            } else {
+                if constexpr (PF == PF_UYVY) g[3] = v.x; else g[2] = v.x;
+            }
+        }
+    }
+    template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<In> (&v)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) put(r, x + i, v[i].v);
+    }
+    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { put(row(y, z, p), x, v); }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+        put_run<V>(row(y, z, p), x, v);
+    }
+    FKD_HD static bool rows_aligned(const Params&) { return true; }   // element-wise either way
+    using Plane = WriteYUV;
+    FKD_DEV static const Params& plane_params(const Params& p, int) { return p; }
 #endif
 };
 

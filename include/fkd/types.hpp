@@ -125,6 +125,12 @@ struct RawNV12 {
     const u8* data;
     u32 width, height, pitch;
 };
+// Any other pixel-format frame (semi-planar 16-bit, packed 4:2:2): same fields, width and height in pixels.
+using RawYUV = RawNV12;
+struct RawYUVOut {
+    u8* data;
+    u32 width, height, pitch;
+};
 
 #if defined(FKD_HOST_NAMES)
 template <class T> struct TypeName;

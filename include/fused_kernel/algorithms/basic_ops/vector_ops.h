@@ -1,4 +1,5 @@
-// VectorReorder<T, i0, i1, i2, i3>: out[c] = in[i_c].  Interface counterpart: FK/algorithms/basic_ops/vector_ops.h:43-56.
+// VectorReorder<T, i0, i1, i2, i3>: out[c] = in[i_c]; Discard<I, O>: the first cn<O> channels; AddLast<I, O>: one more
+// channel holding the parameter.  Interface counterpart: FK/algorithms/basic_ops/vector_ops.h:22-56, 94-118.
 #ifndef FK_AMD_VECTOR_OPS_H
 #define FK_AMD_VECTOR_OPS_H
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
@@ -10,7 +11,29 @@ template <typename T, int... Idx> struct VectorReorder : UnaryOperation<T, T, Ve
     static_assert(cn<T> >= 2, "Minimum number of channels to reorder: 2");
     static_assert(sizeof...(Idx) == cn<T>, "Wrong number of indexes for the vector type");
 };
+template <typename I, typename O> struct Discard : UnaryOperation<I, O, Discard<I, O>> {
+    using Parent = UnaryOperation<I, O, Discard<I, O>>;
+    FK_STATIC_STRUCT(Discard, Discard)
+    static_assert(cn<I> > cn<O>, "Output type should at least have one channel less");
+    static_assert(std::is_same_v<VBase<I>, VBase<O>>, "Base types should be the same");
+};
+template <typename I, typename O> struct AddLast : BinaryOperation<I, VBase<I>, O, AddLast<I, O>> {
+    using Parent = BinaryOperation<I, VBase<I>, O, AddLast<I, O>>;
+    FK_STATIC_STRUCT(AddLast, AddLast)
+    static_assert(cn<I> == cn<O> - 1, "Output type should have one channel more");
+    static_assert(std::is_same_v<VBase<I>, VBase<O>>, "Base types should be the same");
+};
 namespace amd {
+template <typename I, typename O> struct Lower<Discard<I, O>> {
+    static constexpr bool available = true;
+    using type = fkd::Discard<dev_t<I>, dev_t<O>>;
+    static typename type::Params params(const OperationData<Discard<I, O>>&) { return {}; }
+};
+template <typename I, typename O> struct Lower<AddLast<I, O>> {
+    static constexpr bool available = true;
+    using type = fkd::AddLast<dev_t<I>>;
+    static typename type::Params params(const OperationData<AddLast<I, O>>& d) { return typename type::Params{d.params}; }
+};
 template <typename T, int I0, int I1> struct Lower<VectorReorder<T, I0, I1>> {
     static constexpr bool available = true;
     using type = fkd::Reorder<dev_t<T>, I0, I1, 2, 3>;

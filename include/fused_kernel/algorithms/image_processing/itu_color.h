@@ -1,7 +1,7 @@
-// Colour-format vocabulary: colour spaces, ranges, primaries, depths and pixel formats, with the per-format
-// traits the NV12 reader needs.  Interface counterpart: FK/algorithms/image_processing/itu_color.h:21-101.
-// The YCbCr->RGB matrix itself is evaluated inside the device code (fkd::YUV2RGB709Full8), in binary32 and in
-// the reference's expression order (itu_color.h:185-265).
+// Colour-format vocabulary: colour spaces, ranges, primaries, depths and pixel formats, with the per-format traits
+// and per-depth constants.  Interface counterpart: FK/algorithms/image_processing/itu_color.h:21-183.
+// The YCbCr<->RGB matrices themselves are evaluated at compile time inside the device code (fkd::color_matrix), in
+// binary32 and in the reference's expression order (itu_color.h:185-265).
 #ifndef FK_AMD_ITU_COLOR_H
 #define FK_AMD_ITU_COLOR_H
 
@@ -41,6 +41,53 @@ template <> struct PixelFormatTraits<PixelFormat::NV21> {
     static constexpr size_t cn = 3;
     static constexpr ResolutionFactors rf{1.f, 1.5f};
 };
+template <> struct PixelFormatTraits<PixelFormat::YV12> {
+    static constexpr ColorSpace space = ColorSpace::YUV420;
+    static constexpr ColorDepth depth = ColorDepth::p8bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{1.f, 1.5f};
+};
+template <> struct PixelFormatTraits<PixelFormat::P010> {
+    static constexpr ColorSpace space = ColorSpace::YUV420;
+    static constexpr ColorDepth depth = ColorDepth::p10bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{1.f, 1.5f};
+};
+template <> struct PixelFormatTraits<PixelFormat::P210> {
+    static constexpr ColorSpace space = ColorSpace::YUV422;
+    static constexpr ColorDepth depth = ColorDepth::p10bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{1.f, 2.f};
+};
+template <> struct PixelFormatTraits<PixelFormat::Y210> {
+    static constexpr ColorSpace space = ColorSpace::YUV422;
+    static constexpr ColorDepth depth = ColorDepth::p10bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{2.f, 1.f};
+};
+template <> struct PixelFormatTraits<PixelFormat::Y416> {
+    static constexpr ColorSpace space = ColorSpace::YUV444;
+    static constexpr ColorDepth depth = ColorDepth::p12bit;
+    static constexpr size_t cn = 4;
+    static constexpr ResolutionFactors rf{4.f, 1.f};
+};
+template <> struct PixelFormatTraits<PixelFormat::UYVY> {
+    static constexpr ColorSpace space = ColorSpace::YUV422;
+    static constexpr ColorDepth depth = ColorDepth::p8bit;
+    static constexpr size_t cn = 3;
+    static constexpr ResolutionFactors rf{2.f, 1.f};
+};
+
+// Largest sample value of a depth (1.f for the normalised-float depths).
+template <ColorDepth CD> constexpr ColorDepthPixelBaseType<CD> maxDepthValue{};
+template <> inline constexpr uchar maxDepthValue<ColorDepth::p8bit>{255u};
+template <> inline constexpr ushort maxDepthValue<ColorDepth::p10bit>{1023u};
+template <> inline constexpr ushort maxDepthValue<ColorDepth::p12bit>{4095u};
+template <> inline constexpr float maxDepthValue<ColorDepth::fn8bit>{1.f};
+template <> inline constexpr float maxDepthValue<ColorDepth::fn10bit>{1.f};
+template <> inline constexpr float maxDepthValue<ColorDepth::fn12bit>{1.f};
+
+enum class ColorConversionDir { YCbCr2RGB, RGB2YCbCr };
 
 } // namespace fk
 #endif

@@ -9,12 +9,13 @@
 #include <math.h>
 #include <string.h>
 
-/* One value travelling through the chain: either uchar or float channels. */
+/* One value travelling through the chain: uchar, ushort or float channels. */
 typedef struct {
-    int elem; /* FKLO_U8 / FKLO_F32 */
+    int elem; /* FKLO_U8 / FKLO_F32 / FKLO_U16 */
     int cn;
     float f[4];
     uint8_t u[4];
+    uint16_t h[4];
 } fklo_val;
 
 /* ---- scalar helpers ---------------------------------------------------- */
@@ -56,6 +57,68 @@ uint8_t fklo_saturate_cast_u8(float s) {
     if (r >= 255.0f) return 255;
     if (r <= 0.0f) return 0;
     return (uint8_t)r;
+}
+
+uint16_t fklo_saturate_cast_u16(float s) {
+    if (s != s) return 0;
+    const float r = fklo_banker_round(s);
+    if (r >= 65535.0f) return 65535;
+    if (r <= 0.0f) return 0;
+    return (uint16_t)r;
+}
+
+/* maxDepthValue, subCoefficients, rangeLimits: FK/algorithms/image_processing/itu_color.h:103-183.  The normalised
+ * float depths divide the integer constants by the integer depth's largest value, in binary32. */
+typedef struct { float max_v, luma, chroma, limit_y, limit_c; } depth_consts;
+static int depth_constants(int depth, depth_consts *d) {
+    static const float tab[3][5] = {
+        {255.0f, 16.0f, 128.0f, 219.0f, 224.0f},
+        {1023.0f, 64.0f, 512.0f, 876.0f, 896.0f},
+        {4095.0f, 256.0f, 2048.0f, 3504.0f, 3584.0f}};
+    if (depth < 0 || depth > 5) return FKLO_EINVAL;
+    const float *t = tab[depth % 3];
+    if (depth < 3) {
+        d->max_v = t[0]; d->luma = t[1]; d->chroma = t[2]; d->limit_y = t[3]; d->limit_c = t[4];
+    } else {
+        d->max_v = 1.0f; d->luma = t[1] / t[0]; d->chroma = t[2] / t[0]; d->limit_y = t[3] / t[0]; d->limit_c = t[4] / t[0];
+    }
+    return FKLO_OK;
+}
+int fklo_depth_constants(int32_t depth, float *max_value, float *luma_offset, float *chroma_offset) {
+    depth_consts d;
+    if (depth_constants(depth, &d)) return FKLO_EINVAL;
+    *max_value = d.max_v; *luma_offset = d.luma; *chroma_offset = d.chroma;
+    return FKLO_OK;
+}
+
+/* computeMatrix<CR, CP, direction, CD>, FK/algorithms/image_processing/itu_color.h:185-265, with the luma weights
+ * of itu_color.h:150-158.  All arithmetic in binary32, same expression order; limited range scales the luma and
+ * chroma columns (to RGB) or rows (to YCbCr). */
+int fklo_color_matrix(int32_t depth, int32_t range, int32_t primaries, int32_t to_rgb, float m[9]) {
+    static const float kr[3] = {0.299f, 0.2126f, 0.2627f}, kb[3] = {0.114f, 0.0722f, 0.0593f};
+    depth_consts d;
+    if (depth_constants(depth, &d) || primaries < 0 || primaries > 2 || (range != FKLO_LIMITED && range != FKLO_FULL))
+        return FKLO_EINVAL;
+    const float Kr = kr[primaries], Kb = kb[primaries];
+    const float Kg = 1.0f - Kr - Kb;
+    if (to_rgb) {
+        m[0] = 1.0f; m[1] = 0.0f;                           m[2] = 2.0f * (1.0f - Kr);
+        m[3] = 1.0f; m[4] = -2.0f * Kb * (1.0f - Kb) / Kg;  m[5] = -2.0f * Kr * (1.0f - Kr) / Kg;
+        m[6] = 1.0f; m[7] = 2.0f * (1.0f - Kb);             m[8] = 0.0f;
+        if (range == FKLO_LIMITED) {
+            const float scale_y = d.max_v / d.limit_y, scale_c = d.max_v / d.limit_c;
+            for (int r = 0; r < 3; ++r) { m[3 * r] *= scale_y; m[3 * r + 1] *= scale_c; m[3 * r + 2] *= scale_c; }
+        }
+    } else {
+        m[0] = Kr;                          m[1] = Kg;                          m[2] = Kb;
+        m[3] = -Kr / (2.0f * (1.0f - Kb));  m[4] = -Kg / (2.0f * (1.0f - Kb));  m[5] = 0.5f;
+        m[6] = 0.5f;                        m[7] = -Kg / (2.0f * (1.0f - Kr));  m[8] = -Kb / (2.0f * (1.0f - Kr));
+        if (range == FKLO_LIMITED) {
+            const float scale_y = d.limit_y / d.max_v, scale_c = d.limit_c / d.max_v;
+            for (int i = 0; i < 3; ++i) { m[i] *= scale_y; m[3 + i] *= scale_c; m[6 + i] *= scale_c; }
+        }
+    }
+    return FKLO_OK;
 }
 
 /* computeMatrix<Full, bt709, YCbCr2RGB, p8bit>, FK/algorithms/image_processing/itu_color.h:185-265.
@@ -134,8 +197,19 @@ void fklo_compute_resize_params(int32_t src_w, int32_t src_h, int32_t dst_w, int
 /* ---- ops on values ----------------------------------------------------- */
 
 static float chan_as_float(const fklo_val *v, int c) {
-    return v->elem == FKLO_F32 ? v->f[c] : (float)v->u[c];
+    return v->elem == FKLO_F32 ? v->f[c] : (v->elem == FKLO_U16 ? (float)v->h[c] : (float)v->u[c]);
 }
+
+/* MxVFloat3<UnaryType>::exec, FK/algorithms/basic_ops/algebraic.h:42-56: per row three products, (a + b) + c. */
+static void mxv3(const float m[9], const float v[3], float out[3]) {
+    for (int r = 0; r < 3; ++r) {
+        const float a = v[0] * m[3 * r + 0];
+        const float b = v[1] * m[3 * r + 1];
+        const float c = v[2] * m[3 * r + 2];
+        out[r] = (a + b) + c;
+    }
+}
+static int depth_elem(int depth) { return depth == FKLO_P8 ? FKLO_U8 : (depth <= FKLO_P12 ? FKLO_U16 : FKLO_F32); }
 
 /* Add/Sub/Mul/Div<I,P,O,BinaryType>::exec, FK/algorithms/basic_ops/arithmetic.h:26-124 with the
  * channel-wise operators of FK/core/utils/vector_utils.h:508-563 (uchar op float -> float);
@@ -162,7 +236,68 @@ static int apply_op(const fklo_op *op, fklo_val *v) {
             if (s < 0 || s >= v->cn) return FKLO_EINVAL;
             v->f[c] = t.f[s];
             v->u[c] = t.u[s];
+            v->h[c] = t.h[s];
         }
+        return FKLO_OK;
+    }
+    /* ConvertYUVToRGB / ConvertRGBToYUV<CD, CR, CP>::exec, FK/algorithms/image_processing/color_conversion.h:150-201:
+     * offsets subtracted before (to RGB) or added after (to YCbCr) the matrix, luma offset only for limited range. */
+    case FKLO_YUV2RGB: case FKLO_RGB2YUV: {
+        depth_consts d;
+        float m[9];
+        const int to_rgb = op->code == FKLO_YUV2RGB;
+        if (fklo_color_matrix(op->idx[0], op->idx[1], op->idx[2], to_rgb, m) || depth_constants(op->idx[0], &d)) return FKLO_EINVAL;
+        if (v->elem != depth_elem(op->idx[0]) || v->cn != 3) return FKLO_ETYPE;
+        float in[3], out[3];
+        for (int c = 0; c < 3; ++c) in[c] = chan_as_float(v, c);
+        if (to_rgb) {
+            if (op->idx[1] == FKLO_LIMITED) in[0] = in[0] - d.luma;
+            in[1] = in[1] - d.chroma;
+            in[2] = in[2] - d.chroma;
+            mxv3(m, in, out);
+        } else {
+            mxv3(m, in, out);
+            if (op->idx[1] == FKLO_LIMITED) out[0] = out[0] + d.luma;
+            out[1] = out[1] + d.chroma;
+            out[2] = out[2] + d.chroma;
+        }
+        for (int c = 0; c < 3; ++c) v->f[c] = out[c];
+        v->elem = FKLO_F32;
+        return FKLO_OK;
+    }
+    /* RGB2Gray<I, O, CCIR_601>::exec, color_conversion.h:49-80: (R*0.299f + G*0.587f) + B*0.114f through nearbyint
+     * (ties to even) and a plain conversion to O.  That includes float outputs: the branch order is is_unsigned,
+     * is_signed, is_floating_point, and float is signed. */
+    case FKLO_RGB2GRAY: {
+        if (v->cn < 3) return FKLO_ETYPE;
+        const float l = (chan_as_float(v, 0) * 0.299f + chan_as_float(v, 1) * 0.587f) + chan_as_float(v, 2) * 0.114f;
+        v->cn = 1;
+        v->elem = op->idx[0];
+        if (v->elem == FKLO_F32) v->f[0] = nearbyintf(l);
+        else if (v->elem == FKLO_U8) v->u[0] = (uint8_t)(unsigned)nearbyintf(l);
+        else if (v->elem == FKLO_U16) v->h[0] = (uint16_t)(unsigned)nearbyintf(l);
+        else return FKLO_ETYPE;
+        return FKLO_OK;
+    }
+    /* AddLast<I, O>::exec, FK/algorithms/basic_ops/vector_ops.h:94-118 (AddOpaqueAlpha: color_conversion.h:81-93). */
+    case FKLO_ADD_LAST: {
+        if (v->cn > 3) return FKLO_ETYPE;
+        if (v->elem == FKLO_F32) v->f[v->cn] = op->p[0];
+        else if (v->elem == FKLO_U8) v->u[v->cn] = (uint8_t)op->p[0];
+        else v->h[v->cn] = (uint16_t)op->p[0];
+        v->cn += 1;
+        return FKLO_OK;
+    }
+    /* Discard<I, O>::exec, FK/algorithms/basic_ops/vector_ops.h:22-41. */
+    case FKLO_DISCARD: {
+        if (op->idx[0] < 1 || op->idx[0] >= v->cn) return FKLO_ETYPE;
+        v->cn = op->idx[0];
+        return FKLO_OK;
+    }
+    case FKLO_SATCAST_U16: {
+        if (v->elem != FKLO_F32) return FKLO_ETYPE;
+        for (int c = 0; c < v->cn; ++c) v->h[c] = fklo_saturate_cast_u16(v->f[c]);
+        v->elem = FKLO_U16;
         return FKLO_OK;
     }
     case FKLO_SATCAST_U8: {
@@ -172,8 +307,8 @@ static int apply_op(const fklo_op *op, fklo_val *v) {
         return FKLO_OK;
     }
     case FKLO_CAST_F32: {
-        if (v->elem == FKLO_U8) {
-            for (int c = 0; c < v->cn; ++c) v->f[c] = (float)v->u[c];
+        if (v->elem != FKLO_F32) {
+            for (int c = 0; c < v->cn; ++c) v->f[c] = chan_as_float(v, c);
             v->elem = FKLO_F32;
         }
         return FKLO_OK;
@@ -195,15 +330,53 @@ static int apply_op(const fklo_op *op, fklo_val *v) {
  * FK/core/data/rawptr.h:202-213: address = data + y*pitch + x*sizeof(T).
  * ReadYUV<NV12>::exec, FK/algorithms/image_processing/color_conversion.h:219-238: Y at (x,y) of the
  * luma plane; (U,V) at element x>>1 of chroma row y>>1, chroma base = data + pitch*height. */
+static uint16_t load_u16(const uint8_t *p) { uint16_t v; memcpy(&v, p, 2); return v; }
+static int read_is_pixel_format(const fklo_read *r) { return r->kind != FKLO_READ_2D; }
+static int pixel_format_elem(int kind) {
+    return (kind == FKLO_READ_P010 || kind == FKLO_READ_P210 || kind == FKLO_READ_Y210) ? FKLO_U16 : FKLO_U8;
+}
 static void read_source(const fklo_read *r, int x, int y, fklo_val *out) {
     const uint8_t *base = (const uint8_t *)r->data;
-    if (r->kind == FKLO_READ_NV12) {
+    if (r->kind == FKLO_READ_NV12 || r->kind == FKLO_READ_NV21) {
+        /* color_conversion.h:219-253; NV21 stores the pair as (V,U) and still yields (Y,U,V) */
+        const int vu = r->kind == FKLO_READ_NV21;
         out->elem = FKLO_U8;
         out->cn = 3;
         out->u[0] = base[(int64_t)y * r->pitch + x];
         const uint8_t *chroma = base + (int64_t)r->pitch * r->height + (int64_t)(y >> 1) * r->pitch;
-        out->u[1] = chroma[2 * (x >> 1) + 0];
-        out->u[2] = chroma[2 * (x >> 1) + 1];
+        out->u[1] = chroma[2 * (x >> 1) + (vu ? 1 : 0)];
+        out->u[2] = chroma[2 * (x >> 1) + (vu ? 0 : 1)];
+        return;
+    }
+    if (r->kind == FKLO_READ_P010 || r->kind == FKLO_READ_P210) {
+        /* color_conversion.h:219-238 with ushort samples; 4:2:0 halves the chroma row index, 4:2:2 does not */
+        const int cy = r->kind == FKLO_READ_P010 ? y >> 1 : y;
+        out->elem = FKLO_U16;
+        out->cn = 3;
+        out->h[0] = load_u16(base + (int64_t)y * r->pitch + 2 * (int64_t)x);
+        const uint8_t *chroma = base + (int64_t)r->pitch * r->height + (int64_t)cy * r->pitch + 4 * (int64_t)(x >> 1);
+        out->h[1] = load_u16(chroma);
+        out->h[2] = load_u16(chroma + 2);
+        return;
+    }
+    if (r->kind == FKLO_READ_Y210) {
+        /* color_conversion.h:254-266: group x>>1 of row y is Y0 U Y1 V */
+        const uint8_t *g = base + (int64_t)y * r->pitch + 8 * (int64_t)(x >> 1);
+        out->elem = FKLO_U16;
+        out->cn = 3;
+        out->h[0] = load_u16(g + ((x & 1) == 0 ? 0 : 4));
+        out->h[1] = load_u16(g + 2);
+        out->h[2] = load_u16(g + 6);
+        return;
+    }
+    if (r->kind == FKLO_READ_UYVY) {
+        /* color_conversion.h:254-266: group x>>1 of row y is U Y0 V Y1 */
+        const uint8_t *g = base + (int64_t)y * r->pitch + 4 * (int64_t)(x >> 1);
+        out->elem = FKLO_U8;
+        out->cn = 3;
+        out->u[0] = g[(x & 1) == 0 ? 1 : 3];
+        out->u[1] = g[0];
+        out->u[2] = g[2];
         return;
     }
     out->elem = r->elem;
@@ -212,6 +385,9 @@ static void read_source(const fklo_read *r, int x, int y, fklo_val *out) {
     if (r->elem == FKLO_U8) {
         const uint8_t *p = row + (int64_t)x * r->cn;
         for (int c = 0; c < r->cn; ++c) out->u[c] = p[c];
+    } else if (r->elem == FKLO_U16) {
+        const uint8_t *p = row + 2 * (int64_t)x * r->cn;
+        for (int c = 0; c < r->cn; ++c) out->h[c] = load_u16(p + 2 * c);
     } else {
         const float *p = (const float *)row + (int64_t)x * r->cn;
         for (int c = 0; c < r->cn; ++c) out->f[c] = p[c];
@@ -245,7 +421,7 @@ static int read_resized(const fklo_read *r, const fklo_resize_params *rp, int x,
         if (!(x >= rp->x1 && x <= rp->x2 && y >= rp->y1 && y <= rp->y2)) {
             /* params.defaultValue: float_<cn> of the tap type (resize.h:74) */
             out->elem = FKLO_F32;
-            out->cn = r->kind == FKLO_READ_NV12 ? 3 : r->cn;
+            out->cn = read_is_pixel_format(r) ? 3 : r->cn;
             for (int c = 0; c < out->cn; ++c) out->f[c] = r->bg[c];
             return FKLO_OK;
         }
@@ -280,31 +456,68 @@ static int read_resized(const fklo_read *r, const fklo_resize_params *rp, int x,
 /* PerThreadWrite<_2D,T>, TensorWrite<T>, TensorSplit<T>: FK/algorithms/basic_ops/memory_operations.h:84-107,
  * 159-179, 181-212; PtrAccessor<_3D>::point, FK/core/data/rawptr.h:215-226 (plane stride =
  * plane_pitch*color_planes with plane_pitch = pitch*height). */
+static const void *val_chan(const fklo_val *v, int c) {
+    return v->elem == FKLO_F32 ? (const void *)&v->f[c] : (v->elem == FKLO_U16 ? (const void *)&v->h[c] : (const void *)&v->u[c]);
+}
+static void store_u16(uint8_t *p, uint16_t s) { memcpy(p, &s, 2); }
+
+/* WriteYUV<PF>::exec, FK/algorithms/image_processing/color_conversion.h:298-389.  The value is (Y,U,V).  Semi-planar
+ * formats store Y per pixel and the chroma pair from the pixels the reference lets store it: even x and even y
+ * (4:2:0) or even x (4:2:2) for NV12/P010/P210; every pixel for NV21, where the z,y,x loop of the CPU backend leaves
+ * the pair of the block's last pixel.  Packed 4:2:2: the even pixel stores U, Y0, V, the odd one Y1. */
+static int write_yuv(const fklo_write *w, int x, int y, const fklo_val *v) {
+    uint8_t *base = (uint8_t *)w->data;
+    const int fmt = w->yuv_format;
+    if (v->cn != 3 || v->elem != pixel_format_elem(fmt)) return FKLO_ETYPE;
+    if (fmt == FKLO_READ_NV12 || fmt == FKLO_READ_NV21) {
+        base[(int64_t)y * w->pitch + x] = v->u[0];
+        uint8_t *c = base + (int64_t)w->pitch * w->height + (int64_t)(y >> 1) * w->pitch + 2 * (int64_t)(x >> 1);
+        if (fmt == FKLO_READ_NV21) { c[0] = v->u[2]; c[1] = v->u[1]; }
+        else if ((x & 1) == 0 && (y & 1) == 0) { c[0] = v->u[1]; c[1] = v->u[2]; }
+        return FKLO_OK;
+    }
+    if (fmt == FKLO_READ_P010 || fmt == FKLO_READ_P210) {
+        store_u16(base + (int64_t)y * w->pitch + 2 * (int64_t)x, v->h[0]);
+        const int cy = fmt == FKLO_READ_P010 ? y >> 1 : y;
+        uint8_t *c = base + (int64_t)w->pitch * w->height + (int64_t)cy * w->pitch + 4 * (int64_t)(x >> 1);
+        if ((x & 1) == 0 && (fmt == FKLO_READ_P210 || (y & 1) == 0)) { store_u16(c, v->h[1]); store_u16(c + 2, v->h[2]); }
+        return FKLO_OK;
+    }
+    if (fmt == FKLO_READ_UYVY) {
+        uint8_t *g = base + (int64_t)y * w->pitch + 4 * (int64_t)(x >> 1);
+        if ((x & 1) == 0) { g[0] = v->u[1]; g[1] = v->u[0]; g[2] = v->u[2]; }
+        else g[3] = v->u[0];
+        return FKLO_OK;
+    }
+    if (fmt == FKLO_READ_Y210) {
+        uint8_t *g = base + (int64_t)y * w->pitch + 8 * (int64_t)(x >> 1);
+        if ((x & 1) == 0) { store_u16(g, v->h[0]); store_u16(g + 2, v->h[1]); store_u16(g + 6, v->h[2]); }
+        else store_u16(g + 4, v->h[0]);
+        return FKLO_OK;
+    }
+    return FKLO_EINVAL;
+}
+
 static int write_value(const fklo_write *w, int x, int y, int z, const fklo_val *v) {
+    if (w->kind == FKLO_WRITE_YUV) return write_yuv(w, x, y, v);
     if (v->elem != w->elem || v->cn != w->cn) return FKLO_ETYPE;
     uint8_t *base = (uint8_t *)w->data;
-    const int64_t esz = w->elem == FKLO_U8 ? 1 : 4;
+    const int64_t esz = w->elem == FKLO_U8 ? 1 : (w->elem == FKLO_U16 ? 2 : 4);
     if (w->kind == FKLO_WRITE_2D) {
         uint8_t *p = base + (int64_t)y * w->pitch + (int64_t)x * esz * w->cn;
-        if (w->elem == FKLO_U8) memcpy(p, v->u, (size_t)w->cn);
-        else memcpy(p, v->f, (size_t)w->cn * 4);
+        for (int c = 0; c < w->cn; ++c) memcpy(p + c * esz, val_chan(v, c), (size_t)esz);
         return FKLO_OK;
     }
     const int64_t plane_pitch = (int64_t)w->pitch * w->height;
     uint8_t *row = base + plane_pitch * w->color_planes * z + (int64_t)y * w->pitch;
     if (w->kind == FKLO_TENSOR_WRITE) {
         uint8_t *p = row + (int64_t)x * esz * w->cn;
-        if (w->elem == FKLO_U8) memcpy(p, v->u, (size_t)w->cn);
-        else memcpy(p, v->f, (size_t)w->cn * 4);
+        for (int c = 0; c < w->cn; ++c) memcpy(p + c * esz, val_chan(v, c), (size_t)esz);
         return FKLO_OK;
     }
     if (w->kind == FKLO_TENSOR_SPLIT) {
         const int64_t plane_px = (int64_t)w->width * w->height;
-        for (int c = 0; c < w->cn; ++c) {
-            uint8_t *p = row + ((int64_t)x + c * plane_px) * esz;
-            if (w->elem == FKLO_U8) *p = v->u[c];
-            else memcpy(p, &v->f[c], 4);
-        }
+        for (int c = 0; c < w->cn; ++c) memcpy(row + ((int64_t)x + c * plane_px) * esz, val_chan(v, c), (size_t)esz);
         return FKLO_OK;
     }
     return FKLO_EINVAL;
@@ -331,7 +544,7 @@ static int read_warped(const fklo_read *r, int x, int y, fklo_val *out) {
     int sw, sh;
     read_extent(r, &sw, &sh);
     out->elem = FKLO_F32;
-    out->cn = r->kind == FKLO_READ_NV12 ? 3 : r->cn;
+    out->cn = read_is_pixel_format(r) ? 3 : r->cn;
     if (!(sx >= 0.f && sx < (float)sw && sy >= 0.f && sy < (float)sh)) {
         for (int c = 0; c < out->cn; ++c) out->f[c] = 0.f;
         return FKLO_OK;
@@ -386,6 +599,7 @@ static int read_deinterlaced(const fklo_read *r, int x, int y, fklo_val *out) {
     out->cn = a.cn;
     for (int c = 0; c < a.cn; ++c) {
         if (a.elem == FKLO_U8) out->f[c] = (float)((int)a.u[c] + (int)b.u[c] + 1) * 0.5f;
+        else if (a.elem == FKLO_U16) out->f[c] = (float)((int)a.h[c] + (int)b.h[c] + 1) * 0.5f;
         else out->f[c] = ((a.f[c] + b.f[c]) + 1.f) * 0.5f;
     }
     return FKLO_OK;
@@ -395,8 +609,8 @@ static int read_deinterlaced(const fklo_read *r, int x, int y, fklo_val *out) {
  * planes at or beyond usedPlanes return params.default_value, whose type is the plane operation's output type
  * (float_<cn> after a resize, the tap type after fused tap operations, else the element type). */
 static void read_default(const fklo_read *r, fklo_val *out) {
-    int cn = r->kind == FKLO_READ_NV12 ? 3 : r->cn;
-    int elem = r->kind == FKLO_READ_NV12 ? FKLO_U8 : r->elem;
+    int cn = read_is_pixel_format(r) ? 3 : r->cn;
+    int elem = read_is_pixel_format(r) ? pixel_format_elem(r->kind) : r->elem;
     if (r->n_tap_ops > 0 || r->has_resize) {
         /* find the type the read yields by running the tap operations on a dummy element */
         fklo_val probe;
@@ -412,6 +626,7 @@ static void read_default(const fklo_read *r, fklo_val *out) {
     out->cn = cn;
     for (int c = 0; c < cn; ++c) {
         if (elem == FKLO_F32) out->f[c] = r->def[c];
+        else if (elem == FKLO_U16) out->h[c] = (uint16_t)r->def[c];
         else out->u[c] = (uint8_t)r->def[c];
     }
 }

@@ -35,11 +35,16 @@
 extern "C" {
 #endif
 
-enum { FKLO_U8 = 0, FKLO_F32 = 1 };
+enum { FKLO_U8 = 0, FKLO_F32 = 1, FKLO_U16 = 2 };
 
 enum fklo_read_kind {
     FKLO_READ_2D = 0,   /* PerThreadRead<_2D,T>: pitched array of cn-channel elements */
-    FKLO_READ_NV12 = 1  /* ReadYUV<NV12>: luma plane + interleaved half-res chroma    */
+    FKLO_READ_NV12 = 1, /* ReadYUV<NV12>: luma plane + interleaved half-res chroma    */
+    FKLO_READ_NV21 = 2, /* ReadYUV<NV21>: as NV12 with the chroma pair stored (V,U)   */
+    FKLO_READ_P010 = 3, /* ReadYUV<P010>: NV12 layout with 16-bit samples             */
+    FKLO_READ_P210 = 4, /* ReadYUV<P210>: 16-bit samples, chroma rows at full height  */
+    FKLO_READ_Y210 = 5, /* ReadYUV<Y210>: packed 16-bit Y0 U Y1 V                     */
+    FKLO_READ_UYVY = 6  /* ReadYUV<UYVY>: packed 8-bit U Y0 V Y1                      */
 };
 
 enum fklo_aspect { FKLO_PRESERVE_AR = 0, FKLO_IGNORE_AR = 1 };
@@ -52,14 +57,26 @@ enum fklo_opcode {
     FKLO_REORDER = 5,          /* out[c] = in[idx[c]]  (BGR<->RGB is idx = 2,1,0)      */
     FKLO_SATCAST_U8 = 6,       /* float -> uchar: NaN->0, round-half-even, clamp       */
     FKLO_CAST_F32 = 7,         /* uchar -> float static_cast (no-op on float)          */
-    FKLO_YUV2RGB_709_FULL = 8  /* uchar3 (Y,U,V) -> float3 RGB, BT.709 full range 8bit */
+    FKLO_YUV2RGB_709_FULL = 8, /* uchar3 (Y,U,V) -> float3 RGB, BT.709 full range 8bit */
+    FKLO_YUV2RGB = 9,          /* ConvertYUVToRGB<depth, range, primaries>: idx[0..2]  */
+    FKLO_RGB2YUV = 10,         /* ConvertRGBToYUV<depth, range, primaries>: idx[0..2]  */
+    FKLO_RGB2GRAY = 11,        /* RGB2Gray<I, O>: idx[0] = element type of O           */
+    FKLO_ADD_LAST = 12,        /* one more channel holding p[0] (AddOpaqueAlpha)       */
+    FKLO_DISCARD = 13,         /* keep the first idx[0] channels                       */
+    FKLO_SATCAST_U16 = 14      /* float -> ushort: NaN->0, round-half-even, clamp      */
 };
 
 enum fklo_write_kind {
     FKLO_WRITE_2D = 0,      /* PerThreadWrite<_2D,T>; one fklo_write per plane when batched */
     FKLO_TENSOR_WRITE = 1,  /* TensorWrite<T>: AoS, plane z at z*plane_pitch*color_planes   */
-    FKLO_TENSOR_SPLIT = 2   /* TensorSplit<T>: planar, channel c at +c*width*height elems   */
+    FKLO_TENSOR_SPLIT = 2,  /* TensorSplit<T>: planar, channel c at +c*width*height elems   */
+    FKLO_WRITE_YUV = 3      /* WriteYUV<PF>: yuv_format names the layout (a fklo_read_kind) */
 };
+
+/* Values of fk::ColorDepth, fk::ColorRange, fk::ColorPrimitives (FK/algorithms/image_processing/itu_color.h:26-29). */
+enum { FKLO_P8 = 0, FKLO_P10 = 1, FKLO_P12 = 2, FKLO_FN8 = 3, FKLO_FN10 = 4, FKLO_FN12 = 5 };
+enum { FKLO_LIMITED = 0, FKLO_FULL = 1 };
+enum { FKLO_BT601 = 0, FKLO_BT709 = 1, FKLO_BT2020 = 2 };
 
 typedef struct {
     int32_t code;
@@ -69,9 +86,9 @@ typedef struct {
 
 typedef struct {
     int32_t kind;            /* fklo_read_kind */
-    int32_t elem;            /* FKLO_U8 / FKLO_F32 (READ_2D); NV12 is always U8 */
-    int32_t cn;              /* channels of one element (READ_2D); NV12 yields 3 */
-    int32_t width, height;   /* READ_2D: element grid; NV12: luma size */
+    int32_t elem;            /* FKLO_U8 / FKLO_F32 / FKLO_U16 (READ_2D); pixel formats fix their own */
+    int32_t cn;              /* channels of one element (READ_2D); pixel formats yield 3 */
+    int32_t width, height;   /* READ_2D: element grid; pixel formats: image size in pixels */
     int32_t pitch;           /* bytes per row */
     const void *data;
     int32_t has_crop;
@@ -96,6 +113,7 @@ typedef struct {
     void *data;
     int32_t width, height, planes, color_planes;
     int32_t pitch;           /* bytes per row */
+    int32_t yuv_format;      /* FKLO_WRITE_YUV: fklo_read_kind of the layout; width, height = image size in pixels */
 } fklo_write;
 
 typedef struct {
@@ -120,6 +138,10 @@ uint8_t fklo_saturate_cast_u8(float v);
 float fklo_banker_round(float v);
 float fklo_round_half_away(float v);
 void fklo_yuv2rgb_709_full_matrix(float m[9]);
+/* ccMatrix<range, primaries, direction, depth> (row major) and the offsets of the depth. */
+int fklo_color_matrix(int32_t depth, int32_t range, int32_t primaries, int32_t to_rgb, float m[9]);
+int fklo_depth_constants(int32_t depth, float *max_value, float *luma_offset, float *chroma_offset);
+uint16_t fklo_saturate_cast_u16(float v);
 void fklo_yuv2rgb_709_full(const uint8_t yuv[3], float rgb[3]);
 /* 4-tap bilinear of one channel given the four tap values already converted
  * to float; (sx, sy) is the source coordinate. */

@@ -24,6 +24,10 @@
 #include <cstdint>
 #include <utility>
 
+// Pixel-format and colour-conversion chains: the same text the GPU case drivers compile against this repository's
+// headers, compiled here against the reference's.
+#include "../tests/cases/color_chains.h"
+
 using namespace fk;
 using CpuDPP = TransformDPP<ParArch::CPU>;
 using CpuDPPTF = TransformDPP<ParArch::CPU, TF::ENABLED>;
@@ -321,6 +325,71 @@ int fklref_resize_params_par(int sw, int sh, int dw, int dh, int32_t* out4, floa
     const auto r = back.then(Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(dw, dh), float3{0.f, 0.f, 0.f}));
     out4[0] = r.params.x1; out4[1] = r.params.y1; out4[2] = r.params.x2; out4[3] = r.params.y2;
     f2[0] = r.params.src_conv_factors.x; f2[1] = r.params.src_conv_factors.y;
+    return 0;
+}
+
+} // extern "C"
+
+// ---- pixel formats and colour conversions (tests/cases/color_chains.h on the reference's CPU backend) ----------
+namespace {
+using RefColor = color_chains::Chains<CpuDPP, CpuStream>;
+template <int CD, int CR, int CP, int DIR> void color_matrix_of(float* m9) {
+    constexpr M3x3Float m = ccMatrix<ColorRange(CR), ColorPrimitives(CP), ColorConversionDir(DIR), ColorDepth(CD)>;
+    m9[0] = m.x.x; m9[1] = m.x.y; m9[2] = m.x.z;
+    m9[3] = m.y.x; m9[4] = m.y.y; m9[5] = m.y.z;
+    m9[6] = m.z.x; m9[7] = m.z.y; m9[8] = m.z.z;
+}
+using MatrixFn = void (*)(float*);
+template <size_t... I> MatrixFn matrix_fn(size_t i, std::index_sequence<I...>) {
+    static constexpr MatrixFn table[] = {&color_matrix_of<int(I / 12), int((I / 6) % 2), int((I / 2) % 3), int(I % 2)>...};
+    return table[i];
+}
+} // namespace
+
+extern "C" {
+
+int fklref_yuv_to_rgb(int pf, int cr, int cp, const void* src, int w, int h, int pitch, float* out, int out_pitch) {
+    CpuStream s;
+    const int rc = RefColor::yuv_to_rgb(s, MemType::Host, pf, cr, cp, src, w, h, pitch, out, out_pitch);
+    s.sync();
+    return rc;
+}
+int fklref_rgb_to_yuv(int pf, int cr, int cp, const void* src, int w, int h, int pitch, void* out, int out_pitch) {
+    CpuStream s;
+    const int rc = RefColor::rgb_to_yuv(s, MemType::Host, pf, cr, cp, src, w, h, pitch, out, out_pitch);
+    s.sync();
+    return rc;
+}
+int fklref_yuv_resize(int pf, const void* src, int w, int h, int pitch, int dw, int dh, float scale, float* out, int out_pitch) {
+    CpuStream s;
+    const int rc = RefColor::yuv_resize(s, MemType::Host, pf, src, w, h, pitch, dw, dh, scale, out, out_pitch);
+    s.sync();
+    return rc;
+}
+int fklref_convert_depth(int cd, int cr, int cp, int to_rgb, const void* src, int w, int h, int pitch, float* out, int out_pitch) {
+    CpuStream s;
+    const int rc = RefColor::convert_depth(s, MemType::Host, cd, cr, cp, to_rgb, src, w, h, pitch, out, out_pitch);
+    s.sync();
+    return rc;
+}
+int fklref_convert_code(int which, const void* src, int w, int h, int pitch, void* out, int out_pitch) {
+    CpuStream s;
+    const int rc = RefColor::convert_code(s, MemType::Host, which, src, w, h, pitch, out, out_pitch);
+    s.sync();
+    return rc;
+}
+int fklref_normalize(int which, const void* src, int w, int h, int pitch, float* out, int out_pitch) {
+    CpuStream s;
+    const int rc = RefColor::normalize(s, MemType::Host, which, src, w, h, pitch, out, out_pitch);
+    s.sync();
+    return rc;
+}
+// ccMatrix<range, primaries, direction, depth> as the reference computes it at compile time, row major.
+// to_rgb = 1 selects YCbCr2RGB.
+int fklref_color_matrix(int cd, int cr, int cp, int to_rgb, float* m9) {
+    if (cd < 0 || cd > 5 || cr < 0 || cr > 1 || cp < 0 || cp > 2) return 1;
+    const size_t dir = to_rgb ? size_t(ColorConversionDir::YCbCr2RGB) : size_t(ColorConversionDir::RGB2YCbCr);
+    matrix_fn(((size_t(cd) * 2 + size_t(cr)) * 3 + size_t(cp)) * 2 + dir, std::make_index_sequence<72>{})(m9);
     return 0;
 }
 

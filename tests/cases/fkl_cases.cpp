@@ -25,6 +25,8 @@
 #include <exception>
 #include <utility>
 
+#include "color_chains.h"   // pixel-format and colour-conversion chains, shared with the reference-backend harness
+
 using namespace fk;
 
 namespace {
@@ -417,6 +419,41 @@ int fklcase_saturate_f32_u8(void* stream_, const float* in, int w, int h, int pi
 }
 int fklcase_crop_swap_u8_b4(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, uint8_t* out) {
     return guarded([&] { crop_swap_u8<4>(stream, src, w, h, pitch, rects, out); });
+}
+
+} // extern "C"
+
+// ---- pixel formats and colour conversions (color_chains.h on the GPU) --------------------------------------------
+namespace {
+using GpuColor = color_chains::Chains<TransformDPP<>, Stream>;
+template <typename F> int guarded_rc(F body) {
+    int rc = 0;
+    const int g = guarded([&] { rc = body(); });
+    return g ? g : rc;
+}
+} // namespace
+
+extern "C" {
+
+int fklcase_yuv_to_rgb(void* stream_, int pf, int cr, int cp, const void* src, int w, int h, int pitch, float* out, int out_pitch) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::yuv_to_rgb(s, MemType::Device, pf, cr, cp, src, w, h, pitch, out, out_pitch); });
+}
+int fklcase_rgb_to_yuv(void* stream_, int pf, int cr, int cp, const void* src, int w, int h, int pitch, void* out, int out_pitch) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::rgb_to_yuv(s, MemType::Device, pf, cr, cp, src, w, h, pitch, out, out_pitch); });
+}
+int fklcase_yuv_resize(void* stream_, int pf, const void* src, int w, int h, int pitch, int dw, int dh, float scale, float* out,
+                       int out_pitch) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::yuv_resize(s, MemType::Device, pf, src, w, h, pitch, dw, dh, scale, out, out_pitch); });
+}
+int fklcase_convert_depth(void* stream_, int cd, int cr, int cp, int to_rgb, const void* src, int w, int h, int pitch, float* out,
+                          int out_pitch) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::convert_depth(s, MemType::Device, cd, cr, cp, to_rgb, src, w, h, pitch, out, out_pitch); });
+}
+int fklcase_convert_code(void* stream_, int which, const void* src, int w, int h, int pitch, void* out, int out_pitch) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::convert_code(s, MemType::Device, which, src, w, h, pitch, out, out_pitch); });
+}
+int fklcase_normalize(void* stream_, int which, const void* src, int w, int h, int pitch, float* out, int out_pitch) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::normalize(s, MemType::Device, which, src, w, h, pitch, out, out_pitch); });
 }
 
 } // extern "C"

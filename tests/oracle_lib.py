@@ -14,11 +14,31 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_SO = os.path.join(ROOT, "oracle", "libfkl_oracle.so")
 REF_SO = os.path.join(ROOT, "oracle", "_ref", "libfkl_ref.so")
 
-U8, F32 = 0, 1
-READ_2D, READ_NV12 = 0, 1
+U8, F32, U16 = 0, 1, 2
+READ_2D, READ_NV12, READ_NV21, READ_P010, READ_P210, READ_Y210, READ_UYVY = 0, 1, 2, 3, 4, 5, 6
 PRESERVE_AR, IGNORE_AR = 0, 1
 MUL, ADD, SUB, DIV, REORDER, SATCAST_U8, CAST_F32, YUV2RGB_709_FULL = 1, 2, 3, 4, 5, 6, 7, 8
-WRITE_2D, TENSOR_WRITE, TENSOR_SPLIT = 0, 1, 2
+YUV2RGB, RGB2YUV, RGB2GRAY, ADD_LAST, DISCARD, SATCAST_U16 = 9, 10, 11, 12, 13, 14
+WRITE_2D, TENSOR_WRITE, TENSOR_SPLIT, WRITE_YUV = 0, 1, 2, 3
+
+# fk::PixelFormat / ColorDepth / ColorRange / ColorPrimitives enumerator values, and what the oracle calls each format
+PF_NV12, PF_NV21, PF_P010, PF_P210, PF_Y210, PF_UYVY = 0, 1, 3, 6, 8, 10
+CD_P8, CD_P10, CD_P12, CD_FN8, CD_FN10, CD_FN12 = 0, 1, 2, 3, 4, 5
+CR_LIMITED, CR_FULL = 0, 1
+CP_BT601, CP_BT709, CP_BT2020 = 0, 1, 2
+PF_READ_KIND = {PF_NV12: READ_NV12, PF_NV21: READ_NV21, PF_P010: READ_P010, PF_P210: READ_P210, PF_Y210: READ_Y210, PF_UYVY: READ_UYVY}
+PF_DEPTH = {PF_NV12: CD_P8, PF_NV21: CD_P8, PF_P010: CD_P10, PF_P210: CD_P10, PF_Y210: CD_P10, PF_UYVY: CD_P8}
+PF_WIDE = {PF_NV12: False, PF_NV21: False, PF_P010: True, PF_P210: True, PF_Y210: True, PF_UYVY: False}
+_NP_ELEM = {np.dtype(np.uint8): U8, np.dtype(np.float32): F32, np.dtype(np.uint16): U16}
+
+
+def frame_shape(pf: int, width: int, height: int):
+    """(rows, samples per row) of the backing array of a width x height frame in pixel format pf."""
+    if pf in (PF_NV12, PF_NV21, PF_P010):
+        return height + height // 2, width
+    if pf == PF_P210:
+        return 2 * height, width
+    return height, 2 * width       # packed 4:2:2
 
 
 class Op(C.Structure):
@@ -44,7 +64,7 @@ class Write(C.Structure):
     _fields_ = [
         ("kind", C.c_int32), ("elem", C.c_int32), ("cn", C.c_int32), ("data", C.c_void_p),
         ("width", C.c_int32), ("height", C.c_int32), ("planes", C.c_int32), ("color_planes", C.c_int32),
-        ("pitch", C.c_int32),
+        ("pitch", C.c_int32), ("yuv_format", C.c_int32),
     ]
 
 
@@ -79,6 +99,12 @@ def oracle():
         lib.fklo_yuv2rgb_709_full_matrix.argtypes = [C.POINTER(C.c_float)]
         lib.fklo_yuv2rgb_709_full.restype = None
         lib.fklo_yuv2rgb_709_full.argtypes = [C.POINTER(C.c_uint8), C.POINTER(C.c_float)]
+        lib.fklo_color_matrix.restype = C.c_int
+        lib.fklo_color_matrix.argtypes = [C.c_int32] * 4 + [C.POINTER(C.c_float)]
+        lib.fklo_depth_constants.restype = C.c_int
+        lib.fklo_depth_constants.argtypes = [C.c_int32] + [C.POINTER(C.c_float)] * 3
+        lib.fklo_saturate_cast_u16.restype = C.c_uint16
+        lib.fklo_saturate_cast_u16.argtypes = [C.c_float]
         lib.fklo_bilinear.restype = C.c_float
         lib.fklo_bilinear.argtypes = [C.c_float] * 6
         lib.fklo_mt_seed.restype = None
@@ -140,7 +166,7 @@ def read_2d(a: np.ndarray, cn: int, crop=None, resize=None, ar=IGNORE_AR, bg=(0,
     """`a` is (H, W, cn) uint8/float32 or (H, W) for cn == 1 (possibly a padded row buffer if pitch given)."""
     r = Read()
     r.kind = READ_2D
-    r.elem = U8 if a.dtype == np.uint8 else F32
+    r.elem = _NP_ELEM[a.dtype]
     r.cn = cn
     r.height = a.shape[0]
     r.width = int(width) if width is not None else a.shape[1]
@@ -160,6 +186,31 @@ def read_nv12(buf: np.ndarray, width: int, height: int, resize=None, ar=IGNORE_A
     r.data = _ptr(buf)
     _fill_common(r, None, resize, ar, (0, 0, 0, 0), tap_ops)
     return r
+
+
+def read_yuv(pf: int, buf: np.ndarray, width: int, height: int, resize=None, ar=IGNORE_AR, tap_ops=None) -> Read:
+    """A frame in pixel format pf (see frame_shape) of uint8 or uint16 samples."""
+    r = Read()
+    r.kind = PF_READ_KIND[pf]
+    r.elem = U16 if PF_WIDE[pf] else U8
+    r.cn = 3
+    r.width, r.height = width, height
+    r.pitch = buf.strides[0]
+    r.data = _ptr(buf)
+    _fill_common(r, None, resize, ar, (0, 0, 0, 0), tap_ops)
+    return r
+
+
+def write_yuv(pf: int, buf: np.ndarray, width: int, height: int) -> Write:
+    w = Write()
+    w.kind = WRITE_YUV
+    w.elem = U16 if PF_WIDE[pf] else U8
+    w.cn = 3
+    w.data = _ptr(buf)
+    w.width, w.height, w.planes, w.color_planes = width, height, 1, 1
+    w.pitch = buf.strides[0]
+    w.yuv_format = PF_READ_KIND[pf]
+    return w
 
 
 def _fill_common(r, crop, resize, ar, bg, tap_ops):
@@ -184,11 +235,11 @@ def write(kind, a: np.ndarray, cn: int, width: int, height: int, planes: int = 1
           pitch=None) -> Write:
     w = Write()
     w.kind = kind
-    w.elem = U8 if a.dtype == np.uint8 else F32
+    w.elem = _NP_ELEM[a.dtype]
     w.cn = cn
     w.data = _ptr(a)
     w.width, w.height, w.planes, w.color_planes = width, height, planes, color_planes
-    esz = 1 if a.dtype == np.uint8 else 4
+    esz = a.dtype.itemsize
     if pitch is None:
         pitch = width * esz * (1 if kind == TENSOR_SPLIT else cn)
     w.pitch = int(pitch)
@@ -430,4 +481,142 @@ def ref_crop_swap_u8(src, rects):
     rc = ref().fklref_crop_swap_u8_b4(C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0],
                                       _i32p(rects), C.c_void_p(_ptr(out)))
     assert rc == 0
+    return out
+
+
+# ---- pixel formats and colour conversions ----------------------------------------------------------------
+
+def oracle_color_matrix(cd, cr, cp, to_rgb):
+    m = (C.c_float * 9)()
+    assert oracle().fklo_color_matrix(cd, cr, cp, int(bool(to_rgb)), m) == 0
+    return np.array(list(m), np.float32)
+
+
+def ref_color_matrix(cd, cr, cp, to_rgb):
+    m = np.zeros(9, np.float32)
+    assert ref().fklref_color_matrix(cd, cr, cp, int(bool(to_rgb)), _f32p(m)) == 0
+    return m
+
+
+def oracle_yuv_to_rgb(pf, cr, cp, frame, width, height):
+    out = np.zeros((height, width, 3), np.float32)
+    execute([read_yuv(pf, frame, width, height)], [op(YUV2RGB, idx=(PF_DEPTH[pf], cr, cp, 0))], [write(WRITE_2D, out, 3, width, height)])
+    return out
+
+
+def ref_yuv_to_rgb(pf, cr, cp, frame, width, height):
+    out = np.zeros((height, width, 3), np.float32)
+    rc = ref().fklref_yuv_to_rgb(pf, cr, cp, C.c_void_p(_ptr(frame)), width, height, frame.strides[0], C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
+    return out
+
+
+def _satcast(pf):
+    return SATCAST_U16 if PF_WIDE[pf] else SATCAST_U8
+
+
+def oracle_rgb_to_yuv(pf, cr, cp, rgb, frame):
+    """rgb (H,W,3) uint8/uint16; `frame` is the pre-filled backing array the chain stores into (returned)."""
+    h, w = rgb.shape[:2]
+    execute([read_2d(rgb, 3)], [op(RGB2YUV, idx=(PF_DEPTH[pf], cr, cp, 0)), op(_satcast(pf))], [write_yuv(pf, frame, w, h)])
+    return frame
+
+
+def ref_rgb_to_yuv(pf, cr, cp, rgb, frame):
+    h, w = rgb.shape[:2]
+    rc = ref().fklref_rgb_to_yuv(pf, cr, cp, C.c_void_p(_ptr(rgb)), w, h, rgb.strides[0], C.c_void_p(_ptr(frame)), frame.strides[0])
+    assert rc == 0, rc
+    return frame
+
+
+YUV_RESIZE_COMBO = {PF_NV21: (CR_FULL, CP_BT601), PF_UYVY: (CR_LIMITED, CP_BT709), PF_P010: (CR_LIMITED, CP_BT2020)}
+
+
+def oracle_yuv_resize(pf, frame, width, height, dst, scale):
+    dw, dh = dst
+    cr, cp = YUV_RESIZE_COMBO[pf]
+    out = np.zeros((dh, dw, 3), np.float32)
+    execute([read_yuv(pf, frame, width, height, resize=dst, tap_ops=[op(YUV2RGB, idx=(PF_DEPTH[pf], cr, cp, 0))])],
+            [op(MUL, [scale])], [write(WRITE_2D, out, 3, dw, dh)])
+    return out
+
+
+def ref_yuv_resize(pf, frame, width, height, dst, scale):
+    dw, dh = dst
+    out = np.zeros((dh, dw, 3), np.float32)
+    rc = ref().fklref_yuv_resize(pf, C.c_void_p(_ptr(frame)), width, height, frame.strides[0], dw, dh, C.c_float(scale),
+                                 C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
+    return out
+
+
+def oracle_convert_depth(cd, cr, cp, to_rgb, src):
+    h, w = src.shape[:2]
+    out = np.zeros((h, w, 3), np.float32)
+    execute([read_2d(src, 3)], [op(YUV2RGB if to_rgb else RGB2YUV, idx=(cd, cr, cp, 0))], [write(WRITE_2D, out, 3, w, h)])
+    return out
+
+
+def ref_convert_depth(cd, cr, cp, to_rgb, src):
+    h, w = src.shape[:2]
+    out = np.zeros((h, w, 3), np.float32)
+    rc = ref().fklref_convert_depth(cd, cr, cp, int(bool(to_rgb)), C.c_void_p(_ptr(src)), w, h, src.strides[0], C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
+    return out
+
+
+# ColorConversion codes exercised by the case drivers: which -> (input dtype, cn in, output dtype, cn out, oracle ops)
+_SWAP3, _SWAP4 = (2, 1, 0, 0), (2, 1, 0, 3)
+COLOR_CODES = {
+    0: (np.uint8, 3, np.uint8, 4, lambda: [op(ADD_LAST, [255.0])]),                                    # BGR2BGRA
+    1: (np.uint8, 4, np.uint8, 3, lambda: [op(DISCARD, idx=(3, 0, 0, 0))]),                              # BGRA2BGR
+    2: (np.uint8, 3, np.uint8, 4, lambda: [op(REORDER, idx=_SWAP3), op(ADD_LAST, [255.0])]),            # BGR2RGBA
+    3: (np.uint8, 4, np.uint8, 3, lambda: [op(REORDER, idx=_SWAP4), op(DISCARD, idx=(3, 0, 0, 0))]),     # BGRA2RGB
+    4: (np.uint8, 4, np.uint8, 4, lambda: [op(REORDER, idx=_SWAP4)]),                                   # BGRA2RGBA
+    5: (np.uint8, 3, np.uint8, 1, lambda: [op(RGB2GRAY, idx=(U8, 0, 0, 0))]),                            # RGB2GRAY
+    6: (np.uint8, 3, np.uint8, 1, lambda: [op(REORDER, idx=_SWAP3), op(RGB2GRAY, idx=(U8, 0, 0, 0))]),   # BGR2GRAY
+    7: (np.uint8, 4, np.uint8, 1, lambda: [op(RGB2GRAY, idx=(U8, 0, 0, 0))]),                            # RGBA2GRAY
+    8: (np.uint8, 4, np.uint8, 1, lambda: [op(REORDER, idx=_SWAP4), op(RGB2GRAY, idx=(U8, 0, 0, 0))]),   # BGRA2GRAY
+    9: (np.float32, 3, np.float32, 1, lambda: [op(RGB2GRAY, idx=(F32, 0, 0, 0))]),                       # RGB2GRAY, float
+    10: (np.uint16, 3, np.uint16, 4, lambda: [op(ADD_LAST, [1023.0])]),                                 # BGR2BGRA, 10 bit
+}
+
+
+def _image(shape_hw, cn, dtype):
+    h, w = shape_hw
+    return np.zeros((h, w, cn) if cn > 1 else (h, w), dtype)
+
+
+def oracle_convert_code(which, src):
+    _, cin, odt, cout, ops = COLOR_CODES[which]
+    h, w = src.shape[:2]
+    out = _image((h, w), cout, odt)
+    execute([read_2d(src, cin)], ops(), [write(WRITE_2D, out, cout, w, h)])
+    return out
+
+
+def ref_convert_code(which, src):
+    _, cin, odt, cout, _ = COLOR_CODES[which]
+    h, w = src.shape[:2]
+    out = _image((h, w), cout, odt)
+    rc = ref().fklref_convert_code(which, C.c_void_p(_ptr(src)), w, h, src.strides[0], C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
+    return out
+
+
+NORMALIZE = {0: (np.uint8, 255.0), 1: (np.uint16, 1023.0)}
+
+
+def oracle_normalize(which, src):
+    h, w = src.shape[:2]
+    out = np.zeros((h, w, 3), np.float32)
+    execute([read_2d(src, 3)], [op(DIV, [NORMALIZE[which][1]])], [write(WRITE_2D, out, 3, w, h)])
+    return out
+
+
+def ref_normalize(which, src):
+    h, w = src.shape[:2]
+    out = np.zeros((h, w, 3), np.float32)
+    rc = ref().fklref_normalize(which, C.c_void_p(_ptr(src)), w, h, src.strides[0], C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
     return out

@@ -36,7 +36,7 @@ def test_benchmark_chains_are_compiled_in():
         "Chain<Read2D<f32>,OpList<Add<f32,f32,f32>>,Write2D<f32>>",                          # configuration 2, N = 1
         "Chain<BatchRead<64,ResizeLinear<1,Crop<Read2D<Vec<u8,3>>>>>,OpList<Reorder<",      # configuration 3
         "Chain<BatchRead<100,FusedRead<Read2D<Vec<u8,3>>,Mul<",                              # configuration 4
-        "Chain<ResizeLinear<1,FusedRead<ReadNV12,YUV2RGB709Full8>>,OpList<Mul<Vec<f32,3>,f32,Vec<f32,3>>>,TensorSplit<",  # 5
+        "Chain<ResizeLinear<1,FusedRead<ReadNV12,YUV2RGB<0,1,1>>>,OpList<Mul<Vec<f32,3>,f32,Vec<f32,3>>>,TensorSplit<",  # 5
     ]
     for prefix in want:
         assert any(s.startswith(prefix) for s in sigs), prefix
