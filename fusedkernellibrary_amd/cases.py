@@ -232,3 +232,11 @@ def convert_code(which, src, out):
 def normalize(which, src, out):
     """NormalizePixel<uchar3, p8bit> (which = 0) or <ushort3, p10bit> (which = 1); out (H,W,3) f32 cuda."""
     _ok(cases().fklcase_normalize(_stream(), int(which), _p(src), src.shape[1], src.shape[0], _pitch(src), _p(out), _pitch(out)))
+
+
+def pad(src, border_type, left, top, out, value=(0, 0, 0)):
+    """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out."""
+    v = np.zeros(4, np.float32)
+    v[: len(value)] = value
+    _ok(cases().fklcase_pad(_stream(), 0 if src.element_size() == 1 else 1, int(border_type), _p(src), src.shape[1], src.shape[0], _pitch(src),
+                            int(left), int(top), out.shape[1], out.shape[0], v.ctypes.data_as(C.c_void_p), _p(out), _pitch(out)))

@@ -1123,6 +1123,61 @@ template <class Back> struct Crop {
 #endif
 };
 
+// BorderReader<BT, Params, BackIOp>: FK/algorithms/image_processing/border_reader.h:177-327.  Coordinates outside the
+// back operation's extent are folded back into it (BT = value of fk::BorderType: 1 REPLICATE aaa|abc|ccc, 2 REFLECT
+// cba|abc|cba, 3 WRAP abc|abc|abc, 4 REFLECT_101 cb|abc|ba) or yield a constant (0 CONSTANT).  The index arithmetic
+// is the reference's, in int: the high side is folded first, then the low side.  The extent it reports is the back
+// operation's, so it changes nothing by itself; a Crop with a rectangle that leaves the image is what reaches outside.
+template <int BT, class Back> struct Border {
+    static_assert(BT >= 0 && BT <= 4, "border types: CONSTANT, REPLICATE, REFLECT, WRAP, REFLECT_101");
+    using Out = typename Back::Out;
+    struct Params { Out value; typename Back::Params back; };     // value: CONSTANT only
+    static constexpr bool kTapCursor = false;
+    FKD_NAME("Border<" + istr(BT) + "," + Back::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
+    FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
+    FKD_DEV static int iabs(int v) { return v < 0 ? -v : v; }
+    // n = extent along the axis (last index = n - 1)
+    FKD_DEV static int fold(int i, int n) {
+        const int last = n - 1;
+        if constexpr (BT == 1) {
+            const int hi = i < last ? i : last;
+            return hi > 0 ? hi : 0;
+        } else if constexpr (BT == 2) {
+            const int hi = last - iabs(last - i) + (i > last ? 1 : 0);
+            return (iabs(hi) - (hi < 0 ? 1 : 0)) % (last + 1);
+        } else if constexpr (BT == 3) {
+            const int hi = i < n ? i : i % n;
+            return hi >= 0 ? hi : hi - ((hi - n + 1) / n) * n;
+        } else {
+            const int hi = iabs(last - iabs(last - i)) % (last + 1);
+            return iabs(hi) % (last + 1);
+        }
+    }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        const int w = Back::width(p.back), h = Back::height(p.back);
+        if constexpr (BT == 0) {
+            const bool inside = x >= 0 && x < w && y >= 0 && y < h;
+            // outside lanes read element (0, 0) instead of branching around the load; the select drops it
+            const Out v = Back::exec(inside ? x : 0, inside ? y : 0, z, p.back);
+            return inside ? v : p.value;
+        } else {
+            return Back::exec(fold(x, w), fold(y, h), z, p.back);
+        }
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+    }
+    FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // element-wise either way
+    using Raw = Out;
+    FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
+    struct TapRow {}; struct TapBits {}; struct PairBits {};
+    static constexpr bool kTapOverread = false, kTapPair = false;
+#endif
+};
+
 // FusedOperation<Read..., compute...> used as a Read: FK/core/execution_model/operation_model/fused_operation.h
 // as produced by Fuser::fuse, FK/core/execution_model/operation_model/iop_fuser.h:99-106.
 template <class Back, class... Ops> struct FusedRead {

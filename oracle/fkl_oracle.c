@@ -396,10 +396,45 @@ static void read_source(const fklo_read *r, int x, int y, fklo_val *out) {
 
 /* Crop<BackIOp>::exec, FK/algorithms/image_processing/crop.h:36-39: shift by the rect origin, no clipping;
  * then whatever compute ops were fused into the read (FusedOperation, iop_fuser.h:99-106). */
+/* BorderReader<BT,...>::exec, FK/algorithms/image_processing/border_reader.h:177-327: idx = low(high(i)) in int
+ * arithmetic; n is the extent of the operation behind the border. */
+static int iabs(int v) { return v < 0 ? -v : v; }
+static int border_fold(int type, int i, int n) {
+    const int last = n - 1;
+    switch (type) {
+    case 1: { const int hi = i < last ? i : last; return hi > 0 ? hi : 0; }                               /* REPLICATE   */
+    case 2: { const int hi = last - iabs(last - i) + (i > last); return (iabs(hi) - (hi < 0)) % (last + 1); } /* REFLECT */
+    case 3: { const int hi = i < n ? i : i % n; return hi >= 0 ? hi : hi - ((hi - n + 1) / n) * n; }      /* WRAP        */
+    default: { const int hi = iabs(last - iabs(last - i)) % (last + 1); return iabs(hi) % (last + 1); }   /* REFLECT_101 */
+    }
+}
+
 static int read_tap(const fklo_read *r, int x, int y, fklo_val *out) {
     if (r->has_crop) {
         x += r->crop[0];
         y += r->crop[1];
+    }
+    if (r->border) {
+        const int type = r->border - 1;
+        if (type < 0 || type > 4) return FKLO_EINVAL;
+        if (type == 0) {
+            if (!(x >= 0 && x < r->width && y >= 0 && y < r->height)) {
+                read_source(r, 0, 0, out);     /* for the type and channel count */
+                for (int c = 0; c < out->cn; ++c) {
+                    out->f[c] = r->border_value[c];
+                    out->u[c] = (uint8_t)r->border_value[c];
+                    out->h[c] = (uint16_t)r->border_value[c];
+                }
+                for (int i = 0; i < r->n_tap_ops; ++i) {
+                    const int rc = apply_op(&r->tap_ops[i], out);
+                    if (rc) return rc;
+                }
+                return FKLO_OK;
+            }
+        } else {
+            x = border_fold(type, x, r->width);
+            y = border_fold(type, y, r->height);
+        }
     }
     read_source(r, x, y, out);
     for (int i = 0; i < r->n_tap_ops; ++i) {

@@ -104,6 +104,9 @@ typedef struct {
     int32_t warp;            /* 0 none, 1 Warping<Affine>, 2 Warping<Perspective>; output grid dst_w x dst_h,     */
     float warp_m[9];         /* row-major transform (affine uses the first two rows); excludes has_resize         */
     int32_t deinterlace;     /* 0 none, 1 Deinterlace<BLEND>, 2 <INTER_LINEAR> keeping even lines, 3 keeping odd   */
+    int32_t border;          /* BorderReader between the source and the crop: 0 none, else 1 + fk::BorderType       */
+    float border_value[4];   /* (1 CONSTANT, 2 REPLICATE, 3 REFLECT, 4 WRAP, 5 REFLECT_101); CONSTANT's value, typed  */
+                             /* like the source element                                                             */
 } fklo_read;
 
 typedef struct {

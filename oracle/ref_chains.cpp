@@ -16,6 +16,7 @@
 #include <fused_kernel/algorithms/image_processing/resize.h>
 #include <fused_kernel/algorithms/image_processing/warping.h>
 #include <fused_kernel/algorithms/image_processing/deinterlace.h>
+#include <fused_kernel/algorithms/image_processing/border_reader.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
@@ -27,6 +28,7 @@
 // Pixel-format and colour-conversion chains: the same text the GPU case drivers compile against this repository's
 // headers, compiled here against the reference's.
 #include "../tests/cases/color_chains.h"
+#include "../tests/cases/border_chains.h"
 
 using namespace fk;
 using CpuDPP = TransformDPP<ParArch::CPU>;
@@ -394,3 +396,13 @@ int fklref_color_matrix(int cd, int cr, int cp, int to_rgb, float* m9) {
 }
 
 } // extern "C"
+
+// ---- padding through BorderReader (tests/cases/border_chains.h on the reference's CPU backend) ------------------
+extern "C" int fklref_pad(int elem, int border_type, const void* src, int w, int h, int pitch, int left, int top, int out_w, int out_h,
+                          const float* value, void* out, int out_pitch) {
+    CpuStream s;
+    const int rc = border_chains::Chains<CpuDPP, CpuStream>::pad(s, MemType::Host, elem, border_type, src, w, h, pitch, left, top, out_w,
+                                                                  out_h, value, out, out_pitch);
+    s.sync();
+    return rc;
+}

@@ -179,3 +179,30 @@ constexpr auto warpFusedIOp = warpReadIOp.then(warpIOp);
 static_assert(std::is_same_v<std::decay_t<decltype(warpFusedIOp)>,
                              fk::ReadBack<fk::Warping<fk::WarpType::Perspective, fk::Read<fk::PerThreadRead<fk::ND::_2D, uchar3>>>>>,
               "Unexpected type for fusedIOp");
+
+// ---- BorderReader, as the reference's own test spells it (tests/algorithm/test_border_reader.h:16-24), plus the
+// forms that complete later (.then) ---------------------------------------------------------------------------
+#include <fused_kernel/algorithms/image_processing/border_reader.h>
+constexpr auto borderReadIOp = fk::PerThreadRead<fk::ND::_2D, uchar3>::build(
+    fk::RawPtr<fk::ND::_2D, uchar3>{nullptr, {128, 128, 128 * sizeof(uchar3)}});
+constexpr auto borderIOp = fk::BorderReader<fk::BorderType::CONSTANT>::build(borderReadIOp, fk::make_set<uchar3>(0));
+static_assert(std::is_same_v<std::decay_t<decltype(borderIOp)>,
+                             fk::ReadBack<fk::BorderReader<fk::BorderType::CONSTANT, fk::BorderReaderParameters<fk::BorderType::CONSTANT, uchar3>,
+                                                           fk::Read<fk::PerThreadRead<fk::ND::_2D, uchar3>>>>>,
+              "Unexpected type for borderIOp");
+constexpr auto reflectLater = borderReadIOp.then(fk::BorderReader<fk::BorderType::REFLECT_101>::build());
+static_assert(std::is_same_v<std::decay_t<decltype(reflectLater)>,
+                             fk::ReadBack<fk::BorderReader<fk::BorderType::REFLECT_101, fk::BorderReaderParameters<fk::BorderType::REFLECT_101>,
+                                                           fk::Read<fk::PerThreadRead<fk::ND::_2D, uchar3>>>>>);
+constexpr auto constantLater = borderReadIOp.then(fk::BorderReader<fk::BorderType::CONSTANT>::build(fk::make_set<float3>(1.f)));
+static_assert(std::is_same_v<std::decay_t<decltype(constantLater)>, std::decay_t<decltype(borderIOp)>>,
+              "a border value of another type is converted to the pixels' type");
+
+// ---- Colour vocabulary: every conversion code names a type, every built pixel format has a reader and a writer ----
+static_assert(std::is_same_v<fk::ColorConversion<fk::ColorConversionCodes::COLOR_RGB2GRAY, uchar3, uchar>, fk::RGB2Gray<uchar3, uchar>>);
+static_assert(std::is_same_v<fk::ColorConversion<fk::ColorConversionCodes::COLOR_BGR2BGRA, uchar3, uchar4>, fk::AddOpaqueAlpha<uchar3, fk::ColorDepth::p8bit>>);
+static_assert(std::is_same_v<decltype(fk::ReadYUV<fk::PixelFormat::UYVY>::build(fk::RawImage<fk::PixelFormat::UYVY>{})),
+                             fk::Read<fk::ReadYUV<fk::PixelFormat::UYVY>>>);
+static_assert(std::is_same_v<decltype(fk::WriteYUV<fk::PixelFormat::P010>::build(fk::RawImage<fk::PixelFormat::P010>{})),
+                             fk::Write<fk::WriteYUV<fk::PixelFormat::P010>>>);
+static_assert(fk::maxDepthValue<fk::ColorDepth::p10bit> == 1023 && fk::maxDepthValue<fk::ColorDepth::fn12bit> == 1.f);

@@ -14,6 +14,7 @@
 #include <fused_kernel/algorithms/image_processing/resize.h>
 #include <fused_kernel/algorithms/image_processing/warping.h>
 #include <fused_kernel/algorithms/image_processing/deinterlace.h>
+#include <fused_kernel/algorithms/image_processing/border_reader.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
@@ -26,6 +27,7 @@
 #include <utility>
 
 #include "color_chains.h"   // pixel-format and colour-conversion chains, shared with the reference-backend harness
+#include "border_chains.h"  // padding chains, shared the same way
 
 using namespace fk;
 
@@ -457,3 +459,13 @@ int fklcase_normalize(void* stream_, int which, const void* src, int w, int h, i
 }
 
 } // extern "C"
+
+// ---- padding through BorderReader (border_chains.h on the GPU) ----------------------------------------------------
+extern "C" int fklcase_pad(void* stream_, int elem, int border_type, const void* src, int w, int h, int pitch, int left, int top,
+                           int out_w, int out_h, const float* value, void* out, int out_pitch) {
+    return guarded_rc([&] {
+        Stream s(stream_);
+        return border_chains::Chains<TransformDPP<>, Stream>::pad(s, MemType::Device, elem, border_type, src, w, h, pitch, left, top, out_w,
+                                                                  out_h, value, out, out_pitch);
+    });
+}

@@ -57,6 +57,7 @@ class Read(C.Structure):
         ("use_default", C.c_int32), ("def_", C.c_float * 4),
         ("warp", C.c_int32), ("warp_m", C.c_float * 9),
         ("deinterlace", C.c_int32),
+        ("border", C.c_int32), ("border_value", C.c_float * 4),
     ]
 
 
@@ -618,5 +619,32 @@ def ref_normalize(which, src):
     h, w = src.shape[:2]
     out = np.zeros((h, w, 3), np.float32)
     rc = ref().fklref_normalize(which, C.c_void_p(_ptr(src)), w, h, src.strides[0], C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
+    return out
+
+
+# ---- padding through BorderReader ---------------------------------------------------------------------------
+BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
+
+
+def oracle_pad(src, border_type, left, top, out_w, out_h, value=(0, 0, 0)):
+    """src (H,W,3) uint8 or (H,W) float32; the output grid starts `left`/`top` pixels before the image origin."""
+    cn = 3 if src.ndim == 3 else 1
+    out = np.zeros((out_h, out_w, cn) if cn > 1 else (out_h, out_w), src.dtype)
+    r = read_2d(src, cn, crop=(-left, -top, out_w, out_h))
+    r.border = 1 + border_type
+    for i, v in enumerate(value[:4]):
+        r.border_value[i] = float(v)
+    execute([r], [], [write(WRITE_2D, out, cn, out_w, out_h)])
+    return out
+
+
+def ref_pad(src, border_type, left, top, out_w, out_h, value=(0, 0, 0)):
+    cn = 3 if src.ndim == 3 else 1
+    out = np.zeros((out_h, out_w, cn) if cn > 1 else (out_h, out_w), src.dtype)
+    v = np.zeros(4, np.float32)
+    v[: len(value)] = value
+    rc = ref().fklref_pad(0 if src.dtype == np.uint8 else 1, int(border_type), C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0],
+                          int(left), int(top), int(out_w), int(out_h), _f32p(v), C.c_void_p(_ptr(out)), out.strides[0])
     assert rc == 0, rc
     return out
