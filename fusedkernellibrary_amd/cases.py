@@ -240,3 +240,27 @@ def pad(src, border_type, left, top, out, value=(0, 0, 0)):
     v[: len(value)] = value
     _ok(cases().fklcase_pad(_stream(), 0 if src.element_size() == 1 else 1, int(border_type), _p(src), src.shape[1], src.shape[0], _pitch(src),
                             int(left), int(top), out.shape[1], out.shape[0], v.ctypes.data_as(C.c_void_p), _p(out), _pitch(out)))
+
+
+# ---- divergent launches and the CircularTensor window (tests/cases/circular_chains.h) -------------------------------
+
+def divergent_two(a, b, add, out):
+    """a, b (H,W) i32-typed cuda tensors holding uint32; out (2,H,W): plane 0 = a + add, plane 1 = b, in ONE launch."""
+    _ok(cases().fklcase_divergent_two(_stream(), _p(a), _p(b), a.shape[1], a.shape[0], _pitch(a), C.c_uint32(int(add)), _p(out)))
+
+
+def divergent_mixed(tensor4, mul, img, out):
+    """tensor4 (4,H,W,3) f32 cuda, img (ih,iw,3) u8 cuda, out (4,H,W,3) f32 cuda: planes 0,3 = tensor4 * mul, planes 1,2 = img resized."""
+    _ok(cases().fklcase_divergent_mixed(_stream(), _p(tensor4), tensor4.shape[2], tensor4.shape[1], C.c_float(float(mul)), _p(img), img.shape[1],
+                                        img.shape[0], _pitch(img), _p(out)))
+
+
+def circular(batch, oldest_first, images, fill):
+    """images: list of (H,W,3) u8 cuda tensors fed one by one to CircularTensor::update; returns the tensor after each update,
+    (iters, batch, 3, H, W) float32 on the host."""
+    h, w = images[0].shape[:2]
+    states = np.zeros((len(images), batch, 3, h, w), np.float32)
+    ptrs = (C.c_void_p * len(images))(*[i.data_ptr() for i in images])
+    _ok(cases().fklcase_circular(_stream(), int(batch), int(bool(oldest_first)), ptrs, len(images), w, h, _pitch(images[0]), C.c_float(float(fill)),
+                                 states.ctypes.data_as(C.c_void_p)))
+    return states

@@ -74,8 +74,10 @@ template <class Chain> constexpr bool is_gather_chain() {
 constexpr int kRowsBX = 64;   // lanes along x: one wave per row segment
 constexpr int kRowsBY = 4;    // waves per workgroup
 
+// `kernarg_offset`: where p sits inside the kernel-argument segment (0 when the chain's parameter block is the
+// kernel's first argument); long chains fetch their operations' parameters from there.
 template <class Chain, int V, int ROWS, bool ALIGNED>
-__device__ __forceinline__ void rows_body(const typename Chain::Params& p) {
+__device__ __forceinline__ void rows_body(const typename Chain::Params& p, u32 kernarg_offset = 0) {
     using R = typename Chain::Read;
     using W = typename Chain::Write;
     const int z = blockIdx.z;
@@ -97,7 +99,7 @@ __device__ __forceinline__ void rows_body(const typename Chain::Params& p) {
         }
         // all ROWS*V elements go through the chain together, operation by operation
         Slot<typename Chain::Value> out[ROWS * V];
-        if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<ROWS * V>(in, out, (const FKD_CONSTANT void*)__builtin_amdgcn_kernarg_segment_ptr());
+        if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<ROWS * V>(in, out, (const FKD_CONSTANT char*)__builtin_amdgcn_kernarg_segment_ptr() + kernarg_offset);
         else Chain::template compute_run<ROWS * V>(in, out, p.ops);
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
@@ -115,7 +117,7 @@ __device__ __forceinline__ void rows_body(const typename Chain::Params& p) {
                 Slot<typename R::Out> in[1];
                 Slot<typename Chain::Value> out[1];
                 in[0].v = R::exec(x, y, z, p.read);
-                if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<1>(in, out, (const FKD_CONSTANT void*)__builtin_amdgcn_kernarg_segment_ptr());
+                if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<1>(in, out, (const FKD_CONSTANT char*)__builtin_amdgcn_kernarg_segment_ptr() + kernarg_offset);
                 else Chain::template compute_run<1>(in, out, p.ops);
                 W::exec(x, y, z, out[0].v, p.write);
             }
@@ -140,11 +142,11 @@ template <class Op, class P> FKD_DEV bool write_plane_aligned(const P& p, int z)
     else return Op::rows_aligned(p);
 }
 template <class Chain, int V, int ROWS>
-__device__ __forceinline__ void rows_auto_body(const typename Chain::Params& p) {
+__device__ __forceinline__ void rows_auto_body(const typename Chain::Params& p, u32 kernarg_offset = 0) {
     const int z = blockIdx.z;
     const bool aligned = read_plane_aligned<typename Chain::Read>(p.read, z) && write_plane_aligned<typename Chain::Write>(p.write, z);
-    if (aligned) rows_body<Chain, V, ROWS, true>(p);
-    else rows_body<Chain, V, ROWS, false>(p);
+    if (aligned) rows_body<Chain, V, ROWS, true>(p, kernarg_offset);
+    else rows_body<Chain, V, ROWS, false>(p, kernarg_offset);
 }
 
 // ---- gather bilinear kernel ----------------------------------------------------------------------------
@@ -392,6 +394,39 @@ template <class Chain> struct RowsConfig {
     static constexpr int ROWS = kScattered ? 1 : FKD_ROWS;
 };
 
+// ---- divergent batch kernel -------------------------------------------------------------------------------
+
+// Several chains in one launch of the rows kernel's geometry: plane z runs chain select[z] (wave uniform: the plane is
+// the grid's z index).  Every chain runs through the rows body, bilinear reads included (one element per thread); the
+// grid is laid out for the smallest elements-per-thread of the chains, and workgroups beyond a chain's own extent
+// leave at once.
+template <int A, int... Rest> struct MinOf { static constexpr int value = A; };
+template <int A, int B, int... Rest> struct MinOf<A, B, Rest...> { static constexpr int value = MinOf<(A < B ? A : B), Rest...>::value; };
+template <class... Chains> struct RowsConfig<Divergent<Chains...>> {
+    static constexpr int V = MinOf<RowsConfig<Chains>::V...>::value;
+    static constexpr int ROWS = MinOf<RowsConfig<Chains>::ROWS...>::value;
+};
+template <int I, class First, class... Rest, class P>
+__device__ __forceinline__ void divergent_run(u32 sel, const P& p, const Tup<typename First::Params, typename Rest::Params...>& seq) {
+    if (sel == u32(I)) {
+        const u32 offset = u32(reinterpret_cast<const char*>(&seq.head) - reinterpret_cast<const char*>(&p));
+        rows_auto_body<First, RowsConfig<First>::V, RowsConfig<First>::ROWS>(seq.head, offset);
+    } else if constexpr (sizeof...(Rest) > 0) {
+        divergent_run<I + 1, Rest...>(sel, p, seq.tail);
+    }
+}
+template <class D> struct DivergentBody;
+template <class... Chains> struct DivergentBody<Divergent<Chains...>> {
+    __device__ __forceinline__ static void run(const typename Divergent<Chains...>::Params& p) {
+        const u32 z = blockIdx.z;
+        const u32 sel = __builtin_amdgcn_readfirstlane(u32(p.select[z < u32(Divergent<Chains...>::kMaxPlanes) ? z : 0u]));
+        divergent_run<0, Chains...>(sel, p, p.seq);
+    }
+};
+template <class D> __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_divergent(const typename D::Params p) {
+    DivergentBody<D>::run(p);
+}
+
 // The one kernel of a chain compiled at run time, and what its launcher needs to know about it.  A launcher that
 // only has the parameter block as bytes reads the active grid from its first three words.
 struct JitMeta {
@@ -402,11 +437,15 @@ struct JitMeta {
     u32 reserved;
 };
 template <class Chain> constexpr JitMeta jit_meta() {
-    return JitMeta{is_gather_chain<Chain>() ? 1u : 0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V),
-                   u32(RowsConfig<Chain>::ROWS), u32(FKD_GATHER_XI), u32(FKD_GATHER_YI), u32(kGatherBY), 0u};
+    if constexpr (IsDivergent<Chain>::value)
+        return JitMeta{0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V), u32(RowsConfig<Chain>::ROWS), 0u, 0u, 0u, 0u};
+    else
+        return JitMeta{is_gather_chain<Chain>() ? 1u : 0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V),
+                       u32(RowsConfig<Chain>::ROWS), u32(FKD_GATHER_XI), u32(FKD_GATHER_YI), u32(kGatherBY), 0u};
 }
 template <class Chain> __device__ __forceinline__ void jit_body(const typename Chain::Params& p, const TileGeom& g) {
-    if constexpr (is_gather_chain<Chain>()) gather_body<Chain, FKD_GATHER_XI, FKD_GATHER_YI>(p, g);
+    if constexpr (IsDivergent<Chain>::value) DivergentBody<Chain>::run(p);
+    else if constexpr (is_gather_chain<Chain>()) gather_body<Chain, FKD_GATHER_XI, FKD_GATHER_YI>(p, g);
     else rows_auto_body<Chain, RowsConfig<Chain>::V, RowsConfig<Chain>::ROWS>(p);
 }
 

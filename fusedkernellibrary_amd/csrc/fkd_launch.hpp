@@ -43,9 +43,25 @@ hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, La
     return hipGetLastError();
 }
 
+// Several chains in one launch: the grid of the rows kernel over the largest extent, alignment decided per plane on
+// the device.
+template <class D>
+hipError_t launch_divergent(const typename D::Params& p, hipStream_t stream, LaunchInfo* info) {
+    constexpr int V = RowsConfig<D>::V, ROWS = RowsConfig<D>::ROWS;
+    const unsigned gx = (p.active_w + kRowsBX * V - 1) / (kRowsBX * V);
+    const unsigned gy = (p.active_h + kRowsBY * ROWS - 1) / (kRowsBY * ROWS);
+    const dim3 grid(gx, gy, p.active_z), block(kRowsBX, kRowsBY, 1);
+    if (info) *info = LaunchInfo{"divergent", {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
+    if (grid.y > 65535u || grid.z > unsigned(D::kMaxPlanes)) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_divergent<D>), grid, block, 0, stream, p);
+    return hipGetLastError();
+}
+
 template <class Chain>
 hipError_t launch_chain(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
-    if constexpr (is_gather_chain<Chain>()) return launch_gather<Chain>(p, stream, info);
+    if constexpr (IsDivergent<Chain>::value) return launch_divergent<Chain>(p, stream, info);
+    else if constexpr (is_gather_chain<Chain>()) return launch_gather<Chain>(p, stream, info);
     else return launch_rows<Chain>(p, stream, info);
 }
 

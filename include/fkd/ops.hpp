@@ -953,6 +953,88 @@ template <class T> struct Read3D {
 #endif
 };
 
+// TensorPack<T>: FK/algorithms/basic_ops/memory_operations.h:243-290.  The planar layout TensorSplit writes, read back
+// as a vector: channel c of pixel (x, y, z) sits c * width * height base elements after the position of channel 0.
+template <class T> struct TensorPack {
+    static_assert(cn_v<T> >= 2, "Wrong type for split tensor read. It must be one of <type>2, <type>3 or <type>4.");
+    using Out = T;
+    using B = base_t<T>;
+    using Params = RawPtr3D<const B>;
+    static constexpr bool kTapCursor = false;
+    FKD_NAME("TensorPack<" + type_name<T>() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return int(p.width); }
+    FKD_DEV static int height(const Params& p) { return int(p.height); }
+    FKD_DEV static const B* at(const Params& p, int x, int y, int z) {
+        return reinterpret_cast<const B*>(reinterpret_cast<const char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z +
+                                          size_t(y) * p.pitch) + x;
+    }
+    FKD_DEV static T exec(int x, int y, int z, const Params& p) {
+        const FKD_GLOBAL B* g = detail::gconst<B>(at(p, x, y, z));
+        const size_t px = size_t(p.width) * p.height;
+        T o;
+        chan<0>(o) = g[0];
+        chan<1>(o) = g[px];
+        if constexpr (cn_v<T> > 2) chan<2>(o) = g[2 * px];
+        if constexpr (cn_v<T> > 3) chan<3>(o) = g[3 * px];
+        return o;
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
+        const B* r = at(p, x, y, z);
+        const size_t px = size_t(p.width) * p.height;
+        Slot<B> c[4][V];
+        detail::load_run<B, V, A>(r, c[0]);
+        detail::load_run<B, V, A>(r + px, c[1]);
+        if constexpr (cn_v<T> > 2) detail::load_run<B, V, A>(r + 2 * px, c[2]);
+        if constexpr (cn_v<T> > 3) detail::load_run<B, V, A>(r + 3 * px, c[3]);
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            chan<0>(out[i].v) = c[0][i].v;
+            chan<1>(out[i].v) = c[1][i].v;
+            if constexpr (cn_v<T> > 2) chan<2>(out[i].v) = c[2][i].v;
+            if constexpr (cn_v<T> > 3) chan<3>(out[i].v) = c[3][i].v;
+        }
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) {
+        return detail::dword_aligned(reinterpret_cast<const char*>(p.data) + ptrdiff_t(xoff) * ptrdiff_t(sizeof(B))) && p.pitch % 4 == 0 &&
+               (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 && (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
+    }
+    using Raw = Out;
+    FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
+    struct TapRow {}; struct TapBits {}; struct PairBits {};
+    static constexpr bool kTapOverread = false, kTapPair = false;
+#endif
+};
+
+// Plane index of a circular buffer of BATCH planes whose logical plane 0 is stored at `first`:
+// computeCircularThreadIdx, FK/algorithms/basic_ops/memory_operations.h:422-432.  DIR 0 (Ascendent) walks forward from
+// first, DIR 1 (Descendent) backward.
+template <int DIR, int BATCH> FKD_HD int circular_plane(int z, int first) {
+    if constexpr (DIR == 0) { const int c = z + first; return c >= BATCH ? c - BATCH : c; }
+    else { const int c = first - z; return c < 0 ? BATCH + c : c; }
+}
+
+// CircularTensorRead<direction, Operation, BATCH>: FK/algorithms/basic_ops/memory_operations.h:505-552.
+template <int DIR, int BATCH, class Back> struct CircularRead {
+    using Out = typename Back::Out;
+    struct Params { i32 first; typename Back::Params back; };
+    static constexpr bool kTapCursor = false;
+    FKD_NAME("CircularRead<" + istr(DIR) + "," + istr(BATCH) + "," + Back::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
+    FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return Back::exec(x, y, circular_plane<DIR, BATCH>(z, p.first), p.back); }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        Back::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), p.back, out);
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
+    using Raw = Out;
+    FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
+    struct TapRow {}; struct TapBits {}; struct PairBits {};
+    static constexpr bool kTapOverread = false, kTapPair = false;
+#endif
+};
+
 // ReadYUV<NV12> and ReadYUV<NV21>: FK/algorithms/image_processing/color_conversion.h:219-253.  Y from the luma
 // plane, the chroma pair from element x>>1 of chroma row y>>1; chroma base = data + pitch*height.  NV12 stores the
 // pair as (U,V), NV21 as (V,U) (template argument VU); the value is (Y,U,V) either way.
@@ -1700,6 +1782,40 @@ template <int N, class W> struct BatchWrite {
 #endif
 };
 
+// CircularTensorWrite<direction, Operation, BATCH>: FK/algorithms/basic_ops/memory_operations.h:554-587.
+template <int DIR, int BATCH, class W> struct CircularWrite {
+    using In = typename W::In;
+    struct Params { i32 first; typename W::Params w; };
+    FKD_NAME("CircularWrite<" + istr(DIR) + "," + istr(BATCH) + "," + W::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w); }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+        W::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w);
+    }
+    FKD_HD static bool rows_aligned(const Params& p) { return W::rows_aligned(p.w); }
+#endif
+};
+
+// A MidWrite operation directly before the chain's write (FK/core/execution_model/operation_model/
+// instantiable_operations.h:219-262: it stores its input and hands it on unchanged): the same value goes to both.
+template <class W1, class W2> struct TeeWrite {
+    static_assert(__is_same(typename W1::In, typename W2::In), "both writes take the value the chain produces");
+    using In = typename W2::In;
+    struct Params { typename W1::Params first; typename W2::Params second; };
+    FKD_NAME("TeeWrite<" + W1::name() + "," + W2::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) {
+        W1::exec(x, y, z, v, p.first);
+        W2::exec(x, y, z, v, p.second);
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+        W1::template exec_row<V, A>(x, y, z, v, p.first);
+        W2::template exec_row<V, A>(x, y, z, v, p.second);
+    }
+    FKD_HD static bool rows_aligned(const Params& p) { return W1::rows_aligned(p.first) && W2::rows_aligned(p.second); }
+#endif
+};
+
 // ===================================================================================================
 // A fused chain: one read, a fold of compute operations, one write, over an active grid.
 // ===================================================================================================
@@ -1759,5 +1875,27 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     }
 #endif
 };
+
+// DivergentBatchTransformDPP: FK/core/execution_model/data_parallel_patterns.h:286-381.  Several chains share one launch;
+// plane z of the grid (z counts over the planes of all chains together) runs chain select[z], with z handed to that
+// chain's read and write unchanged.  select[] is SequenceSelector::at(z), evaluated on the host for every plane of
+// the launch (it is a pure function of z), so user code never has to run on the device.  The grid covers the largest
+// chain; each chain keeps its own active extent.
+template <class... Chains> struct Divergent {
+    static_assert(sizeof...(Chains) >= 1 && sizeof...(Chains) <= 255, "one to 255 operation sequences");
+    static constexpr int kMaxPlanes = 256;
+    static constexpr int kChains = int(sizeof...(Chains));
+    struct Params {
+        u32 active_w, active_h, active_z, reserved;     // the launch grid: largest width and height, planes of all chains
+        u8 select[kMaxPlanes];
+        Tup<typename Chains::Params...> seq;
+    };
+#if defined(FKD_HOST_NAMES)
+    static std::string names() { std::string s; ((s += "," + Chains::name()), ...); return s.substr(1); }
+#endif
+    FKD_NAME("Divergent<" + names() + ">")
+};
+template <class T> struct IsDivergent { static constexpr bool value = false; };
+template <class... Chains> struct IsDivergent<Divergent<Chains...>> { static constexpr bool value = true; };
 
 } // namespace fkd

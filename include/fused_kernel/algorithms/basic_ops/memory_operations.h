@@ -1,5 +1,7 @@
 // Per-element memory operations: PerThreadRead / PerThreadWrite (pitched 1-D/2-D/3-D), TensorRead / TensorWrite,
-// TensorSplit (planar writer).  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:26-212.
+// TensorSplit (planar writer) and TensorPack (its reader), and the circular-buffer views CircularTensorRead /
+// CircularTensorWrite.  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:26-212, 243-290, 413-432,
+// 505-587.  The transposed-plane forms (TensorTSplit / TensorTPack) and CircularBatchRead/Write are not built.
 #ifndef FK_AMD_MEMORY_OPERATIONS_H
 #define FK_AMD_MEMORY_OPERATIONS_H
 
@@ -88,7 +90,81 @@ template <typename T> struct TensorSplit : WriteOperation<T, RawPtr<ND::_3D, VBa
     static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
 };
 
+// Planar reader: the layout TensorSplit writes, read back as a vector.
+template <typename T> struct TensorPack : ReadOperation<VBase<T>, RawPtr<ND::_3D, VBase<T>>, T, TF::DISABLED, TensorPack<T>> {
+    using Parent = ReadOperation<VBase<T>, RawPtr<ND::_3D, VBase<T>>, T, TF::DISABLED, TensorPack<T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(TensorPack, TensorPack)
+    static_assert(cn<T> >= 2, "Wrong type for split tensor read. It must be one of <type>2, <type>3 or <type>4.");
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint num_elems_y(const Point, const OperationDataType& opData) { return opData.params.dims.height; }
+    static constexpr uint num_elems_z(const Point, const OperationDataType& opData) { return opData.params.dims.planes; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {opData.params.dims.width, opData.params.dims.height, opData.params.dims.planes};
+    }
+};
+
+// A tensor of BATCH planes used as a circular buffer: logical plane z lives at (first + z) mod BATCH (Ascendent) or
+// (first - z) mod BATCH (Descendent).
+enum class CircularDirection { Ascendent, Descendent };
+template <typename OperationDataTypeArray> struct CircularMemoryParams {
+    int first;
+    OperationDataTypeArray opData;
+};
+
+template <CircularDirection direction, typename Operation, int BATCH>
+struct CircularTensorRead : ReadOperation<typename Operation::ReadDataType, CircularMemoryParams<OperationData<Operation>>,
+                                          typename Operation::OutputType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
+                                          CircularTensorRead<direction, Operation, BATCH>> {
+    using Parent = ReadOperation<typename Operation::ReadDataType, CircularMemoryParams<OperationData<Operation>>, typename Operation::OutputType,
+                                 Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED, CircularTensorRead<direction, Operation, BATCH>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(CircularTensorRead, CircularTensorRead)
+    static constexpr uint num_elems_x(const Point thread, const OperationDataType& opData) { return Operation::num_elems_x(thread, opData.params.opData); }
+    static constexpr uint num_elems_y(const Point thread, const OperationDataType& opData) { return Operation::num_elems_y(thread, opData.params.opData); }
+    // the planes of the view this read was given, not BATCH (BATCH stays the modulus of the circular index)
+    static constexpr uint num_elems_z(const Point thread, const OperationDataType& opData) { return Operation::num_elems_z(thread, opData.params.opData); }
+    static constexpr uint pitch(const Point thread, const OperationDataType& opData) { return Operation::pitch(thread, opData.params.opData); }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {num_elems_x(Point{0, 0, 0}, opData), num_elems_y(Point{0, 0, 0}, opData), num_elems_z(Point{0, 0, 0}, opData)};
+    }
+};
+
+template <CircularDirection direction, typename Operation, int BATCH>
+struct CircularTensorWrite : WriteOperation<typename Operation::InputType, CircularMemoryParams<OperationData<Operation>>,
+                                            typename Operation::WriteDataType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
+                                            CircularTensorWrite<direction, Operation, BATCH>> {
+    using Parent = WriteOperation<typename Operation::InputType, CircularMemoryParams<OperationData<Operation>>, typename Operation::WriteDataType,
+                                  Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED, CircularTensorWrite<direction, Operation, BATCH>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(CircularTensorWrite, CircularTensorWrite)
+    static constexpr uint num_elems_x(const Point thread, const OperationDataType& opData) { return Operation::num_elems_x(thread, opData.params.opData); }
+    static constexpr uint pitch(const Point thread, const OperationDataType& opData) { return Operation::pitch(thread, opData.params.opData); }
+};
+
 namespace amd {
+template <typename T> struct Lower<TensorPack<T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorPack<dev_t<T>>;
+    static typename type::Params params(const OperationData<TensorPack<T>>& d) {
+        return to_dev3<VBase<T>, const typename DevType<VBase<T>>::type>(d.params);
+    }
+};
+template <CircularDirection direction, typename Operation, int BATCH> struct Lower<CircularTensorRead<direction, Operation, BATCH>> {
+    static constexpr bool available = true;
+    using type = fkd::CircularRead<int(direction), BATCH, typename Lower<Operation>::type>;
+    static typename type::Params params(const OperationData<CircularTensorRead<direction, Operation, BATCH>>& d) {
+        return typename type::Params{d.params.first, Lower<Operation>::params(d.params.opData)};
+    }
+};
+template <CircularDirection direction, typename Operation, int BATCH> struct Lower<CircularTensorWrite<direction, Operation, BATCH>> {
+    static constexpr bool available = true;
+    using type = fkd::CircularWrite<int(direction), BATCH, typename Lower<Operation>::type>;
+    static typename type::Params params(const OperationData<CircularTensorWrite<direction, Operation, BATCH>>& d) {
+        return typename type::Params{d.params.first, Lower<Operation>::params(d.params.opData)};
+    }
+};
 template <typename T> struct Lower<PerThreadRead<ND::_2D, T>> {
     static constexpr bool available = true;
     using type = fkd::Read2D<dev_t<T>>;

@@ -16,5 +16,15 @@ struct TransformDPP {
     static constexpr TF THREAD_FUSION = TFEN;
 };
 
+
+// DivergentBatchTransformDPP: several operation sequences in ONE launch; plane z of the launch (z counts over the
+// planes of all sequences together) runs sequence SequenceSelector::at(z), and z reaches that sequence's read and
+// write unchanged.  SequenceSelector is any type with a static `uint at(uint z)`; on this backend it is evaluated on
+// the host for every plane of a launch and travels to the kernel as a table.
+// Interface counterpart: FK/core/execution_model/data_parallel_patterns.h:286-381.
+template <ParArch PA, typename SequenceSelector> struct DivergentBatchTransformDPP {
+    static constexpr ParArch PAR_ARCH = PA;
+};
+
 } // namespace fk
 #endif

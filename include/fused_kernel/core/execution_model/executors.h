@@ -47,33 +47,82 @@ auto lower_compute(std::index_sequence<Is...>, const Tuple& t) {
     return make_tup(lower_iop(std::get<Is + 1>(t))...);
 }
 
-template <typename... IOps> void launch_fused(void* stream, const IOps&... iOps) {
-    constexpr size_t N = sizeof...(IOps);
+// One fused IOp list (complete read, compute operations, [a MidWrite directly before] the write) as a device chain type
+// and its parameter block.
+template <typename... IOps> struct FusedChain {
+    static constexpr size_t N = sizeof...(IOps);
     static_assert(N >= 2, "a chain needs at least a read and a write operation");
-    const auto all = std::forward_as_tuple(iOps...);
     using Tuple = std::tuple<const IOps&...>;
-    using ReadIOp = std::decay_t<std::tuple_element_t<0, Tuple>>;
-    using WriteIOp = std::decay_t<std::tuple_element_t<N - 1, Tuple>>;
+    template <size_t I> using At = std::decay_t<std::tuple_element_t<I, Tuple>>;
+    using ReadIOp = At<0>;
+    using WriteIOp = At<N - 1>;
     static_assert(isAnyCompleteReadType<ReadIOp>, "the first operation must be a complete Read or ReadBack operation");
     static_assert(opIs<WriteType, WriteIOp>, "the last operation must be a Write operation");
+    // A MidWrite stores the value it receives and hands it on; directly before the final write both take the same value.
+    static constexpr bool kTee = N >= 3 && opIs<MidWriteType, At<N >= 3 ? N - 2 : 0>>;
+    static constexpr size_t kCompute = N - 2 - (kTee ? 1 : 0);
+    template <typename Seq> struct Build;
+    template <size_t... Is> struct Build<std::index_sequence<Is...>> {
+        static_assert((isComputeType<At<Is + 1>> && ...),
+                      "only Unary/Binary/Ternary operations may sit between the read and the write (a MidWrite only directly before the write)");
+        using WriteOp = std::conditional_t<kTee, fkd::TeeWrite<device_op_t<At<kTee ? N - 2 : N - 1>>, device_op_t<WriteIOp>>, device_op_t<WriteIOp>>;
+        using Chain = fkd::Chain<device_op_t<ReadIOp>, fkd::OpList<device_op_t<At<Is + 1>>...>, WriteOp>;
+        static typename Chain::Params params(const Tuple& all) {
+            typename Chain::Params p{};
+            const ActiveThreads active = std::get<0>(all).getActiveThreads();
+            p.active_w = active.x;
+            p.active_h = active.y;
+            p.active_z = active.z;
+            p.read = lower_iop(std::get<0>(all));
+            p.ops = make_tup(lower_iop(std::get<Is + 1>(all))...);
+            if constexpr (kTee) {
+                p.write.first = lower_iop(std::get<N - 2>(all));
+                p.write.second = lower_iop(std::get<N - 1>(all));
+            } else {
+                p.write = lower_iop(std::get<N - 1>(all));
+            }
+            return p;
+        }
+    };
+    using Builder = Build<std::make_index_sequence<kCompute>>;
+    using Chain = typename Builder::Chain;
+    static typename Chain::Params params(const IOps&... iOps) { return Builder::params(std::forward_as_tuple(iOps...)); }
+};
 
-    [&]<size_t... Is>(std::index_sequence<Is...>) {
-        static_assert((isComputeType<std::decay_t<std::tuple_element_t<Is + 1, Tuple>>> && ...),
-                      "only Unary/Binary/Ternary operations may sit between the read and the write");
-        using Chain = fkd::Chain<device_op_t<ReadIOp>,
-                                 fkd::OpList<device_op_t<std::decay_t<std::tuple_element_t<Is + 1, Tuple>>>...>,
-                                 device_op_t<WriteIOp>>;
-        typename Chain::Params p{};
-        const ActiveThreads active = std::get<0>(all).getActiveThreads();
-        p.active_w = active.x;
-        p.active_h = active.y;
-        p.active_z = active.z;
-        p.read = lower_iop(std::get<0>(all));
-        p.ops = make_tup(lower_iop(std::get<Is + 1>(all))...);
-        p.write = lower_iop(std::get<N - 1>(all));
-        gpuErrchk(fklhip_launch_handle(kernel_handle<Chain>(), &p, sizeof(p), stream));
-    }(std::make_index_sequence<N - 2>{});
+template <typename... IOps> void launch_fused(void* stream, const IOps&... iOps) {
+    using F = FusedChain<IOps...>;
+    static_assert(!F::kTee, "a MidWrite operation is only supported inside the sequences of a DivergentBatchTransformDPP launch");
+    const typename F::Chain::Params p = F::params(iOps...);
+    gpuErrchk(fklhip_launch_handle(kernel_handle<typename F::Chain>(), &p, sizeof(p), stream));
 }
+
+// Several already back-fused sequences in one launch.
+template <typename SequenceSelector, typename... Seqs> void launch_divergent(void* stream, const Seqs&... seqs) {
+    using D = fkd::Divergent<typename Seqs::Fused::Chain...>;
+    typename D::Params p{};
+    uint w = 0, h = 0, z = 0;
+    auto fill = [&](auto& self, auto& node, const auto& first, const auto&... rest) -> void {
+        node.head = first.params;
+        w = first.params.active_w > w ? first.params.active_w : w;
+        h = first.params.active_h > h ? first.params.active_h : h;
+        z += first.params.active_z;
+        if constexpr (sizeof...(rest) > 0) self(self, node.tail, rest...);
+    };
+    fill(fill, p.seq, seqs...);
+    if (z > uint(D::kMaxPlanes))
+        throw std::runtime_error("GPU Error: a DivergentBatchTransformDPP launch holds at most " + std::to_string(D::kMaxPlanes) + " planes");
+    p.active_w = w; p.active_h = h; p.active_z = z;
+    for (uint i = 0; i < z; ++i) {
+        const uint sel = uint(SequenceSelector::at(i));
+        // a plane no sequence claims runs nothing in the reference; the table entry then names no chain
+        p.select[i] = static_cast<unsigned char>(sel < uint(D::kChains) ? sel : 255u);
+    }
+    gpuErrchk(fklhip_launch_handle(kernel_handle<D>(), &p, sizeof(p), stream));
+}
+template <typename... IOps> struct LoweredSequence {
+    using Fused = FusedChain<IOps...>;
+    typename Fused::Chain::Params params;
+};
 
 } // namespace amd
 
@@ -125,6 +174,26 @@ private:
     friend struct BaseExecutor<Executor<TransformDPP<ParArch::GPU_AMD, TFEN, void>>>;
     template <typename... IOps> static void executeOperations_helper(Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
         amd::launch_fused(stream.getNativeStream(), iOps...);
+    }
+};
+
+
+// Executor of DivergentBatchTransformDPP: every sequence is back-fused like a TransformDPP chain, then all of them go
+// into one launch.  Interface counterpart: FK/core/execution_model/executors.h:360-411.
+template <typename SequenceSelector> struct Executor<DivergentBatchTransformDPP<ParArch::GPU_AMD, SequenceSelector>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::GPU_AMD; }
+    template <typename... IOpSequenceTypes>
+    static void executeOperations(Stream_<ParArch::GPU_AMD>& stream, const IOpSequenceTypes&... iOpSequences) {
+        amd::launch_divergent<SequenceSelector>(stream.getNativeStream(), lower(iOpSequences)...);
+    }
+
+private:
+    template <typename... IOps> static auto lower(const IOpSequence<IOps...>& seq) {
+        const auto fused = std::apply([](const auto&... iOps) { return BackFuser::fuse_back(iOps...); }, seq.iOps);
+        return std::apply([](const auto&... f) {
+            return amd::LoweredSequence<std::decay_t<decltype(f)>...>{amd::FusedChain<std::decay_t<decltype(f)>...>::params(f...)};
+        }, fused);
     }
 };
 

@@ -50,6 +50,18 @@ struct ClosedType {};
 
 struct NullType {};
 template <typename... Ts> struct TypeList {};
+// one_of_v<T, TypeList<...>>: T is one of the listed types.  EquivalentType_t<T, ListA, ListB>: the type of ListB at the
+// position T has in ListA.  Interface counterpart: FK/core/utils/type_lists.h.
+template <typename T, typename TL> struct one_of;
+template <typename T, typename... Ts> struct one_of<T, TypeList<Ts...>> : std::bool_constant<(std::is_same_v<T, Ts> || ...)> {};
+template <typename T, typename TL> constexpr bool one_of_v = one_of<T, TL>::value;
+template <typename T, typename TL1, typename TL2> struct EquivalentType;
+template <typename T, typename A, typename... As, typename B, typename... Bs> struct EquivalentType<T, TypeList<A, As...>, TypeList<B, Bs...>> {
+    static_assert(sizeof...(As) == sizeof...(Bs), "the two lists must have the same length");
+    using type = typename std::conditional_t<std::is_same_v<T, A>, std::type_identity<B>, EquivalentType<T, TypeList<As...>, TypeList<Bs...>>>::type;
+};
+template <typename T> struct EquivalentType<T, TypeList<>, TypeList<>> { using type = void; };
+template <typename T, typename TL1, typename TL2> using EquivalentType_t = typename EquivalentType<T, TL1, TL2>::type;
 
 namespace op_detail {
 template <typename T, typename = void> struct has_instance : std::false_type {};

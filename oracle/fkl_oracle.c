@@ -709,6 +709,18 @@ int fklo_execute(int32_t n_planes, const fklo_read *reads,
     return FKLO_OK;
 }
 
+/* computeCircularThreadIdx<direction, BATCH>, FK/algorithms/basic_ops/memory_operations.h:422-432. */
+int32_t fklo_circular_plane(int32_t direction, int32_t batch, int32_t z, int32_t first) {
+    if (direction == 0) { const int32_t c = z + first; return c >= batch ? c - batch : c; }
+    const int32_t c = first - z;
+    return c < 0 ? batch + c : c;
+}
+/* SequenceSelectorType<CTO, BATCH>::at, FK/core/data/circular_tensor.h:26-35. */
+int32_t fklo_window_sequence(int32_t order, int32_t batch, int32_t z) {
+    if (order == 0) return z > 0 ? 1 : 0;
+    return z != batch - 1 ? 1 : 0;
+}
+
 /* ---- synthetic inputs: std::mt19937 ------------------------------------ */
 
 void fklo_mt_seed(fklo_mt19937 *g, uint32_t seed) {

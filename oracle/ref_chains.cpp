@@ -20,6 +20,8 @@
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
+#include <fused_kernel/core/data/circular_tensor.h>
+#include <fused_kernel/core/data/ptr_utils.h>
 
 #include <array>
 #include <cstdint>
@@ -29,6 +31,7 @@
 // headers, compiled here against the reference's.
 #include "../tests/cases/color_chains.h"
 #include "../tests/cases/border_chains.h"
+#include "../tests/cases/circular_chains.h"
 
 using namespace fk;
 using CpuDPP = TransformDPP<ParArch::CPU>;
@@ -406,3 +409,23 @@ extern "C" int fklref_pad(int elem, int border_type, const void* src, int w, int
     s.sync();
     return rc;
 }
+
+// ---- divergent launches and the CircularTensor window (tests/cases/circular_chains.h on the reference's CPU backend) ----
+extern "C" {
+int fklref_divergent_two(const uint32_t* a, const uint32_t* b, int w, int h, int pitch, uint32_t add, uint32_t* out) {
+    CpuStream s;
+    circular_chains::Chains<ParArch::CPU>::divergent_two(s, MemType::Host, a, b, w, h, pitch, add, out);
+    s.sync();
+    return 0;
+}
+int fklref_divergent_mixed(const float* tensor4, int w, int h, float mul, const uint8_t* img, int iw, int ih, int ipitch, float* out) {
+    CpuStream s;
+    circular_chains::Chains<ParArch::CPU>::divergent_mixed(s, MemType::Host, tensor4, w, h, mul, img, iw, ih, ipitch, out);
+    s.sync();
+    return 0;
+}
+int fklref_circular(int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch, float fill, float* states) {
+    CpuStream s;
+    return circular_chains::Chains<ParArch::CPU>::circular(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Host, fill, states);
+}
+} // extern "C"

@@ -18,6 +18,7 @@
 #include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/algorithms/image_processing/image.h>
 #include <fused_kernel/fused_kernel.h>
+#include <fused_kernel/core/data/circular_tensor.h>
 
 #include <array>
 #include <cstdint>
@@ -28,6 +29,7 @@
 
 #include "color_chains.h"   // pixel-format and colour-conversion chains, shared with the reference-backend harness
 #include "border_chains.h"  // padding chains, shared the same way
+#include "circular_chains.h"  // divergent launches and the CircularTensor window, shared the same way
 
 using namespace fk;
 
@@ -469,3 +471,21 @@ extern "C" int fklcase_pad(void* stream_, int elem, int border_type, const void*
                                                                   out_h, value, out, out_pitch);
     });
 }
+
+// ---- divergent launches and the CircularTensor window (circular_chains.h on the GPU) -------------------------------
+extern "C" {
+int fklcase_divergent_two(void* stream_, const uint32_t* a, const uint32_t* b, int w, int h, int pitch, uint32_t add, uint32_t* out) {
+    return guarded([&] { Stream s(stream_); circular_chains::Chains<ParArch::GPU_AMD>::divergent_two(s, MemType::Device, a, b, w, h, pitch, add, out); });
+}
+int fklcase_divergent_mixed(void* stream_, const float* tensor4, int w, int h, float mul, const uint8_t* img, int iw, int ih, int ipitch, float* out) {
+    return guarded([&] { Stream s(stream_); circular_chains::Chains<ParArch::GPU_AMD>::divergent_mixed(s, MemType::Device, tensor4, w, h, mul, img, iw, ih, ipitch, out); });
+}
+// images: `iters` device pointers to uchar3 images; states: host memory, iters x batch x 3 x h x w floats
+int fklcase_circular(void* stream_, int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch, float fill,
+                     float* states) {
+    return guarded_rc([&] {
+        Stream s(stream_);
+        return circular_chains::Chains<ParArch::GPU_AMD>::circular(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Device, fill, states);
+    });
+}
+} // extern "C"

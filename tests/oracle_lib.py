@@ -648,3 +648,85 @@ def ref_pad(src, border_type, left, top, out_w, out_h, value=(0, 0, 0)):
                           int(left), int(top), int(out_w), int(out_h), _f32p(v), C.c_void_p(_ptr(out)), out.strides[0])
     assert rc == 0, rc
     return out
+
+
+# ---- divergent launches and the CircularTensor window -----------------------------------------------------------
+# A DivergentBatchTransformDPP launch is, plane by plane, an ordinary chain (data_parallel_patterns.h:322-331): the
+# helpers below pick the sequence of each plane and let the C oracle run that plane's chain.
+
+def oracle_divergent_mixed(tensor4, mul, img):
+    """tensor4 (4,h,w,3) f32; planes 0 and 3: tensor plane * mul; planes 1 and 2: img (ih,iw,3) u8 resized to (w,h)."""
+    _, h, w, _ = tensor4.shape
+    out = np.zeros((4, h, w, 3), np.float32)
+    for z in range(4):
+        if z in (0, 3):
+            execute([read_2d(tensor4[z], 3)], [op(MUL, [mul])], [write(WRITE_2D, out[z], 3, w, h)])
+        else:
+            execute([read_2d(img, 3, resize=(w, h))], [], [write(WRITE_2D, out[z], 3, w, h)])
+    return out
+
+
+def ref_divergent_two(a, b, add):
+    h, w = a.shape
+    out = np.zeros((2, h, w), np.uint32)
+    assert ref().fklref_divergent_two(C.c_void_p(_ptr(a)), C.c_void_p(_ptr(b)), w, h, a.strides[0], C.c_uint32(add), C.c_void_p(_ptr(out))) == 0
+    return out
+
+
+def ref_divergent_mixed(tensor4, mul, img):
+    _, h, w, _ = tensor4.shape
+    out = np.zeros((4, h, w, 3), np.float32)
+    assert ref().fklref_divergent_mixed(C.c_void_p(_ptr(tensor4)), w, h, C.c_float(mul), C.c_void_p(_ptr(img)), img.shape[1], img.shape[0],
+                                        img.strides[0], C.c_void_p(_ptr(out))) == 0
+    return out
+
+
+class OracleWindow:
+    """CircularTensor<float, 3, batch, order, Standard> restated (circular_tensor.h:111-161): `out` is the tensor the
+    caller sees (batch, 3, h, w), `temp` the hidden circular copy, whose planes hold nothing defined (NaN here)
+    until an update has stored into them."""
+
+    def __init__(self, batch, oldest_first, w, h, fill):
+        self.batch, self.order, self.w, self.h = batch, int(bool(oldest_first)), w, h
+        self.out = np.full((batch, 3, h, w), fill, np.float32)
+        self.temp = np.full((batch, 3, h, w), np.nan, np.float32)
+        self.next = 0
+        lib = oracle()
+        lib.fklo_circular_plane.restype = C.c_int32
+        lib.fklo_circular_plane.argtypes = [C.c_int32] * 4
+        lib.fklo_window_sequence.restype = C.c_int32
+        lib.fklo_window_sequence.argtypes = [C.c_int32] * 3
+
+    def update(self, img):
+        """img (h,w,3) u8 -> SaturateCast<uchar3, float3> -> TensorSplit."""
+        lib = oracle()
+        value = np.zeros((1, 3, self.h, self.w), np.float32)
+        execute([read_2d(img, 3)], [op(CAST_F32)], [write(TENSOR_SPLIT, value, 3, self.w, self.h, 1, 3)])
+        read_dir = 0 if self.order == 1 else 1            # OldestFirst reads Ascendent, NewestFirst Descendent
+        new = self.out.copy()
+        for z in range(self.batch):
+            if lib.fklo_window_sequence(self.order, self.batch, z) == 0:
+                self.temp[lib.fklo_circular_plane(0, self.batch, z, self.next)] = value[0]      # MidWrite, Ascendent
+                new[z] = value[0]
+        for z in range(self.batch):
+            if lib.fklo_window_sequence(self.order, self.batch, z) == 1:
+                new[z] = self.temp[lib.fklo_circular_plane(read_dir, self.batch, z, self.next)]
+        self.out = new
+        self.next = (self.next + 1) % self.batch
+        return self.out
+
+
+def oracle_circular(batch, oldest_first, images, fill):
+    """States after each update, (iters, batch, 3, h, w); planes copied from never-written hidden planes are NaN."""
+    h, w = images[0].shape[:2]
+    win = OracleWindow(batch, oldest_first, w, h, fill)
+    return np.stack([win.update(img).copy() for img in images])
+
+
+def ref_circular(batch, oldest_first, images, fill):
+    h, w = images[0].shape[:2]
+    states = np.zeros((len(images), batch, 3, h, w), np.float32)
+    ptrs = (C.c_void_p * len(images))(*[_ptr(i) for i in images])
+    rc = ref().fklref_circular(batch, int(bool(oldest_first)), ptrs, len(images), w, h, images[0].strides[0], C.c_float(fill), C.c_void_p(_ptr(states)))
+    assert rc == 0, rc
+    return states
