@@ -163,6 +163,9 @@ __device__ __forceinline__ void rows_auto_body(const typename Chain::Params& p, 
 #ifndef FKD_GATHER_BY
 #define FKD_GATHER_BY 4
 #endif
+#ifndef FKD_GATHER_DEPTH
+#define FKD_GATHER_DEPTH 2
+#endif
 constexpr int kGatherBX = 64;
 constexpr int kGatherBY = FKD_GATHER_BY;
 
@@ -273,11 +276,21 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     //   kSingles  one access per tap, whole dwords;
     //   kSafe     one access per tap, never touching a byte outside the elements (channel by channel for 3- and
     //             6-byte elements): for waves whose taps reach the last row of the image.
-    constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3;
+    //   kPairsPrepared  kPairs for images whose rows all start at the same offset inside their dword (pitch a multiple
+    //             of 4): the image is a buffer resource, a row a scalar offset, and the lane's window offset and byte
+    //             shift are worked out once per column instead of once per tap;
+    constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3, kPairsPrepared = 4;
     const int yend = y0 + YI < ah ? y0 + YI : ah;
     auto rows = [&](auto mode_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
-        constexpr bool PAIRED = MODE == kPairs || MODE == kPairsSel;
+        constexpr bool PAIRED = MODE == kPairs || MODE == kPairsSel || MODE == kPairsPrepared;
+        detail::PairPrep prep[XI];
+        detail::TapImage image;
+        if constexpr (MODE == kPairsPrepared) {
+            image = Back::tap_image(z, q.back);
+#pragma unroll
+            for (int i = 0; i < XI; ++i) prep[i] = Back::pair_prepare(image, x1[i], q.back);
+        }
         struct RowTaps {
             typename Back::TapBits a[PAIRED ? 1 : XI], b[PAIRED ? 1 : XI], c[PAIRED ? 1 : XI], d[PAIRED ? 1 : XI];
             typename Back::PairBits ab[PAIRED ? XI : 1], cd[PAIRED ? XI : 1];
@@ -293,11 +306,19 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
             const int yi = __builtin_amdgcn_readfirstlane(int(f1));
             const int ya = yi < 0 ? 0 : (yi < sh - 1 ? yi : sh - 1);
             const int yb = ya + 1 < sh - 1 ? ya + 1 : sh - 1;
-            t.ra = Back::tap_row(0, ya, z, q.back);
-            t.rb = Back::tap_row(0, yb, z, q.back);
+            if constexpr (MODE != kPairsPrepared) {
+                t.ra = Back::tap_row(0, ya, z, q.back);
+                t.rb = Back::tap_row(0, yb, z, q.back);
+            } else {
+                t.ra = typename Back::TapRow{};     // rows are scalar offsets into the image's buffer resource
+                t.rb = typename Back::TapRow{};
+            }
 #pragma unroll
             for (int i = 0; i < XI; ++i) {
-                if constexpr (PAIRED) {
+                if constexpr (MODE == kPairsPrepared) {
+                    t.ab[i] = Back::pair_load_prepared(image, Back::tap_row_offset(ya, q.back), prep[i], q.back);
+                    t.cd[i] = Back::pair_load_prepared(image, Back::tap_row_offset(yb, q.back), prep[i], q.back);
+                } else if constexpr (PAIRED) {
                     const int xl = MODE == kPairsSel ? x1[i] - int(clamped[i]) : x1[i];
                     t.ab[i] = Back::pair_load(t.ra, xl, q.back);
                     t.cd[i] = Back::pair_load(t.rb, xl, q.back);
@@ -346,14 +367,30 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
                 for (int i = 0; i < XI; ++i) if (xof(i) < aw) WP::put(orow, xof(i), res[i].v);
             }
         };
-        RowTaps t0, t1;
-        request(y0, t0);
+        if constexpr (FKD_GATHER_DEPTH <= 2) {
+            RowTaps t0, t1;
+            request(y0, t0);
 #pragma unroll 1
-        for (int y = y0; y < yend; y += 2) {
-            if (y + 1 < yend) request(y + 1, t1);      // wave uniform
-            produce(y, t0);
-            if (y + 2 < yend) request(y + 2, t0);
-            produce(y + 1, t1);
+            for (int y = y0; y < yend; y += 2) {
+                if (y + 1 < yend) request(y + 1, t1);      // wave uniform
+                produce(y, t0);
+                if (y + 2 < yend) request(y + 2, t0);
+                produce(y + 1, t1);
+            }
+        } else {
+            // A ring of DEPTH tap sets: DEPTH - 1 rows of loads stay in flight behind the row being blended.
+            constexpr int D = FKD_GATHER_DEPTH;
+            RowTaps t[D];
+#pragma unroll
+            for (int k = 0; k < D - 1; ++k) if (y0 + k < yend) request(y0 + k, t[k]);
+#pragma unroll 1
+            for (int y = y0; y < yend; y += D) {
+#pragma unroll
+                for (int k = 0; k < D; ++k) {
+                    if (y + k + D - 1 < yend) request(y + k + D - 1, t[(k + D - 1) % D]);
+                    produce(y + k, t[k]);
+                }
+            }
         }
     };
     // Whole-dword reads of 3- and 6-byte elements (and pair reads) touch up to 3 bytes past what they need.  Inside
@@ -369,7 +406,13 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
         rows(IntTag<kSafe>{});
     } else {
         if constexpr (Back::kTapPair) {
-            if (!any_clamped) { rows(IntTag<kPairs>{}); return; }
+            if (!any_clamped) {
+                if constexpr (detail::tap_prepared<Back>()) {
+                    if (Back::tap_rows_share_alignment(q.back)) { rows(IntTag<kPairsPrepared>{}); return; }
+                }
+                rows(IntTag<kPairs>{});
+                return;
+            }
             if (sw >= 2) { rows(IntTag<kPairsSel>{}); return; }
         }
         rows(IntTag<kSingles>{});

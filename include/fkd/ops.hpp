@@ -315,6 +315,54 @@ template <class T> FKD_DEV PairWindow<T> load_pair_window(const char* row, u32 o
     else { const u32x4_t v = *gconst<u32x4_a4>(a); p.w[0] = v.x; p.w[1] = v.y; p.w[2] = v.z; p.w[3] = v.w; }
     return p;
 }
+// The same window through a buffer resource, for images whose rows all start at the same offset inside their dword
+// (pitch a multiple of 4) and that are smaller than 4 GB.  The image is described once per wave as a raw buffer
+// starting at the dword at or below its first byte; a row is then a 32-bit SCALAR byte offset and a column a 32-bit
+// per-lane one (window start and bytes to drop, prepared once per column because they no longer depend on the row), so
+// a tap costs one buffer_load with no address arithmetic at all.  The resource's size field is left open: staying
+// inside the allocation is the caller's business exactly as for the global-memory loads.
+struct PairPrep { u32 off, shift; };
+template <class B> constexpr bool tap_prepared() {
+    if constexpr (requires { B::kTapPrepared; }) return B::kTapPrepared; else return false;
+}
+struct TapImage {
+#if defined(FKD_DEVICE_CODE)
+    __amdgpu_buffer_rsrc_t rsrc;
+#endif
+    u32 lo;       // bytes between the resource's base and the image's first byte
+};
+#if defined(FKD_DEVICE_CODE)
+FKD_DEV TapImage make_tap_image(const void* data) {
+    TapImage im;
+    im.lo = u32(reinterpret_cast<uintptr_t>(data)) & 3u;
+    // word 3 = 0x00020000: 32-bit raw data format of the gfx9 family, no swizzle, no index stride
+    im.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(data)) - im.lo, 0, 0xffffffffu, 0x00020000);
+    return im;
+}
+template <class T> FKD_DEV PairPrep prepare_pair_window(const TapImage& im, u32 off) {
+    PairPrep pp;
+    if constexpr (PairWindow<T>::kShift) {
+        off += im.lo;
+        pp.shift = off & 3u;
+        pp.off = off & ~3u;
+    } else {
+        pp.shift = 0;
+        pp.off = off + im.lo;
+    }
+    return pp;
+}
+template <class T> FKD_DEV PairWindow<T> load_prepared_pair_window(const TapImage& im, u32 row_off, const PairPrep& pp) {
+    using PW = PairWindow<T>;
+    PW p;
+    p.shift = pp.shift;
+    constexpr int W = PW::kWords;
+    if constexpr (W == 1) { p.w[0] = __builtin_amdgcn_raw_buffer_load_b32(im.rsrc, pp.off, row_off, 0); }
+    else if constexpr (W == 2) { const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(im.rsrc, pp.off, row_off, 0); p.w[0] = v.x; p.w[1] = v.y; }
+    else if constexpr (W == 3) { const u32x3_t v = __builtin_amdgcn_raw_buffer_load_b96(im.rsrc, pp.off, row_off, 0); p.w[0] = v.x; p.w[1] = v.y; p.w[2] = v.z; }
+    else { const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(im.rsrc, pp.off, row_off, 0); p.w[0] = v.x; p.w[1] = v.y; p.w[2] = v.z; p.w[3] = v.w; }
+    return p;
+}
+#endif
 template <class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& first, T& second) {
     using PW = PairWindow<T>;
     u32 v[PW::kOut];
@@ -924,6 +972,20 @@ template <class T> struct Read2D {
     FKD_DEV static void pair_values(const PairBits& b, const TapRow&, int, Raw& first, Raw& second) {
         detail::pair_window_values<T>(b, first, second);
     }
+    // Buffer-resource form of pair_load for images whose rows share their alignment (see detail::TapImage): the image
+    // once per wave, a prepared column once per lane, a scalar offset per row.
+    static constexpr bool kTapPrepared = true;
+    FKD_DEV static bool tap_rows_share_alignment(const Params& p) { return p.pitch % 4 == 0 && size_t(p.pitch) * p.height < 0xfffffff0ull; }
+    using TapImage = detail::TapImage;
+    using PairPrep = detail::PairPrep;
+    FKD_DEV static TapImage tap_image(int, const Params& p) { return detail::make_tap_image(p.data); }
+    FKD_DEV static u32 tap_row_offset(int y, const Params& p) { return u32(y) * p.pitch; }
+    FKD_DEV static PairPrep pair_prepare(const TapImage& im, int x, const Params&) {
+        return detail::prepare_pair_window<T>(im, u32(x) * u32(sizeof(T)));
+    }
+    FKD_DEV static PairBits pair_load_prepared(const TapImage& im, u32 row_off, const PairPrep& pp, const Params&) {
+        return detail::load_prepared_pair_window<T>(im, row_off, pp);
+    }
 #endif
 };
 
@@ -1202,6 +1264,24 @@ template <class Back> struct Crop {
     using PairBits = typename Back::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
+    static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
+    FKD_DEV static bool tap_rows_share_alignment(const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_rows_share_alignment(p.back); else return false;
+    }
+    using TapImage = detail::TapImage;
+    using PairPrep = detail::PairPrep;
+    FKD_DEV static TapImage tap_image(int z, const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_image(z, p.back); else return TapImage{};
+    }
+    FKD_DEV static u32 tap_row_offset(int y, const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_row_offset(y + p.y, p.back); else return 0u;
+    }
+    FKD_DEV static PairPrep pair_prepare(const TapImage& im, int x, const Params& p) {
+        if constexpr (kTapPrepared) return Back::pair_prepare(im, x + p.x, p.back); else return PairPrep{};
+    }
+    FKD_DEV static PairBits pair_load_prepared(const TapImage& im, u32 row_off, const PairPrep& pp, const Params& p) {
+        if constexpr (kTapPrepared) return Back::pair_load_prepared(im, row_off, pp, p.back); else return PairBits{};
+    }
 #endif
 };
 
@@ -1295,6 +1375,24 @@ template <class Back, class... Ops> struct FusedRead {
     using PairBits = typename Back::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
+    static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
+    FKD_DEV static bool tap_rows_share_alignment(const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_rows_share_alignment(p.back); else return false;
+    }
+    using TapImage = detail::TapImage;
+    using PairPrep = detail::PairPrep;
+    FKD_DEV static TapImage tap_image(int z, const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_image(z, p.back); else return TapImage{};
+    }
+    FKD_DEV static u32 tap_row_offset(int y, const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_row_offset(y, p.back); else return 0u;
+    }
+    FKD_DEV static PairPrep pair_prepare(const TapImage& im, int x, const Params& p) {
+        if constexpr (kTapPrepared) return Back::pair_prepare(im, x, p.back); else return PairPrep{};
+    }
+    FKD_DEV static PairBits pair_load_prepared(const TapImage& im, u32 row_off, const PairPrep& pp, const Params& p) {
+        if constexpr (kTapPrepared) return Back::pair_load_prepared(im, row_off, pp, p.back); else return PairBits{};
+    }
 #endif
 };
 
