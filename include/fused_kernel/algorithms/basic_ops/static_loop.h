@@ -1,5 +1,6 @@
 // StaticLoop<Operation, ITERATIONS>: a Binary operation that applies Operation ITERATIONS times with the same
-// parameters.  Interface counterpart: FK/algorithms/basic_ops/static_loop.h:21-44.
+// parameters -- and once for ITERATIONS = 0, as the reference does (its first application is unconditional).
+// Interface counterpart: FK/algorithms/basic_ops/static_loop.h:21-44.
 #ifndef FK_AMD_STATIC_LOOP_H
 #define FK_AMD_STATIC_LOOP_H
 
@@ -13,7 +14,7 @@ struct StaticLoop : BinaryOperation<typename Operation::InputType, typename Oper
     using Parent = BinaryOperation<typename Operation::InputType, typename Operation::ParamsType, typename Operation::OutputType,
                                    StaticLoop<Operation, ITERATIONS>>;
     FK_STATIC_STRUCT(StaticLoop, StaticLoop)
-    static_assert(ITERATIONS >= 1, "StaticLoop needs at least one iteration");
+    static_assert(ITERATIONS >= 0, "StaticLoop cannot run a negative number of iterations");
     static_assert(std::is_same_v<typename Operation::InputType, typename Operation::OutputType>,
                   "the looped operation must map a type onto itself");
 };
@@ -21,7 +22,7 @@ struct StaticLoop : BinaryOperation<typename Operation::InputType, typename Oper
 namespace amd {
 template <typename Operation, int ITERATIONS> struct Lower<StaticLoop<Operation, ITERATIONS>> {
     static constexpr bool available = Lower<Operation>::available;
-    using type = fkd::StaticLoop<typename Lower<Operation>::type, ITERATIONS>;
+    using type = fkd::StaticLoop<typename Lower<Operation>::type, (ITERATIONS < 1 ? 1 : ITERATIONS)>;
     static typename type::Params params(const OperationData<StaticLoop<Operation, ITERATIONS>>& d) {
         return Lower<Operation>::params(OperationData<Operation>{d.params});
     }

@@ -7,6 +7,7 @@
 #include <atomic>
 #include <cstdlib>
 #include <stdexcept>
+#include <vector>
 #include <type_traits>
 
 #include <fused_kernel/core/data/rawptr.h>

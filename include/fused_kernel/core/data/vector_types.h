@@ -13,7 +13,21 @@ namespace fk {
     struct Name##3 { T x, y, z; };                                  \
     struct alignas(A4) Name##4 { T x, y, z, w; };
 
-FK_AMD_VEC_FAMILY(Bool, bool, 2, 4)
+// Results of channel-wise comparisons; in a boolean context a BoolN is true when every channel is.
+struct Bool1 { bool x; constexpr operator bool() const { return x; } };
+struct alignas(2) Bool2 { bool x, y; constexpr operator bool() const { return x && y; } };
+struct Bool3 { bool x, y, z; constexpr operator bool() const { return x && y && z; } };
+struct alignas(4) Bool4 { bool x, y, z, w; constexpr operator bool() const { return x && y && z && w; } };
+struct Bool {
+    static constexpr bool vAnd(const Bool1& b) { return b.x; }
+    static constexpr bool vAnd(const Bool2& b) { return b.x && b.y; }
+    static constexpr bool vAnd(const Bool3& b) { return b.x && b.y && b.z; }
+    static constexpr bool vAnd(const Bool4& b) { return b.x && b.y && b.z && b.w; }
+    static constexpr bool vOr(const Bool1& b) { return b.x; }
+    static constexpr bool vOr(const Bool2& b) { return b.x || b.y; }
+    static constexpr bool vOr(const Bool3& b) { return b.x || b.y || b.z; }
+    static constexpr bool vOr(const Bool4& b) { return b.x || b.y || b.z || b.w; }
+};
 FK_AMD_VEC_FAMILY(Char, signed char, 2, 4)
 FK_AMD_VEC_FAMILY(Uchar, unsigned char, 2, 4)
 FK_AMD_VEC_FAMILY(Short, short, 4, 8)

@@ -109,15 +109,17 @@ constexpr bool vec_operands = (isVector<A> || isVector<B>) && (!isVector<A> || !
     }
 FK_AMD_VEC_OP(+) FK_AMD_VEC_OP(-) FK_AMD_VEC_OP(*) FK_AMD_VEC_OP(/)
 #undef FK_AMD_VEC_OP
-template <typename A, typename B, std::enable_if_t<fk::vec_detail::vec_operands<A, B> && fk::isVector<A> && fk::isVector<B>, int> = 0>
-constexpr bool operator==(const A& a, const B& b) {
-    bool eq = fk::vectorAt<0>(a) == fk::vectorAt<0>(b);
-    if constexpr (fk::cn<A> > 1) eq = eq && a.y == b.y;
-    if constexpr (fk::cn<A> > 2) eq = eq && a.z == b.z;
-    if constexpr (fk::cn<A> > 3) eq = eq && a.w == b.w;
-    return eq;
-}
-template <typename A, typename B, std::enable_if_t<fk::vec_detail::vec_operands<A, B> && fk::isVector<A> && fk::isVector<B>, int> = 0>
-constexpr bool operator!=(const A& a, const B& b) { return !(a == b); }
+// Comparisons and logical operators are channel-wise too and yield a boolN, which converts to bool as "all channels".
+#define FK_AMD_VEC_CMP(op)                                                                                         \
+    template <typename A, typename B, std::enable_if_t<fk::vec_detail::vec_operands<A, B>, int> = 0>               \
+    constexpr auto operator op(const A& a, const B& b) {                                                           \
+        constexpr int N = fk::isVector<A> ? fk::cn<A> : fk::cn<B>;                                                 \
+        using O = typename fk::VectorType<bool, N>::type_v;                                                        \
+        const auto r = fk::vec_detail::zip(a, b, [](auto x, auto y) -> bool { return x op y; });                   \
+        if constexpr (N == 1) return O{fk::vectorAt<0>(r)}; else return r;                                         \
+    }
+FK_AMD_VEC_CMP(==) FK_AMD_VEC_CMP(!=) FK_AMD_VEC_CMP(<) FK_AMD_VEC_CMP(>) FK_AMD_VEC_CMP(<=) FK_AMD_VEC_CMP(>=)
+FK_AMD_VEC_CMP(&&) FK_AMD_VEC_CMP(||)
+#undef FK_AMD_VEC_CMP
 
 #endif

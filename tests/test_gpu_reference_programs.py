@@ -1,0 +1,52 @@
+"""The reference library's OWN test and benchmark programs, compiled unchanged from the reference tree against this
+repository's headers and libfklhip.so (oracle/Makefile, target `programs`), run on the GPU through this backend.
+
+Each program checks its results itself (the tests compare against values computed on the host, the benchmarks compare
+the two executions they time) and reports through its exit code.  The programs are built where the reference tree is
+present and travel as binaries; where they are missing the tests are skipped."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROGRAMS = os.path.join(ROOT, "oracle", "_ref", "programs")
+
+TESTS = ["tests_algorithm_test_crop", "tests_algorithm_test_batchresize_build", "tests_algorithm_test_deinterlace",
+         "tests_algorithm_test_warp", "tests_algorithm_test_border_reader", "tests_data_test_ptr_nd", "tests_data_test_rect",
+         "tests_data_test_circular_tensor", "tests_data_parallel_patterns_test_divergent_batch",
+         "tests_examples_compiler_explorer_example", "tests_buildAPI_batch_build_compilation_time"]
+BENCHMARKS = ["benchmarks_fusion_benchmark_horizontal_fusion", "benchmarks_fusion_benchmark_thread_fusion",
+              "benchmarks_latencyhiding_benchmark_latency_hiding", "benchmarks_numinstructions_benchmark_numinstructions_x_operation"]
+
+
+def run_program(name, tmp_path):
+    exe = os.path.join(PROGRAMS, name)
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/programs was not built (needs the reference tree at build time)")
+    r = subprocess.run([exe], cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, f"{name} exited with {r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
+    return r.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", TESTS)
+def test_reference_test_program_passes(device, name, tmp_path):
+    out = run_program(name, tmp_path)
+    assert "Failed" not in out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", BENCHMARKS)
+def test_reference_benchmark_program_runs_and_checks_out(device, name, tmp_path):
+    out = run_program(name, tmp_path)
+    assert "Mismatch" not in out and "Failed" not in out
+    # every benchmark leaves its table(s) for this architecture
+    assert any(f.endswith("_GPU_AMD.csv") for f in os.listdir(tmp_path))
+
+
+def test_reference_programs_are_built_where_the_reference_tree_is():
+    if not os.path.isdir("/root/reference/tests"):
+        pytest.skip("no reference tree here")
+    missing = [n for n in TESTS + BENCHMARKS if not os.path.exists(os.path.join(PROGRAMS, n))]
+    assert not missing, f"run __graft_entry__.build(): not built: {missing}"
