@@ -777,6 +777,22 @@ template <class I> struct AddLast {
     }
 };
 
+// VectorReduce<T, Operation>: the channels of the input folded left to right with a binary operation,
+// op(op(x, y), z): FK/algorithms/basic_ops/vector_ops.h:82-92 -> cxp::vector_reduce, FK/core/constexpr_libs/
+// constexpr_vector.h:94-110.  BinOp is one of Add/Sub/Mul on scalars (its parameter is the right-hand operand).
+template <class T, class BinOp> struct VectorReduce {
+    static_assert(cn_v<T> >= 2 && cn_v<typename BinOp::In> == 1 && cn_v<typename BinOp::Out> == 1, "a vector in, a scalar operation");
+    using In = T; using Out = typename BinOp::Out; using Params = Empty;
+    FKD_NAME("VectorReduce<" + type_name<T>() + "," + BinOp::name() + ">")
+    FKD_DEV static Out exec(const T& a, const Params&) {
+        using P = typename BinOp::Params;
+        Out r = BinOp::exec(a.x, P{a.y});
+        if constexpr (cn_v<T> > 2) r = BinOp::exec(r, P{a.z});
+        if constexpr (cn_v<T> > 3) r = BinOp::exec(r, P{a.w});
+        return r;
+    }
+};
+
 // Discard<I, O>: the first cn<O> channels of the input.  FK/algorithms/basic_ops/vector_ops.h:22-41.
 template <class I, class O> struct Discard {
     static_assert(cn_v<I> > cn_v<O> && __is_same(base_t<I>, base_t<O>), "fewer channels out, same sample type");

@@ -23,7 +23,17 @@ template <typename I, typename O> struct AddLast : BinaryOperation<I, VBase<I>, 
     static_assert(cn<I> == cn<O> - 1, "Output type should have one channel more");
     static_assert(std::is_same_v<VBase<I>, VBase<O>>, "Base types should be the same");
 };
+// The channels of the input folded left to right with a binary Operation on scalars: op(op(x, y), z).
+template <typename T, typename Operation> struct VectorReduce : UnaryOperation<T, typename Operation::OutputType, VectorReduce<T, Operation>> {
+    using Parent = UnaryOperation<T, typename Operation::OutputType, VectorReduce<T, Operation>>;
+    FK_STATIC_STRUCT(VectorReduce, VectorReduce)
+};
 namespace amd {
+template <typename T, typename Operation> struct Lower<VectorReduce<T, Operation>> {
+    static constexpr bool available = Lower<Operation>::available;
+    using type = fkd::VectorReduce<dev_t<T>, typename Lower<Operation>::type>;
+    static typename type::Params params(const OperationData<VectorReduce<T, Operation>>&) { return {}; }
+};
 template <typename I, typename O> struct Lower<Discard<I, O>> {
     static constexpr bool available = true;
     using type = fkd::Discard<dev_t<I>, dev_t<O>>;
