@@ -1113,6 +1113,34 @@ template <int DIR, int BATCH, class Back> struct CircularRead {
 #endif
 };
 
+// CircularBatchRead<direction, Operation, BATCH>: FK/algorithms/basic_ops/memory_operations.h:434-474.  BATCH separate
+// reads used as a circular buffer: logical plane z is read number circular_plane(z).
+template <int DIR, int BATCH, class PlaneOp> struct CircularBatchRead {
+    using Out = typename PlaneOp::Out;
+    struct Params { i32 first; typename PlaneOp::Params plane[BATCH]; };
+    static constexpr bool kTapCursor = false;
+    FKD_NAME("CircularBatchRead<" + istr(DIR) + "," + istr(BATCH) + "," + PlaneOp::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static int width(const Params& p) { return PlaneOp::width(p.plane[0]); }
+    FKD_DEV static int height(const Params& p) { return PlaneOp::height(p.plane[0]); }
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        const int c = circular_plane<DIR, BATCH>(z, p.first);
+        return PlaneOp::exec(x, y, c, p.plane[c]);
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        const int c = circular_plane<DIR, BATCH>(z, p.first);
+        PlaneOp::template exec_row<V, A>(x, y, c, p.plane[c], out);
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) {
+        for (int i = 0; i < BATCH; ++i) if (!PlaneOp::rows_aligned(p.plane[i], xoff)) return false;
+        return true;
+    }
+    FKD_HD static bool plane_rows_aligned(const Params& p, int z, int xoff) {
+        return PlaneOp::rows_aligned(p.plane[circular_plane<DIR, BATCH>(z, p.first)], xoff);
+    }
+#endif
+};
+
 // ReadYUV<NV12> and ReadYUV<NV21>: FK/algorithms/image_processing/color_conversion.h:219-253.  Y from the luma
 // plane, the chroma pair from element x>>1 of chroma row y>>1; chroma base = data + pitch*height.  NV12 stores the
 // pair as (U,V), NV21 as (V,U) (template argument VU); the value is (Y,U,V) either way.
@@ -1907,6 +1935,28 @@ template <int DIR, int BATCH, class W> struct CircularWrite {
         W::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w);
     }
     FKD_HD static bool rows_aligned(const Params& p) { return W::rows_aligned(p.w); }
+#endif
+};
+
+// CircularBatchWrite<direction, Operation, BATCH>: FK/algorithms/basic_ops/memory_operations.h:476-503.
+template <int DIR, int BATCH, class W> struct CircularBatchWrite {
+    using In = typename W::In;
+    struct Params { i32 first; typename W::Params plane[BATCH]; };
+    FKD_NAME("CircularBatchWrite<" + istr(DIR) + "," + istr(BATCH) + "," + W::name() + ">")
+#if defined(FKD_DEVICE_CODE)
+    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) {
+        const int c = circular_plane<DIR, BATCH>(z, p.first);
+        W::exec(x, y, c, v, p.plane[c]);
+    }
+    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+        const int c = circular_plane<DIR, BATCH>(z, p.first);
+        W::template exec_row<V, A>(x, y, c, v, p.plane[c]);
+    }
+    FKD_HD static bool rows_aligned(const Params& p) {
+        for (int i = 0; i < BATCH; ++i) if (!W::rows_aligned(p.plane[i])) return false;
+        return true;
+    }
+    FKD_HD static bool plane_rows_aligned(const Params& p, int z) { return W::rows_aligned(p.plane[circular_plane<DIR, BATCH>(z, p.first)]); }
 #endif
 };
 

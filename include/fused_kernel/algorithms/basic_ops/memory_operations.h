@@ -1,7 +1,7 @@
 // Per-element memory operations: PerThreadRead / PerThreadWrite (pitched 1-D/2-D/3-D), TensorRead / TensorWrite,
 // TensorSplit (planar writer) and TensorPack (its reader), and the circular-buffer views CircularTensorRead /
 // CircularTensorWrite.  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:26-212, 243-290, 413-432,
-// 505-587.  The transposed-plane forms (TensorTSplit / TensorTPack) and CircularBatchRead/Write are not built.
+// 505-587.  CircularBatchRead / CircularBatchWrite (434-503) too.  The transposed-plane forms (TensorTSplit / TensorTPack) are not built.
 #ifndef FK_AMD_MEMORY_OPERATIONS_H
 #define FK_AMD_MEMORY_OPERATIONS_H
 
@@ -113,6 +113,37 @@ template <typename OperationDataTypeArray> struct CircularMemoryParams {
     OperationDataTypeArray opData;
 };
 
+// BATCH separate reads (or writes) used as a circular buffer: logical plane z is operation number (first +- z) mod BATCH.
+template <CircularDirection direction, typename Operation, int BATCH>
+struct CircularBatchRead : ReadOperation<typename Operation::ReadDataType, CircularMemoryParams<OperationData<Operation>[BATCH]>,
+                                         typename Operation::OutputType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
+                                         CircularBatchRead<direction, Operation, BATCH>> {
+    using Parent = ReadOperation<typename Operation::ReadDataType, CircularMemoryParams<OperationData<Operation>[BATCH]>,
+                                 typename Operation::OutputType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
+                                 CircularBatchRead<direction, Operation, BATCH>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(CircularBatchRead, CircularBatchRead)
+    static constexpr uint num_elems_x(const Point thread, const OperationDataType& opData) { return Operation::num_elems_x(thread, opData.params.opData[thread.z]); }
+    static constexpr uint num_elems_y(const Point thread, const OperationDataType& opData) { return Operation::num_elems_y(thread, opData.params.opData[thread.z]); }
+    static constexpr uint num_elems_z(const Point, const OperationDataType&) { return BATCH; }
+    static constexpr uint pitch(const Point thread, const OperationDataType& opData) { return Operation::pitch(thread, opData.params.opData[thread.z]); }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {num_elems_x(Point{0, 0, 0}, opData), num_elems_y(Point{0, 0, 0}, opData), uint(BATCH)};
+    }
+};
+template <CircularDirection direction, typename Operation, int BATCH>
+struct CircularBatchWrite : WriteOperation<typename Operation::InputType, CircularMemoryParams<OperationData<Operation>[BATCH]>,
+                                           typename Operation::WriteDataType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
+                                           CircularBatchWrite<direction, Operation, BATCH>> {
+    using Parent = WriteOperation<typename Operation::InputType, CircularMemoryParams<OperationData<Operation>[BATCH]>,
+                                  typename Operation::WriteDataType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
+                                  CircularBatchWrite<direction, Operation, BATCH>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(CircularBatchWrite, CircularBatchWrite)
+    static constexpr uint num_elems_x(const Point thread, const OperationDataType& opData) { return Operation::num_elems_x(thread, opData.params.opData[thread.z]); }
+    static constexpr uint pitch(const Point thread, const OperationDataType& opData) { return Operation::pitch(thread, opData.params.opData[thread.z]); }
+};
+
 template <CircularDirection direction, typename Operation, int BATCH>
 struct CircularTensorRead : ReadOperation<typename Operation::ReadDataType, CircularMemoryParams<OperationData<Operation>>,
                                           typename Operation::OutputType, Operation::THREAD_FUSION ? TF::ENABLED : TF::DISABLED,
@@ -149,6 +180,26 @@ template <typename T> struct Lower<TensorPack<T>> {
     using type = fkd::TensorPack<dev_t<T>>;
     static typename type::Params params(const OperationData<TensorPack<T>>& d) {
         return to_dev3<VBase<T>, const typename DevType<VBase<T>>::type>(d.params);
+    }
+};
+template <CircularDirection direction, typename Operation, int BATCH> struct Lower<CircularBatchRead<direction, Operation, BATCH>> {
+    static constexpr bool available = true;
+    using type = fkd::CircularBatchRead<int(direction), BATCH, typename Lower<Operation>::type>;
+    static typename type::Params params(const OperationData<CircularBatchRead<direction, Operation, BATCH>>& d) {
+        typename type::Params p{};
+        p.first = d.params.first;
+        for (int i = 0; i < BATCH; ++i) p.plane[i] = Lower<Operation>::params(d.params.opData[i]);
+        return p;
+    }
+};
+template <CircularDirection direction, typename Operation, int BATCH> struct Lower<CircularBatchWrite<direction, Operation, BATCH>> {
+    static constexpr bool available = true;
+    using type = fkd::CircularBatchWrite<int(direction), BATCH, typename Lower<Operation>::type>;
+    static typename type::Params params(const OperationData<CircularBatchWrite<direction, Operation, BATCH>>& d) {
+        typename type::Params p{};
+        p.first = d.params.first;
+        for (int i = 0; i < BATCH; ++i) p.plane[i] = Lower<Operation>::params(d.params.opData[i]);
+        return p;
     }
 };
 template <CircularDirection direction, typename Operation, int BATCH> struct Lower<CircularTensorRead<direction, Operation, BATCH>> {

@@ -16,7 +16,7 @@ TESTS = ["tests_algorithm_test_crop", "tests_algorithm_test_batchresize_build", 
          "tests_algorithm_test_warp", "tests_algorithm_test_border_reader", "tests_data_test_ptr_nd", "tests_data_test_rect",
          "tests_data_test_circular_tensor", "tests_data_parallel_patterns_test_divergent_batch",
          "tests_examples_compiler_explorer_example", "tests_buildAPI_batch_build_compilation_time",
-         "utests_core_execution_model_utest_executors"]
+         "tests_operation_test_cricular_batch", "utests_core_execution_model_utest_executors"]
 BENCHMARKS = ["benchmarks_fusion_benchmark_horizontal_fusion", "benchmarks_fusion_benchmark_thread_fusion",
               "benchmarks_latencyhiding_benchmark_latency_hiding", "benchmarks_numinstructions_benchmark_numinstructions_x_operation"]
 
