@@ -65,10 +65,16 @@ struct ResizeComplete : ReadBackOperation<typename BackIOp_::Operation::OutputTy
 };
 
 namespace resize_detail {
-// cxp::round of the reference at run time is std::round: half away from zero.
-inline int round_to_int(float v) { return static_cast<int>(std::round(v)); }
+// cxp::round of the reference is std::round (half away from zero); written out so that build() stays constexpr.
+// The operands here are letterbox sizes: non-negative and far below 2^23.
+constexpr int round_to_int(float v) {
+    const float a = v < 0.f ? -v : v;
+    const int t = static_cast<int>(a);
+    const int r = (a - static_cast<float>(t)) >= 0.5f ? t + 1 : t;
+    return v < 0.f ? -r : r;
+}
 
-template <AspectRatio AR> inline Size target_size(const Size& srcSize, const Size& dstSize) {
+template <AspectRatio AR> constexpr Size target_size(const Size& srcSize, const Size& dstSize) {
     const float scaleFactor = dstSize.height / (float)srcSize.height;
     const int targetHeight = dstSize.height;
     const int targetWidth = round_to_int(scaleFactor * srcSize.width);
@@ -112,7 +118,7 @@ struct Resize : IncompleteReadBackOperation<NullType, IncompleteResizeParams<AR,
 
     // Completion against the read behind it.
     template <typename NewBackIOp, std::enable_if_t<isOperation<NewBackIOp>, int> = 0>
-    static auto build(const NewBackIOp& backIOp, const InstantiableType& iOp) {
+    static constexpr auto build(const NewBackIOp& backIOp, const InstantiableType& iOp) {
         static_assert(isCompleteOperation<NewBackIOp>, "NewBackIOp must be a complete IOp");
         using NewDefaultType = float_<cn<typename NewBackIOp::Operation::OutputType>>;
         static_assert(std::is_same_v<NewDefaultType, DefaultType>, "Default value type and Op::OutputType must be the same.");
@@ -120,8 +126,8 @@ struct Resize : IncompleteReadBackOperation<NullType, IncompleteResizeParams<AR,
     }
 
     template <typename NewBackIOp, std::enable_if_t<isOperation<NewBackIOp>, int> = 0>
-    static auto build(const NewBackIOp& backIOp, const Size& dstSize,
-                      const VectorType_t<float, cn<typename NewBackIOp::Operation::OutputType>>& backgroundValue) {
+    static constexpr auto build(const NewBackIOp& backIOp, const Size& dstSize,
+                                const VectorType_t<float, cn<typename NewBackIOp::Operation::OutputType>>& backgroundValue) {
         static_assert(isCompleteOperation<NewBackIOp>, "NewBackIOp must be a complete IOp");
         const Size srcSize = NumElems::size(Point{0, 0, 0}, backIOp);
         const Size targetSize = resize_detail::target_size<AR>(srcSize, dstSize);
