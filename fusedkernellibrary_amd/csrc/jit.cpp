@@ -9,6 +9,10 @@
 //
 // The generated kernel takes the chain's parameter block by value followed by a TileGeom, and publishes a JitMeta
 // constant; the launcher below needs nothing else: the active grid is the first three words of the block.
+//
+// With the environment variable FKLHIP_JIT_CACHE naming a directory, compiled code objects are kept there and reused
+// by later processes.  A file's name is a hash of everything that went into it (signature, architecture, compiler
+// flags, the text of the embedded headers), so a library rebuilt from changed headers never picks up a stale kernel.
 #include <fklhip.h>
 #include "registry.hpp"
 #include <fkd/launch_info.hpp>
@@ -16,8 +20,10 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 
 #include <mutex>
 #include <string>
@@ -73,6 +79,51 @@ bool signature_is_clean(const char* s) {
         if (!ok) return false;
     }
     return true;
+}
+
+// ---- on-disk cache of code objects (opt in: FKLHIP_JIT_CACHE=<directory>) -----------------------------------------
+
+unsigned long long fnv1a(unsigned long long h, const char* data, size_t n) {
+    for (size_t i = 0; i < n; ++i) { h ^= static_cast<unsigned char>(data[i]); h *= 1099511628211ull; }
+    return h;
+}
+unsigned long long fnv1a(unsigned long long h, const std::string& s) { return fnv1a(fnv1a(h, s.data(), s.size()), "\0", 1); }
+
+// Path of the cache file for this signature on this architecture, or empty when the cache is off.
+std::string cache_path(const char* signature, const std::string& arch) {
+    const char* dir = getenv("FKLHIP_JIT_CACHE");
+    if (!dir || !dir[0]) return std::string();
+    unsigned long long a = fnv1a(14695981039346656037ull, std::string(signature));
+    unsigned long long b = fnv1a(0x9e3779b97f4a7c15ull, arch);
+    for (int i = 0; i < kJitFlagCount; ++i) b = fnv1a(b, std::string(kJitFlags[i]));
+    for (int i = 0; i < kJitHeaderCount; ++i) { b = fnv1a(b, std::string(kJitHeaderNames[i])); b = fnv1a(b, std::string(kJitHeaderTexts[i])); }
+    a = fnv1a(a, std::string(reinterpret_cast<const char*>(&b), sizeof(b)));
+    char name[64];
+    snprintf(name, sizeof(name), "/fklhip-%016llx%016llx.co", a, b);
+    return std::string(dir) + name;
+}
+bool read_file(const std::string& path, std::vector<char>* out) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) return false;
+    bool ok = false;
+    if (fseek(f, 0, SEEK_END) == 0) {
+        const long n = ftell(f);
+        if (n > 0 && fseek(f, 0, SEEK_SET) == 0) {
+            out->resize(size_t(n));
+            ok = fread(out->data(), 1, size_t(n), f) == size_t(n);
+        }
+    }
+    fclose(f);
+    return ok;
+}
+// Written under a private name and renamed into place, so a reader never sees half a file; failures are silent
+// (the cache is an optimisation).
+void write_file(const std::string& path, const std::vector<char>& data) {
+    const std::string tmp = path + ".tmp" + std::to_string(long(getpid()));
+    FILE* f = fopen(tmp.c_str(), "wb");
+    if (!f) return;
+    const bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
+    if (fclose(f) != 0 || !ok || rename(tmp.c_str(), path.c_str()) != 0) remove(tmp.c_str());
 }
 
 int get_function(JitKernel* k, hipFunction_t* fn) {
@@ -136,6 +187,75 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
 
 const char* jit_last_log() { return g_log.c_str(); }
 
+// Compile (or fetch from the cache directory) and register; the caller holds g_compile_mu.
+static int build_and_register(const char* signature, bool may_read_cache) {
+    const std::string arch_name = device_arch();
+    const std::string cached = cache_path(signature, arch_name);
+    JitKernel* k = new JitKernel();   // lives as long as the registry entry: for the life of the process
+    k->signature = signature;
+    const bool from_cache = may_read_cache && !cached.empty() && read_file(cached, &k->code);
+    if (!from_cache) {
+        std::string src = "#define FKD_DEVICE_CODE 1\n#define FKD_NO_NAMES 1\n#include \"fkd_kernels.hpp\"\nusing namespace fkd;\nusing JitChain = ";
+        src += signature;
+        src += ";\n"
+               "extern \"C\" __device__ const JitMeta fkd_jit_meta = jit_meta<JitChain>();\n"
+               "extern \"C\" __global__ __launch_bounds__(256) void fkd_jit_kernel(const JitChain::Params p, const TileGeom g) {\n"
+               "    jit_body<JitChain>(p, g);\n"
+               "}\n";
+        hiprtcProgram prog = nullptr;
+        hiprtcResult r = hiprtcCreateProgram(&prog, src.c_str(), "fkd_jit_chain.hip", kJitHeaderCount, kJitHeaderTexts, kJitHeaderNames);
+        if (r != HIPRTC_SUCCESS) { g_log = hiprtcGetErrorString(r); delete k; return FKLHIP_EUNKNOWN_SIGNATURE; }
+        const std::string arch = "--offload-arch=" + arch_name;
+        std::vector<const char*> opts;
+        opts.push_back(arch.c_str());
+        for (int i = 0; i < kJitFlagCount; ++i) opts.push_back(kJitFlags[i]);
+        r = hiprtcCompileProgram(prog, int(opts.size()), opts.data());
+        size_t log_size = 0;
+        if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {
+            g_log.resize(log_size);
+            hiprtcGetProgramLog(prog, &g_log[0]);
+        }
+        if (r != HIPRTC_SUCCESS) {
+            if (g_log.empty()) g_log = hiprtcGetErrorString(r);
+            hiprtcDestroyProgram(&prog);
+            delete k;
+            return FKLHIP_EUNKNOWN_SIGNATURE;
+        }
+        size_t code_size = 0;
+        hiprtcGetCodeSize(prog, &code_size);
+        k->code.resize(code_size);
+        hiprtcGetCode(prog, k->code.data());
+        hiprtcDestroyProgram(&prog);
+    }
+    // The metadata constant is read back from the module itself (on the current device).
+    hipModule_t mod = nullptr;
+    hipError_t e = hipModuleLoadData(&mod, k->code.data());
+    hipDeviceptr_t meta_ptr = nullptr;
+    size_t meta_bytes = 0;
+    if (e == hipSuccess) e = hipModuleGetGlobal(&meta_ptr, &meta_bytes, mod, "fkd_jit_meta");
+    if (e == hipSuccess && meta_bytes != sizeof(JitMeta)) e = hipErrorInvalidValue;
+    if (e == hipSuccess) e = hipMemcpyDtoH(&k->meta, meta_ptr, sizeof(JitMeta));
+    hipFunction_t fn = nullptr;
+    if (e == hipSuccess) e = hipModuleGetFunction(&fn, mod, "fkd_jit_kernel");
+    if (e != hipSuccess) {
+        if (mod) hipModuleUnload(mod);
+        delete k;
+        if (from_cache) {
+            // an unreadable or foreign file: compile afresh (which replaces it)
+            return build_and_register(signature, false);
+        }
+        g_log = std::string("loading the compiled chain failed: ") + hipGetErrorString(e);
+        return int(e);
+    }
+    if (from_cache) g_log = "loaded from " + cached;
+    else if (!cached.empty()) write_file(cached, k->code);
+    int dev = 0;
+    hipGetDevice(&dev);
+    k->per_device.emplace(dev, fn);
+    register_chain(k->signature.c_str(), k->meta.params_bytes, &jit_launch, k);
+    return FKLHIP_OK;
+}
+
 int jit_compile_and_register(const char* signature) {
     g_log.clear();
     if (!jit_enabled()) { g_log = "run-time compilation is switched off (FKLHIP_JIT=0)"; return FKLHIP_EUNKNOWN_SIGNATURE; }
@@ -150,58 +270,7 @@ int jit_compile_and_register(const char* signature) {
             }
         }
     }
-    std::string src = "#define FKD_DEVICE_CODE 1\n#define FKD_NO_NAMES 1\n#include \"fkd_kernels.hpp\"\nusing namespace fkd;\nusing JitChain = ";
-    src += signature;
-    src += ";\n"
-           "extern \"C\" __device__ const JitMeta fkd_jit_meta = jit_meta<JitChain>();\n"
-           "extern \"C\" __global__ __launch_bounds__(256) void fkd_jit_kernel(const JitChain::Params p, const TileGeom g) {\n"
-           "    jit_body<JitChain>(p, g);\n"
-           "}\n";
-    hiprtcProgram prog = nullptr;
-    hiprtcResult r = hiprtcCreateProgram(&prog, src.c_str(), "fkd_jit_chain.hip", kJitHeaderCount, kJitHeaderTexts, kJitHeaderNames);
-    if (r != HIPRTC_SUCCESS) { g_log = hiprtcGetErrorString(r); return FKLHIP_EUNKNOWN_SIGNATURE; }
-    const std::string arch = "--offload-arch=" + device_arch();
-    std::vector<const char*> opts;
-    opts.push_back(arch.c_str());
-    for (int i = 0; i < kJitFlagCount; ++i) opts.push_back(kJitFlags[i]);
-    r = hiprtcCompileProgram(prog, int(opts.size()), opts.data());
-    size_t log_size = 0;
-    if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {
-        g_log.resize(log_size);
-        hiprtcGetProgramLog(prog, &g_log[0]);
-    }
-    if (r != HIPRTC_SUCCESS) {
-        if (g_log.empty()) g_log = hiprtcGetErrorString(r);
-        hiprtcDestroyProgram(&prog);
-        return FKLHIP_EUNKNOWN_SIGNATURE;
-    }
-    JitKernel* k = new JitKernel();   // lives as long as the registry entry: for the life of the process
-    k->signature = signature;
-    size_t code_size = 0;
-    hiprtcGetCodeSize(prog, &code_size);
-    k->code.resize(code_size);
-    hiprtcGetCode(prog, k->code.data());
-    hiprtcDestroyProgram(&prog);
-    // The metadata constant is read back from the module itself (on the current device).
-    hipModule_t mod = nullptr;
-    hipError_t e = hipModuleLoadData(&mod, k->code.data());
-    hipDeviceptr_t meta_ptr = nullptr;
-    size_t meta_bytes = 0;
-    if (e == hipSuccess) e = hipModuleGetGlobal(&meta_ptr, &meta_bytes, mod, "fkd_jit_meta");
-    if (e == hipSuccess && meta_bytes != sizeof(JitMeta)) e = hipErrorInvalidValue;
-    if (e == hipSuccess) e = hipMemcpyDtoH(&k->meta, meta_ptr, sizeof(JitMeta));
-    hipFunction_t fn = nullptr;
-    if (e == hipSuccess) e = hipModuleGetFunction(&fn, mod, "fkd_jit_kernel");
-    if (e != hipSuccess) {
-        g_log = std::string("loading the compiled chain failed: ") + hipGetErrorString(e);
-        delete k;
-        return int(e);
-    }
-    int dev = 0;
-    hipGetDevice(&dev);
-    k->per_device.emplace(dev, fn);
-    register_chain(k->signature.c_str(), k->meta.params_bytes, &jit_launch, k);
-    return FKLHIP_OK;
+    return build_and_register(signature, true);
 }
 
 } // namespace fklhip

@@ -95,7 +95,9 @@ int fklhip_launch(const char *signature, const void *blob, size_t blob_bytes, vo
  * the environment variable FKLHIP_JIT=0).  This is the library's stand-in for nvcc compiling the user's translation
  * unit, FK/core/execution_model/executors.h:316-351 being instantiated for whatever chain the user wrote.  When the
  * lookup fails, fklhip_jit_log returns the device compiler's messages for the last attempt on this thread (valid
- * until the next lookup on the thread). */
+ * until the next lookup on the thread).  With the environment variable FKLHIP_JIT_CACHE naming an existing directory,
+ * compiled code objects are kept there (file name = hash of signature, architecture, flags and header text) and
+ * reused by later processes; after such a reuse the log reads "loaded from <file>". */
 int fklhip_jit_log(const char **log);
 
 /* Introspection for tests and benchmarks: what the last fklhip_launch* on this thread launched.

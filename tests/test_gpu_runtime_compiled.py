@@ -60,3 +60,47 @@ def test_float4_resize_compiled_on_first_use(device):
     want = np.zeros((dst[1], dst[0], 4), np.float32)
     ol.execute([ol.read_2d(img, 4, resize=dst, ar=ol.IGNORE_AR)], [], [ol.write(ol.WRITE_2D, want, 4, dst[0], dst[1])])
     assert out.cpu().numpy().tobytes() == want.tobytes()
+
+
+_CACHE_SCRIPT = r"""
+import ctypes, os, sys, time
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, os.path.join(sys.argv[1], "tests"))
+import numpy as np, torch
+from fusedkernellibrary_amd import cases, lib
+dev = torch.device("cuda:0")
+x = np.random.RandomState(5).rand(33, 70).astype(np.float32)
+src = torch.from_numpy(x).to(dev); out = torch.zeros_like(src)
+t0 = time.time(); cases.uncompiled_pointwise_f32(src, out); torch.cuda.synchronize(); dt = time.time() - t0
+log = ctypes.c_char_p(); lib().fklhip_jit_log(ctypes.byref(log))
+np.save(sys.argv[2], out.cpu().numpy())
+print("LOG:" + (log.value or b"").decode()); print("SECONDS:%.3f" % dt)
+"""
+
+
+def test_code_objects_are_reused_from_the_cache_directory(device, tmp_path):
+    """FKLHIP_JIT_CACHE: the first process compiles and leaves a file, the second loads it; both give the same result."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cache = tmp_path / "cache"
+    cache.mkdir()
+    env = dict(os.environ, FKLHIP_JIT_CACHE=str(cache))
+    outs = []
+    for run in range(2):
+        res = tmp_path / f"out{run}.npy"
+        r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(res)], env=env, capture_output=True, text=True, timeout=240)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs.append((np.load(res), r.stdout))
+        files = [f for f in os.listdir(cache) if f.endswith(".co")]
+        assert len(files) == 1 and not any(f.endswith(".tmp") for f in os.listdir(cache)), os.listdir(cache)
+    assert "loaded from" not in outs[0][1] and "loaded from" in outs[1][1], (outs[0][1], outs[1][1])
+    assert outs[0][0].tobytes() == outs[1][0].tobytes()
+    # a damaged file is replaced, not trusted
+    path = os.path.join(cache, files[0])
+    with open(path, "wb") as f:
+        f.write(b"not a code object")
+    res = tmp_path / "out2.npy"
+    r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(res)], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert np.load(res).tobytes() == outs[0][0].tobytes() and os.path.getsize(path) > 1000
