@@ -165,6 +165,29 @@ def main():
                lambda: cases.crop_resize_default_norm_split(src3, rects8, (224, 224), 5, (0.0, 0.0, 0.0), c3["sub"], c3["div"], o8),
                args.steps, args.warmup)
 
+        # the read-back operations, pixel formats and launch patterns either side of the path (1080p unless noted)
+        W, H = 1920, 1080
+        fo = torch.zeros((H, W, 3), dtype=torch.float32, device=dev)
+        record("deinterlace_blend_1080p_u8x3", W * H, W * H * (3 + 12), lambda: cases.deinterlace(img, 1, fo), args.steps, args.warmup)
+        po = torch.zeros((H + 32, W + 32, 3), dtype=torch.uint8, device=dev)
+        record("pad_reflect101_16px_1080p_u8x3", (W + 32) * (H + 32), W * H * 3 + (W + 32) * (H + 32) * 3,
+               lambda: cases.pad(img, 4, 16, 16, po), args.steps, args.warmup)
+        uyvy = torch.from_numpy(rng.randint(0, 256, (H, 2 * W)).astype(np.uint8)).to(dev)
+        record("uyvy_to_rgb_full709_1080p", W * H, W * H * (2 + 12), lambda: cases.yuv_to_rgb(10, 1, 1, uyvy, W, H, fo), args.steps, args.warmup)
+        nv12 = torch.zeros((H + H // 2, W), dtype=torch.uint8, device=dev)
+        record("rgb_to_nv12_limited709_1080p", W * H, W * H * 3 + W * H * 3 // 2, lambda: cases.rgb_to_yuv(0, 0, 1, img, nv12), args.steps, args.warmup)
+        t4 = torch.from_numpy(rng.rand(4, H, W, 3).astype(np.float32)).to(dev)
+        small = torch.from_numpy(rng.randint(0, 256, (540, 960, 3)).astype(np.uint8)).to(dev)
+        d4 = torch.zeros((4, H, W, 3), dtype=torch.float32, device=dev)
+        record("divergent_2_pointwise_2_resize_planes_1080p", 4 * W * H, 2 * W * H * 24 + 2 * (960 * 540 * 3 + W * H * 12),
+               lambda: cases.divergent_mixed(t4, 1.5, small, d4), args.steps, args.warmup)
+        frames = [torch.from_numpy(rng.randint(0, 256, (720, 1280, 3)).astype(np.uint8)).to(dev) for _ in range(3)]
+        px = 1280 * 720
+        record("circular_tensor_update_b8_720p", 8 * px, px * 3 + 2 * px * 12 + 7 * 2 * px * 12, lambda: cases.circular_update_b8(frames),
+               max(10, args.steps // 4), max(2, args.warmup // 4))
+        cases.circular_update_b8(frames, release=True)
+        del fo, po, uyvy, nv12, t4, d4, frames
+
     # ---- CPU baseline: the same chain on this machine's host cores, one thread, bounded sample --------------------
     cpu = None
     if not args.no_cpu:

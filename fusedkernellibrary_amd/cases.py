@@ -29,6 +29,8 @@ def cases() -> C.CDLL:
 
 
 def _ok(rc: int) -> None:
+    if rc == 2:
+        raise RuntimeError("the case driver has no chain for this combination of arguments (see tests/cases/*_chains.h)")
     if rc != 0:
         raise RuntimeError(cases().fklcase_last_error().decode())
 
@@ -264,3 +266,10 @@ def circular(batch, oldest_first, images, fill):
     _ok(cases().fklcase_circular(_stream(), int(batch), int(bool(oldest_first)), ptrs, len(images), w, h, _pitch(images[0]), C.c_float(float(fill)),
                                  states.ctypes.data_as(C.c_void_p)))
     return states
+
+
+def circular_update_b8(images, release=False):
+    """One CircularTensor<float,3,8,NewestFirst>::update per repetition (set_reps), cycling through `images` ((H,W,3) u8 cuda)."""
+    h, w = images[0].shape[:2]
+    ptrs = (C.c_void_p * len(images))(*[i.data_ptr() for i in images])
+    _ok(cases().fklcase_circular_update_b8(_stream(), ptrs, len(images), w, h, _pitch(images[0]), int(bool(release))))

@@ -461,8 +461,14 @@ __device__ __forceinline__ void divergent_run(u32 sel, const P& p, const Tup<typ
 template <class D> struct DivergentBody;
 template <class... Chains> struct DivergentBody<Divergent<Chains...>> {
     __device__ __forceinline__ static void run(const typename Divergent<Chains...>::Params& p) {
-        const u32 z = blockIdx.z;
-        const u32 sel = __builtin_amdgcn_readfirstlane(u32(p.select[z < u32(Divergent<Chains...>::kMaxPlanes) ? z : 0u]));
+        using D = Divergent<Chains...>;
+        const u32 z = blockIdx.z < u32(D::kMaxPlanes) ? blockIdx.z : 0u;
+        // The table entry is fetched from the kernel-argument segment itself (the parameter block is the kernel's first
+        // argument): indexing the by-value copy with a run-time index would make the compiler keep that copy in
+        // scratch memory, for every lane.
+        const FKD_CONSTANT u32* words = (const FKD_CONSTANT u32*)__builtin_amdgcn_kernarg_segment_ptr();
+        const u32 at = u32(__builtin_offsetof(typename D::Params, select)) + z;
+        const u32 sel = __builtin_amdgcn_readfirstlane((words[at / 4u] >> ((at & 3u) * 8u)) & 0xffu);
         divergent_run<0, Chains...>(sel, p, p.seq);
     }
 };

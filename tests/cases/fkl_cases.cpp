@@ -430,9 +430,10 @@ int fklcase_crop_swap_u8_b4(void* stream, const uint8_t* src, int w, int h, int 
 // ---- pixel formats and colour conversions (color_chains.h on the GPU) --------------------------------------------
 namespace {
 using GpuColor = color_chains::Chains<TransformDPP<>, Stream>;
+// body() runs once per repetition asked for with fklcase_set_reps (benchmarks time the whole run)
 template <typename F> int guarded_rc(F body) {
     int rc = 0;
-    const int g = guarded([&] { rc = body(); });
+    const int g = guarded([&] { for (int rep = 0; rep < g_reps && rc == 0; ++rep) rc = body(); });
     return g ? g : rc;
 }
 } // namespace
@@ -475,17 +476,37 @@ extern "C" int fklcase_pad(void* stream_, int elem, int border_type, const void*
 // ---- divergent launches and the CircularTensor window (circular_chains.h on the GPU) -------------------------------
 extern "C" {
 int fklcase_divergent_two(void* stream_, const uint32_t* a, const uint32_t* b, int w, int h, int pitch, uint32_t add, uint32_t* out) {
-    return guarded([&] { Stream s(stream_); circular_chains::Chains<ParArch::GPU_AMD>::divergent_two(s, MemType::Device, a, b, w, h, pitch, add, out); });
+    return guarded_rc([&] { Stream s(stream_); circular_chains::Chains<ParArch::GPU_AMD>::divergent_two(s, MemType::Device, a, b, w, h, pitch, add, out); return 0; });
 }
 int fklcase_divergent_mixed(void* stream_, const float* tensor4, int w, int h, float mul, const uint8_t* img, int iw, int ih, int ipitch, float* out) {
-    return guarded([&] { Stream s(stream_); circular_chains::Chains<ParArch::GPU_AMD>::divergent_mixed(s, MemType::Device, tensor4, w, h, mul, img, iw, ih, ipitch, out); });
+    return guarded_rc([&] { Stream s(stream_); circular_chains::Chains<ParArch::GPU_AMD>::divergent_mixed(s, MemType::Device, tensor4, w, h, mul, img, iw, ih, ipitch, out); return 0; });
 }
 // images: `iters` device pointers to uchar3 images; states: host memory, iters x batch x 3 x h x w floats
 int fklcase_circular(void* stream_, int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch, float fill,
                      float* states) {
-    return guarded_rc([&] {
+    int rc = 0;
+    const int g = guarded([&] {
         Stream s(stream_);
-        return circular_chains::Chains<ParArch::GPU_AMD>::circular(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Device, fill, states);
+        rc = circular_chains::Chains<ParArch::GPU_AMD>::circular(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Device, fill, states);
+    });
+    return g ? g : rc;
+}
+// Benchmark form of the window: an 8-plane float window (NewestFirst, planar), one update per repetition asked for with
+// fklcase_set_reps, cycling through the given uchar3 images; nothing is downloaded.  The window lives until `release`.
+int fklcase_circular_update_b8(void* stream_, const uint8_t* const* images, int n_images, int w, int h, int pitch, int release) {
+    using Window = CircularTensor<float, 3, 8, CircularTensorOrder::NewestFirst, ColorPlanes::Standard>;
+    static Window* window = nullptr;
+    static int next = 0;
+    return guarded([&] {
+        if (release) { delete window; window = nullptr; next = 0; return; }
+        Stream s(stream_);
+        if (!window) { const uint uw = uint(w), uh = uint(h); window = new Window(uw, uh); setTo(0.f, *window, s); }
+        for (int rep = 0; rep < g_reps; ++rep) {
+            const auto in = dev2d<uchar3>(images[next % n_images], w, h, pitch);
+            window->update(s, Read<PerThreadRead<ND::_2D, uchar3>>{in.ptr()}, Unary<SaturateCast<uchar3, float3>>{},
+                           Write<TensorSplit<float3>>{window->ptr()});
+            ++next;
+        }
     });
 }
 } // extern "C"
