@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--list-compiled", action="store_true",
+                    help="print to stderr the kernel symbol and signature of every chain compiled at run time")
     ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
@@ -84,6 +86,7 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     fkl.lib()   # raises if the HIP library is missing: there is no fallback
+    built_in = {s for s, _ in fkl.signatures()}
     dev = torch.device("cuda:0")
     timer = Timer(torch, fkl, cases)
     only = set(filter(None, args.only.split(","))) or {"c1", "c2", "c3", "c4", "c5", "ext"}
@@ -187,6 +190,14 @@ def main():
                max(10, args.steps // 4), max(2, args.warmup // 4))
         cases.circular_update_b8(frames, release=True)
         del fo, po, uyvy, nv12, t4, d4, frames
+
+    if args.list_compiled:
+        # kernel symbol of every chain compiled at run time ("fkd_jit_" + FNV-1a of the signature), for reading profiles
+        for sig in (s for s, _ in fkl.signatures() if s not in built_in):
+            h = 14695981039346656037
+            for b in sig.encode() + b"\0":
+                h = ((h ^ b) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+            print(f"fkd_jit_{h:016x}  {sig}", file=sys.stderr)
 
     # ---- CPU baseline: the same chain on this machine's host cores, one thread, bounded sample --------------------
     cpu = None

@@ -74,6 +74,38 @@ template <class Chain> constexpr bool is_gather_chain() {
 constexpr int kRowsBX = 64;   // lanes along x: one wave per row segment
 constexpr int kRowsBY = 4;    // waves per workgroup
 
+// The full-width part of the rows kernel: every lane has V elements in each of its ROWS rows.  MODE as in
+// detail::load_run.
+template <class Chain, int V, int ROWS, int MODE>
+__device__ __forceinline__ void rows_full(const typename Chain::Params& p, u32 kernarg_offset, int x0, int ybase, int z, int ah) {
+    using R = typename Chain::Read;
+    using W = typename Chain::Write;
+
+    // All loads first, unconditionally (rows past the end re-read the last row, which is in bounds), so every
+    // lane has ROWS independent wide loads in flight before the first use; only the stores are predicated.
+    Slot<typename R::Out> in[ROWS * V];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int y = ybase + r < ah ? ybase + r : ah - 1;
+        Slot<typename R::Out> row[V];
+        R::template exec_row<V, MODE>(x0, y, z, p.read, row);
+#pragma unroll
+        for (int i = 0; i < V; ++i) in[r * V + i].v = row[i].v;
+    }
+    // all ROWS*V elements go through the chain together, operation by operation
+    Slot<typename Chain::Value> out[ROWS * V];
+    if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<ROWS * V>(in, out, (const FKD_CONSTANT char*)__builtin_amdgcn_kernarg_segment_ptr() + kernarg_offset);
+    else Chain::template compute_run<ROWS * V>(in, out, p.ops);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int y = ybase + r;
+        Slot<typename Chain::Value> row[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) row[i].v = out[r * V + i].v;
+        if (y < ah) W::template exec_row<V, MODE>(x0, y, z, row, p.write);
+    }
+}
+
 // `kernarg_offset`: where p sits inside the kernel-argument segment (0 when the chain's parameter block is the
 // kernel's first argument); long chains fetch their operations' parameters from there.
 template <class Chain, int V, int ROWS, bool ALIGNED>
@@ -85,30 +117,16 @@ __device__ __forceinline__ void rows_body(const typename Chain::Params& p, u32 k
     const int ybase = (blockIdx.y * kRowsBY + threadIdx.y) * ROWS;
     const int aw = int(p.active_w), ah = int(p.active_h);
     if (x0 >= aw || ybase >= ah) return;
+    // Wave-cooperative accesses (mode 2 of load_run / store_run) need every lane of the wave on a full run.
+    constexpr bool kExchange = ALIGNED && (detail::wave_exchange_ok<typename R::Out>(V) || detail::wave_exchange_ok<typename W::In>(V));
+    if constexpr (kExchange) {
+        if (int(blockIdx.x * kRowsBX + kRowsBX) * V <= aw) {
+            rows_full<Chain, V, ROWS, 2>(p, kernarg_offset, x0, ybase, z, ah);
+            return;
+        }
+    }
     if (x0 + V <= aw) {
-        // All loads first, unconditionally (rows past the end re-read the last row, which is in bounds), so every
-        // lane has ROWS independent wide loads in flight before the first use; only the stores are predicated.
-        Slot<typename R::Out> in[ROWS * V];
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            const int y = ybase + r < ah ? ybase + r : ah - 1;
-            Slot<typename R::Out> row[V];
-            R::template exec_row<V, ALIGNED>(x0, y, z, p.read, row);
-#pragma unroll
-            for (int i = 0; i < V; ++i) in[r * V + i].v = row[i].v;
-        }
-        // all ROWS*V elements go through the chain together, operation by operation
-        Slot<typename Chain::Value> out[ROWS * V];
-        if constexpr (Chain::kLongChain) Chain::template compute_run_kernarg<ROWS * V>(in, out, (const FKD_CONSTANT char*)__builtin_amdgcn_kernarg_segment_ptr() + kernarg_offset);
-        else Chain::template compute_run<ROWS * V>(in, out, p.ops);
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            const int y = ybase + r;
-            Slot<typename Chain::Value> row[V];
-#pragma unroll
-            for (int i = 0; i < V; ++i) row[i].v = out[r * V + i].v;
-            if (y < ah) W::template exec_row<V, ALIGNED>(x0, y, z, row, p.write);
-        }
+        rows_full<Chain, V, ROWS, ALIGNED ? 1 : 0>(p, kernarg_offset, x0, ybase, z, ah);
     } else {
         for (int r = 0; r < ROWS; ++r) {
             const int y = ybase + r;

@@ -102,6 +102,13 @@ std::string cache_path(const char* signature, const std::string& arch) {
     snprintf(name, sizeof(name), "/fklhip-%016llx%016llx.co", a, b);
     return std::string(dir) + name;
 }
+// Every compiled chain gets a kernel symbol of its own, so that profilers tell the chains apart: "fkd_jit_" and the
+// FNV-1a hash of the signature text (terminating zero included) as 16 hex digits.
+std::string kernel_symbol(const std::string& signature) {
+    char name[32];
+    snprintf(name, sizeof(name), "fkd_jit_%016llx", fnv1a(14695981039346656037ull, signature));
+    return name;
+}
 bool read_file(const std::string& path, std::vector<char>* out) {
     FILE* f = fopen(path.c_str(), "rb");
     if (!f) return false;
@@ -136,7 +143,7 @@ int get_function(JitKernel* k, hipFunction_t* fn) {
     hipModule_t mod = nullptr;
     if ((e = hipModuleLoadData(&mod, k->code.data())) != hipSuccess) return int(e);
     hipFunction_t f = nullptr;
-    if ((e = hipModuleGetFunction(&f, mod, "fkd_jit_kernel")) != hipSuccess) return int(e);
+    if ((e = hipModuleGetFunction(&f, mod, kernel_symbol(k->signature).c_str())) != hipSuccess) return int(e);
     k->per_device.emplace(dev, f);   // the module stays loaded for the life of the process
     *fn = f;
     return FKLHIP_OK;
@@ -199,7 +206,9 @@ static int build_and_register(const char* signature, bool may_read_cache) {
         src += signature;
         src += ";\n"
                "extern \"C\" __device__ const JitMeta fkd_jit_meta = jit_meta<JitChain>();\n"
-               "extern \"C\" __global__ __launch_bounds__(256) void fkd_jit_kernel(const JitChain::Params p, const TileGeom g) {\n"
+               "extern \"C\" __global__ __launch_bounds__(256) void ";
+        src += kernel_symbol(k->signature);
+        src += "(const JitChain::Params p, const TileGeom g) {\n"
                "    jit_body<JitChain>(p, g);\n"
                "}\n";
         hiprtcProgram prog = nullptr;
@@ -236,7 +245,7 @@ static int build_and_register(const char* signature, bool may_read_cache) {
     if (e == hipSuccess && meta_bytes != sizeof(JitMeta)) e = hipErrorInvalidValue;
     if (e == hipSuccess) e = hipMemcpyDtoH(&k->meta, meta_ptr, sizeof(JitMeta));
     hipFunction_t fn = nullptr;
-    if (e == hipSuccess) e = hipModuleGetFunction(&fn, mod, "fkd_jit_kernel");
+    if (e == hipSuccess) e = hipModuleGetFunction(&fn, mod, kernel_symbol(k->signature).c_str());
     if (e != hipSuccess) {
         if (mod) hipModuleUnload(mod);
         delete k;

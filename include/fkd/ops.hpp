@@ -181,8 +181,74 @@ template <class T> constexpr bool wide_ok(int v) {
     const int bytes = int(sizeof(T)) * v;
     return v > 1 && bytes % 4 == 0 && (bytes <= 16 || bytes % 16 == 0) && sizeof(T) == sizeof(base_t<T>) * cn_v<T>;
 }
-template <class T, int V, bool ALIGNED> FKD_DEV void load_run(const T* p, Slot<T> (&out)[V]) {
-    if constexpr (ALIGNED && wide_ok<T>(V)) {
+// Runs of 32, 48 or 64 bytes per lane (four float2/float3/float4) as wide accesses would leave gaps between the lanes
+// of one instruction: lane i moves 16 bytes at i * 48, and the memory pipeline sees three sparse passes over the
+// same 3 KiB.  When the whole wave is active on consecutive runs (mode 2) the wave instead moves its segment as
+// dense instructions, lane i taking 16 bytes at k * 1024 + i * 16, and exchanges the dwords through a wave-private
+// piece of LDS.  The exchange is between lanes of one wave, whose LDS accesses complete in order, so a compiler
+// fence is all the synchronisation it needs.
+constexpr int kRowsWaves = 4;            // waves per workgroup of the rows kernels
+constexpr int kStageDwords = 64 * 16 + 64;
+template <class T> constexpr bool wave_exchange_ok(int v) {
+    const int bytes = int(sizeof(T)) * v;
+    return wide_ok<T>(v) && sizeof(base_t<T>) <= 4 && (bytes == 32 || bytes == 48 || bytes == 64);
+}
+FKD_DEV u32* wave_stage() {
+    __shared__ __attribute__((aligned(16))) u32 stage[kRowsWaves * kStageDwords];
+    return stage + threadIdx.y * kStageDwords;
+}
+// Where dword f of the wave's segment sits in the stage: runs of 32 and 64 bytes get 16 bytes of padding per 256 so
+// that the 16 lanes of one LDS pass fall on distinct banks; runs of 48 bytes already do.
+template <int W> FKD_DEV u32 stage_at(u32 f) { return W == 12 ? f : f + (f >> 6) * 4u; }
+FKD_DEV void wave_exchange_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
+template <int W> FKD_DEV void load_words_wave(const void* p, u32 (&w)[W]) {
+    const u32 lane = threadIdx.x;
+    u32* stage = wave_stage();
+    // p is this lane's run; the segment starts W dwords per lane earlier
+    const char* seg = reinterpret_cast<const char*>(p) - size_t(lane) * (W * 4);
+    u32x4_t q[W / 4];
+#pragma unroll
+    for (int k = 0; k < W / 4; ++k) q[k] = *gconst<u32x4_a4>(seg + k * 1024 + lane * 16);
+    wave_exchange_fence();   // the previous exchange's reads come first
+#pragma unroll
+    for (int k = 0; k < W / 4; ++k) *reinterpret_cast<u32x4_t*>(stage + stage_at<W>(u32(k) * 256u + lane * 4u)) = q[k];
+    wave_exchange_fence();
+#pragma unroll
+    for (int j = 0; j < W / 4; ++j) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage + stage_at<W>(lane * W + u32(j) * 4u));
+        w[4 * j] = v.x; w[4 * j + 1] = v.y; w[4 * j + 2] = v.z; w[4 * j + 3] = v.w;
+    }
+}
+template <int W> FKD_DEV void store_words_wave(void* p, const u32 (&w)[W]) {
+    const u32 lane = threadIdx.x;
+    u32* stage = wave_stage();
+    char* seg = reinterpret_cast<char*>(p) - size_t(lane) * (W * 4);
+    wave_exchange_fence();
+#pragma unroll
+    for (int j = 0; j < W / 4; ++j) {
+        u32x4_t v; v.x = w[4 * j]; v.y = w[4 * j + 1]; v.z = w[4 * j + 2]; v.w = w[4 * j + 3];
+        *reinterpret_cast<u32x4_t*>(stage + stage_at<W>(lane * W + u32(j) * 4u)) = v;
+    }
+    wave_exchange_fence();
+#pragma unroll
+    for (int k = 0; k < W / 4; ++k)
+        *gmut<u32x4_a4>(seg + k * 1024 + lane * 16) = *reinterpret_cast<const u32x4_t*>(stage + stage_at<W>(u32(k) * 256u + lane * 4u));
+}
+
+// MODE 0: nothing is known about p.  MODE 1: p is dword aligned.  MODE 2: as 1, and all 64 lanes of the wave are in
+// this call with consecutive runs (lane i at p0 + i * V elements).
+template <class T, int V, int MODE> FKD_DEV void load_run(const T* p, Slot<T> (&out)[V]) {
+    constexpr bool ALIGNED = MODE != 0;
+    if constexpr (MODE == 2 && wave_exchange_ok<T>(V)) {
+        constexpr int W = int(sizeof(T)) * V / 4;
+        u32 w[W];
+        load_words_wave<W>(p, w);
+        unpack_words<T, V, W>(w, out);
+    } else if constexpr (ALIGNED && wide_ok<T>(V)) {
         constexpr int W = int(sizeof(T)) * V / 4;
         u32 w[W];
         load_words<W>(p, w);
@@ -198,8 +264,14 @@ template <class T, int V, bool ALIGNED> FKD_DEV void load_run(const T* p, Slot<T
         for (int i = 0; i < V; ++i) out[i].v = load_elem(p + i);
     }
 }
-template <class T, int V, bool ALIGNED> FKD_DEV void store_run(T* p, const Slot<T> (&in)[V]) {
-    if constexpr (ALIGNED && wide_ok<T>(V)) {
+template <class T, int V, int MODE> FKD_DEV void store_run(T* p, const Slot<T> (&in)[V]) {
+    constexpr bool ALIGNED = MODE != 0;
+    if constexpr (MODE == 2 && wave_exchange_ok<T>(V)) {
+        constexpr int W = int(sizeof(T)) * V / 4;
+        u32 w[W];
+        pack_words<T, V, W>(in, w);
+        store_words_wave<W>(p, w);
+    } else if constexpr (ALIGNED && wide_ok<T>(V)) {
         constexpr int W = int(sizeof(T)) * V / 4;
         u32 w[W];
         pack_words<T, V, W>(in, w);
@@ -951,7 +1023,7 @@ template <class T> struct Read2D {
     FKD_DEV static T exec(int x, int y, int, const Params& p) {
         return detail::load_elem(detail::row_ptr(p.data, p.pitch, x, y));
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<T> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<T> (&out)[V]) {
         detail::load_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), out);
     }
     // True when every row start (shifted by xoff elements) is dword aligned: the launcher's licence to use
@@ -1021,7 +1093,7 @@ template <class T> struct Read3D {
     FKD_DEV static T exec(int x, int y, int z, const Params& p) {
         return detail::load_elem(detail::row_ptr(plane(p, z), p.pitch, x, y));
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
         detail::load_run<T, V, A>(detail::row_ptr(plane(p, z), p.pitch, x, y), out);
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) {
@@ -1057,7 +1129,7 @@ template <class T> struct TensorPack {
         if constexpr (cn_v<T> > 3) chan<3>(o) = g[3 * px];
         return o;
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
         const B* r = at(p, x, y, z);
         const size_t px = size_t(p.width) * p.height;
         Slot<B> c[4][V];
@@ -1102,7 +1174,7 @@ template <int DIR, int BATCH, class Back> struct CircularRead {
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return Back::exec(x, y, circular_plane<DIR, BATCH>(z, p.first), p.back); }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         Back::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), p.back, out);
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
@@ -1127,7 +1199,7 @@ template <int DIR, int BATCH, class PlaneOp> struct CircularBatchRead {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         return PlaneOp::exec(x, y, c, p.plane[c]);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         PlaneOp::template exec_row<V, A>(x, y, c, p.plane[c], out);
     }
@@ -1160,7 +1232,7 @@ template <bool VU> struct ReadNV {
         o.z = c[VU ? 0 : 1];
         return o;
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
@@ -1264,7 +1336,7 @@ template <int PF> struct ReadYUV {
         }
         return o;
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
@@ -1289,7 +1361,7 @@ template <class Back> struct Crop {
     FKD_DEV static int width(const Params& p) { return p.w; }
     FKD_DEV static int height(const Params& p) { return p.h; }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) { return Back::exec(x + p.x, y + p.y, 0, p.back); }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<Out> (&out)[V]) {
         Back::template exec_row<V, A>(x + p.x, y + p.y, 0, p.back, out);
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff + p.x); }
@@ -1372,7 +1444,7 @@ template <int BT, class Back> struct Border {
             return Back::exec(fold(x, w), fold(y, h), z, p.back);
         }
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
@@ -1397,7 +1469,7 @@ template <class Back, class... Ops> struct FusedRead {
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
         return fold<Ops...>(Back::exec(x, y, z, p.back), p.ops);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         Slot<typename Back::Out> t[V];
         Back::template exec_row<V, A>(x, y, z, p.back, t);
 #pragma unroll
@@ -1503,7 +1575,7 @@ template <int AR, class Back> struct ResizeLinear {
         const Src d = Back::exec(t.x2r, t.y2r, z, p.back);
         return blend(a, b, c, d, t);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
@@ -1547,7 +1619,7 @@ template <int DT, class Back> struct Deinterlace {
         lines(y, p, ya, yb, average);
         return mix(Back::exec(x, ya, z, p.back), Back::exec(x, yb, z, p.back), average);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         int ya, yb; bool average;
         lines(y, p, ya, yb, average);
         Slot<Src> ra[V], rb[V];
@@ -1614,7 +1686,7 @@ template <int WT, class Back> struct Warp {
         }
         return o;
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
@@ -1633,7 +1705,7 @@ template <int N, class PlaneOp> struct BatchRead {
     FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         PlaneOp::template exec_row<V, A>(x, y, z, p.plane[z], out);
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) {
@@ -1657,7 +1729,7 @@ template <int N, class PlaneOp> struct BatchReadDefault {
         if (p.used <= z) return p.def;
         return PlaneOp::exec(x, y, z, p.plane[z]);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         if (p.used <= z) {
 #pragma unroll
             for (int i = 0; i < V; ++i) out[i].v = p.def;
@@ -1685,7 +1757,7 @@ template <class T> struct ReadSet {
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static T exec(int, int, int, const Params& p) { return p.value; }
-    template <int V, bool A> FKD_DEV static void exec_row(int, int, int, const Params& p, Slot<T> (&out)[V]) {
+    template <int V, int A> FKD_DEV static void exec_row(int, int, int, const Params& p, Slot<T> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = p.value;
     }
@@ -1706,7 +1778,7 @@ template <class T> struct Write2D {
     FKD_DEV static void exec(int x, int y, int, const T& v, const Params& p) {
         detail::store_elem(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int, const Slot<T> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Slot<T> (&v)[V], const Params& p) {
         detail::store_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
     FKD_HD static bool rows_aligned(const Params& p) { return detail::dword_aligned(p.data) && p.pitch % 4 == 0; }
@@ -1739,7 +1811,7 @@ template <class T> struct TensorWrite {
     FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
         detail::store_elem(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         detail::store_run<T, V, A>(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
     }
     FKD_HD static bool rows_aligned(const Params& p) {
@@ -1780,7 +1852,7 @@ template <class T> struct TensorSplit {
         if constexpr (cn_v<T> > 2) gw[2 * px] = chan<2>(v);
         if constexpr (cn_v<T> > 3) gw[3 * px] = chan<3>(v);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         B* w = at(p, x, y, z);
         const size_t px = size_t(p.width) * p.height;
         Slot<B> c0[V], c1[V];
@@ -1891,7 +1963,7 @@ template <int PF> struct WriteYUV {
         for (int i = 0; i < V; ++i) put(r, x + i, v[i].v);
     }
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { put(row(y, z, p), x, v); }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         put_run<V>(row(y, z, p), x, v);
     }
     FKD_HD static bool rows_aligned(const Params&) { return true; }   // element-wise either way
@@ -1907,7 +1979,7 @@ template <int N, class W> struct BatchWrite {
     FKD_NAME("BatchWrite<" + istr(N) + "," + W::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, z, v, p.plane[z]); }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         W::template exec_row<V, A>(x, y, z, v, p.plane[z]);
     }
     FKD_HD static bool rows_aligned(const Params& p) {
@@ -1931,7 +2003,7 @@ template <int DIR, int BATCH, class W> struct CircularWrite {
     FKD_NAME("CircularWrite<" + istr(DIR) + "," + istr(BATCH) + "," + W::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w); }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         W::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w);
     }
     FKD_HD static bool rows_aligned(const Params& p) { return W::rows_aligned(p.w); }
@@ -1948,7 +2020,7 @@ template <int DIR, int BATCH, class W> struct CircularBatchWrite {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         W::exec(x, y, c, v, p.plane[c]);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         W::template exec_row<V, A>(x, y, c, v, p.plane[c]);
     }
@@ -1972,7 +2044,7 @@ template <class W1, class W2> struct TeeWrite {
         W1::exec(x, y, z, v, p.first);
         W2::exec(x, y, z, v, p.second);
     }
-    template <int V, bool A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         W1::template exec_row<V, A>(x, y, z, v, p.first);
         W2::template exec_row<V, A>(x, y, z, v, p.second);
     }
