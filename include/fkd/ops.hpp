@@ -1647,6 +1647,9 @@ template <int WT, class Back> struct Warp {
     };
     static constexpr bool kTapCursor = false;
     static constexpr bool kGatherRead = true;     // taps are scattered: one element per thread
+    static constexpr bool kPairTaps = [] {
+        if constexpr (requires { Back::kTapPair; }) return Back::kTapCursor && Back::kTapPair; else return false;
+    }();
     FKD_NAME("Warp<" + istr(WT) + "," + Back::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return p.dst_w; }
@@ -1662,6 +1665,39 @@ template <int WT, class Back> struct Warp {
         }
         const int sw = Back::width(p.back), sh = Back::height(p.back);
         Out o;
+        if constexpr (kPairTaps) {
+            // Taps x1 and x1 + 1 of a source line in one access each, issued by every lane (lanes whose source point
+            // lies outside take the taps of pixel (0, 0) and drop them), so that no load waits behind a branch.  A wave
+            // that touches the image's last line, where such an access could reach past the allocation, takes the
+            // element-wise path below instead, all lanes together.
+            const bool inside = sx >= 0.f && sx < f32(sw) && sy >= 0.f && sy < f32(sh);
+            const f32 cx = inside ? sx : 0.f, cy = inside ? sy : 0.f;
+            const int x1 = int(__builtin_floorf(cx)), y1 = int(__builtin_floorf(cy));
+            const int y2r = y1 + 1 < sh - 1 ? y1 + 1 : sh - 1;
+            const auto ra = Back::tap_row(0, y1, z, p.back), rb = Back::tap_row(0, y2r, z, p.back);
+            const bool risky = sw < 2 || Back::tap_last(ra) || Back::tap_last(rb);
+            if (__builtin_amdgcn_ballot_w64(risky) == 0) {
+                const bool edge = x1 >= sw - 1;           // x1 + 1 is past the line: both taps are the last pixel
+                const int xp = edge ? sw - 2 : x1;
+                const auto wa = Back::pair_load(ra, xp, p.back), wb = Back::pair_load(rb, xp, p.back);
+                const f32 ax = f32(x1 + 1) - cx, bx = cx - f32(x1), ay = f32(y1 + 1) - cy, by = cy - f32(y1);
+                const f32 w00 = ax * ay, w10 = bx * ay, w01 = ax * by, w11 = bx * by;
+                typename Back::Raw a0, a1, b0, b1;
+                Back::pair_values(wa, ra, xp, a0, a1);
+                Back::pair_values(wb, rb, xp, b0, b1);
+                const Src a = Back::finish(edge ? a1 : a0, p.back), b = Back::finish(a1, p.back);
+                const Src c = Back::finish(edge ? b1 : b0, p.back), d = Back::finish(b1, p.back);
+                auto one = [&](auto pa, auto pb, auto pc, auto pd) {
+                    const f32 v = ((f32(pa) * w00 + f32(pb) * w10) + f32(pc) * w01) + f32(pd) * w11;
+                    return inside ? v : 0.f;
+                };
+                chan<0>(o) = one(chan<0>(a), chan<0>(b), chan<0>(c), chan<0>(d));
+                if constexpr (cn_v<Src> > 1) chan<1>(o) = one(chan<1>(a), chan<1>(b), chan<1>(c), chan<1>(d));
+                if constexpr (cn_v<Src> > 2) chan<2>(o) = one(chan<2>(a), chan<2>(b), chan<2>(c), chan<2>(d));
+                if constexpr (cn_v<Src> > 3) chan<3>(o) = one(chan<3>(a), chan<3>(b), chan<3>(c), chan<3>(d));
+                return o;
+            }
+        }
         if (sx >= 0.f && sx < f32(sw) && sy >= 0.f && sy < f32(sh)) {
             const f32 f1x = __builtin_floorf(sx), f1y = __builtin_floorf(sy);
             const int x1 = int(f1x), y1 = int(f1y);
