@@ -308,7 +308,11 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     //   kPairsPrepared  kPairs for images whose rows all start at the same offset inside their dword (pitch a multiple
     //             of 4): the image is a buffer resource, a row a scalar offset, and the lane's window offset and byte
     //             shift are worked out once per column instead of once per tap;
-    constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3, kPairsPrepared = 4;
+    //   kWhole    both scale factors are whole numbers (4K -> 1080p): every source point is a pixel, the weights are
+    //             1, 0, 0, 0, and the blend is the first tap; the others are not fetched.  Only for reads whose taps are
+    //             always finite (a zero weight times them is a zero), and a lane whose first tap is a negative zero,
+    //             where the zeros of the other three terms decide the sign of the sum, takes all four after all.
+    constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3, kPairsPrepared = 4, kWhole = 5;
     const int yend = y0 + YI < ah ? y0 + YI : ah;
     auto rows = [&](auto mode_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
@@ -351,6 +355,8 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
                     const int xl = MODE == kPairsSel ? x1[i] - int(clamped[i]) : x1[i];
                     t.ab[i] = Back::pair_load(t.ra, xl, q.back);
                     t.cd[i] = Back::pair_load(t.rb, xl, q.back);
+                } else if constexpr (MODE == kWhole) {
+                    t.a[i] = Back::template tap_load<false>(t.ra, x1[i], q.back);
                 } else {
                     t.a[i] = Back::template tap_load<MODE == kSingles>(t.ra, x1[i], q.back);
                     t.b[i] = Back::template tap_load<MODE == kSingles>(t.ra, x2[i], q.back);
@@ -370,6 +376,31 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
                 typename RZ::Taps tp;
                 tp.w00 = ax[i] * t.ay; tp.w10 = bx[i] * t.ay; tp.w01 = ax[i] * t.by; tp.w11 = bx[i] * t.by;
                 Raw a, b, c, d;
+                if constexpr (MODE == kWhole) {
+                    using Src = typename RZ::Src;
+                    const Src first = Back::finish(Back::tap_value(t.a[i]), q.back);
+                    typename RZ::Out v;
+                    bool negative_zero = false;
+                    auto take = [&](auto pa) {
+                        const f32 f = f32(pa);
+                        if constexpr (__is_same(base_t<Src>, f32) || __is_same(base_t<Src>, f64))
+                            negative_zero = negative_zero || __builtin_bit_cast(u32, f) == 0x80000000u;
+                        return f;
+                    };
+                    chan<0>(v) = take(chan<0>(first));
+                    if constexpr (cn_v<Src> > 1) chan<1>(v) = take(chan<1>(first));
+                    if constexpr (cn_v<Src> > 2) chan<2>(v) = take(chan<2>(first));
+                    if constexpr (cn_v<Src> > 3) chan<3>(v) = take(chan<3>(first));
+                    if (negative_zero) {
+                        b = Back::tap_value(Back::template tap_load<false>(t.ra, x2[i], q.back));
+                        c = Back::tap_value(Back::template tap_load<false>(t.rb, x1[i], q.back));
+                        d = Back::tap_value(Back::template tap_load<false>(t.rb, x2[i], q.back));
+                        v = RZ::blend(first, Back::finish(b, q.back), Back::finish(c, q.back), Back::finish(d, q.back), tp);
+                    }
+                    if constexpr (RZ::kAR != IGNORE_AR) { if (!(yin && xin[i])) v = q.bg; }
+                    res[i].v = Chain::compute_checked_ops(v, ops);
+                    continue;
+                }
                 if constexpr (PAIRED) {
                     const int xl = MODE == kPairsSel ? x1[i] - int(clamped[i]) : x1[i];
                     Back::pair_values(t.ab[i], t.ra, xl, a, b);
@@ -430,6 +461,12 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
         const int yl = int(__builtin_floorf(f32(ylast - oy) * q.fy));
         const int yb = yl + 1 < sh - 1 ? yl + 1 : sh - 1;
         tail = Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back));
+    }
+    if constexpr (detail::finite_taps<Back>()) {
+        // whole factors, and every source coordinate an exact float
+        const bool whole = q.fx >= 1.0f && q.fy >= 1.0f && q.fx == __builtin_floorf(q.fx) && q.fy == __builtin_floorf(q.fy) &&
+                           f32(aw) * q.fx <= 16777216.0f && f32(ah) * q.fy <= 16777216.0f;
+        if (whole) { rows(IntTag<kWhole>{}); return; }
     }
     if (tail) {
         rows(IntTag<kSafe>{});

@@ -410,6 +410,15 @@ struct PairPrep { u32 off, shift; };
 template <class B> constexpr bool tap_prepared() {
     if constexpr (requires { B::kTapPrepared; }) return B::kTapPrepared; else return false;
 }
+// Reads whose taps, after everything fused into the read, are finite numbers whatever the image holds (integer
+// pixels through operations without run-time parameters): a tap with weight zero then contributes a zero and can be
+// left out of a blend.  Compute operations say so with kFiniteMap.
+template <class B> constexpr bool finite_taps() {
+    if constexpr (requires { B::kFiniteTaps; }) return B::kFiniteTaps; else return false;
+}
+template <class Op> constexpr bool finite_map() {
+    if constexpr (requires { Op::kFiniteMap; }) return Op::kFiniteMap; else return false;
+}
 struct TapImage {
 #if defined(FKD_DEVICE_CODE)
     __amdgpu_buffer_rsrc_t rsrc;
@@ -668,6 +677,7 @@ template <class I, class O> struct Cast {
 // reached through ColorConversion<COLOR_BGR2RGB,...>, FK/algorithms/image_processing/color_conversion.h:472-476.
 template <class T, int I0, int I1, int I2 = 2, int I3 = 3> struct Reorder {
     using In = T; using Out = T; using Params = Empty;
+    static constexpr bool kFiniteMap = true;
     FKD_NAME("Reorder<" + type_name<T>() + "," + istr(I0) + "," + istr(I1) + "," + istr(I2) + "," + istr(I3) + ">")
     FKD_DEV static T exec(const T& a, const Params&) {
         T o;
@@ -803,6 +813,7 @@ FKD_DEV Vec<f32, 3> color_mxv(const ColorMatrix& c, f32 a, f32 b, f32 d) {
 // depth's offsets (luma only for limited range) times the matrix; no clamp.
 template <int CD, int CR, int CP> struct YUV2RGB {
     using In = Vec<typename DepthConsts<CD>::base, 3>; using Out = Vec<f32, 3>; using Params = Empty;
+    static constexpr bool kFiniteMap = true;
     FKD_NAME("YUV2RGB<" + istr(CD) + "," + istr(CR) + "," + istr(CP) + ">")
     FKD_DEV static Out exec(const In& a, const Params&) {
         using D = DepthConsts<CD>;
@@ -1029,6 +1040,7 @@ template <class T> struct Read2D {
     using Out = T;
     using Params = RawPtr2D<const T>;
     static constexpr bool kTapCursor = true;
+    static constexpr bool kFiniteTaps = !(__is_same(base_t<T>, f32) || __is_same(base_t<T>, f64));
     FKD_NAME("Read2D<" + type_name<T>() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -1233,6 +1245,7 @@ template <bool VU> struct ReadNV {
     using Out = Vec<u8, 3>;
     using Params = RawNV12;
     static constexpr bool kTapCursor = true;
+    static constexpr bool kFiniteTaps = true;
     FKD_NAME(VU ? "ReadNV21" : "ReadNV12")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -1371,6 +1384,7 @@ template <class Back> struct Crop {
     static constexpr bool kTapCursor = Back::kTapCursor;
     FKD_NAME("Crop<" + Back::name() + ">")
 #if defined(FKD_DEVICE_CODE)
+    static constexpr bool kFiniteTaps = detail::finite_taps<Back>();
     FKD_DEV static int width(const Params& p) { return p.w; }
     FKD_DEV static int height(const Params& p) { return p.h; }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) { return Back::exec(x + p.x, y + p.y, 0, p.back); }
@@ -1477,6 +1491,7 @@ template <class Back, class... Ops> struct FusedRead {
     static constexpr bool kTapCursor = Back::kTapCursor;
     FKD_NAME("FusedRead<" + Back::name() + OpList<Ops...>::names() + ">")
 #if defined(FKD_DEVICE_CODE)
+    static constexpr bool kFiniteTaps = detail::finite_taps<Back>() && (detail::finite_map<Ops>() && ...);
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
