@@ -112,6 +112,20 @@ def div_f32(src, d, out):
                                 _p(out), out.stride(0) * 4))
 
 
+def div_mode(d) -> int:
+    """0 generic division, 1 five-instruction sequence, 2 two-instruction sequence proven exact for this divisor."""
+    l = cases()
+    l.fklcase_div_mode.argtypes = [C.c_float]
+    return int(l.fklcase_div_mode(C.c_float(d)))
+
+
+def div_f32_forced(src, d, mode, out):
+    """Read2D<float> -> Div(d) -> Write2D<float> with the division sequence given by the caller (see div_mode)."""
+    h, w = src.shape
+    _ok(cases().fklcase_div_f32_forced(_stream(), _p(src), w, h, src.stride(0) * 4, C.c_float(float(d)), int(mode), _p(out),
+                                       out.stride(0) * 4))
+
+
 def div_f32x3(src, d, out):
     """src/out (H,W,3) f32 cuda, d three divisors (one per channel)."""
     dd = _host(d, np.float32)

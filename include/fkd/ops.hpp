@@ -52,6 +52,14 @@ typedef u32x4_t u32x4_a4 __attribute__((aligned(4)));
 // the non-temporal hint: the L2s then hand the lines on early instead of keeping them dirty until the kernel ends,
 // when all of them would have to be written back at once (a 3840x2160 float copy: 10.6 -> 9.9 us).
 template <class Q> FKD_DEV void gstore(FKD_GLOBAL Q* p, const Q& v) { __builtin_nontemporal_store(v, p); }
+// One element of 4 or 8 bytes written through the L2 (a relaxed store at system scope: global_store ... sc0 sc1), for
+// writers whose lanes each store single elements: the planar writer of the bilinear kernel runs configuration 3 in
+// 11.1 us with these, 11.5 us with the non-temporal hint and 12.9 us with plain stores.  Other sizes take gstore.
+template <class B> FKD_DEV void gstore_through(FKD_GLOBAL B* p, const B& v) {
+    if constexpr (sizeof(B) == 4) __hip_atomic_store(reinterpret_cast<FKD_GLOBAL u32*>(p), __builtin_bit_cast(u32, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    else if constexpr (sizeof(B) == 8) __hip_atomic_store(reinterpret_cast<FKD_GLOBAL unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    else *p = v;
+}
 // One whole-dword load of a row run; STREAM marks data that no cache can hold until its next use (see the rows kernel).
 template <bool STREAM, class Q> FKD_DEV Q gload_run(const FKD_GLOBAL Q* p) {
     if constexpr (STREAM) return __builtin_nontemporal_load(p);
@@ -581,10 +589,24 @@ FKD_BINARY_OP(Mul, x * y)
 // That argument needs every intermediate free of underflow and overflow: the host enables the path only for
 // 2^-40 <= |y| <= 2^40, and the device takes it only for elements with 2^-60 <= |x| <= 2^60 in every channel;
 // everything else (zeros, denormals, infinities, NaNs, extreme magnitudes) goes through the generic division.
+//
+// For most divisors two instructions are enough (fast == 2): with the reciprocal held in two floats, r = RN(1/y) and
+// l = RN(1/y - r),
+//     q = fma(x, r, x*l)
+// is computed from t = x*r + RN(x*l), and |t - x/y| < 1.5 * 2^-47 |x/y|, i.e. less than 1.5 * 2^-23 ulp of the
+// quotient.  RN(t) can differ from RN(x/y) only if x/y lies that close to the midpoint of two floats.  Write
+// |x| = X 2^a, |y| = Y 2^b with 24-bit integers X, Y; the midpoints of the quotient's binade are (2Q+1) / 2^(25+s)
+// (s = 0 for X >= Y, 1 otherwise) and the distance of X/Y from one of them is |2^(24+s) X - (2Q+1) Y| / (2Y) ulp.  The
+// integer D = 2^(24+s) X - (2Q+1) Y is never 0 and must be below 6 in magnitude for a failure, so for a given y all
+// candidate numerators are the solutions X of 2^(24+s) X = D (mod Y), |D| <= 8, a few dozen at most.  The host
+// finds them with a modular inverse and runs the two instructions on each one; if every result equals the correctly
+// rounded quotient the sequence is exact for that divisor and ALL x (powers of two only shift exponents; the range
+// conditions above, with 2^-30 <= |y| <= 2^30, keep every intermediate normal or harmlessly small), otherwise the divisor
+// keeps the five-instruction form.
 template <class I, class P, class O> struct Div {
     using In = I; using Out = O;
     static constexpr bool kReciprocal = __is_same(base_t<I>, f32) && __is_same(base_t<P>, f32) && __is_same(base_t<O>, f32);
-    struct Params { P v; P rcp; i32 fast; };
+    struct Params { P v; P rcp; P rcp_lo; i32 fast; };
     FKD_NAME("Div<" + type_name<I>() + "," + type_name<P>() + "," + type_name<O>() + ">")
 
 #if !defined(FKD_DEVICE_CODE)
@@ -600,19 +622,71 @@ template <class I, class P, class O> struct Div {
         }
         return best;
     }
+    // The low part of the reciprocal: 1 - d*r is exact in double, its quotient by d is rounded once to double and once
+    // to float (the second rounding can cost one more unit in the last place of l, which the proof's margin covers).
+    static f32 reciprocal_low(f32 d, f32 r) { return f32((1.0 - double(d) * double(r)) / double(d)); }
+    // What the device computes, with the same roundings.
+    static f32 two_step(f32 x, f32 r, f32 l) {
+        volatile f32 low = x * l;
+        return __builtin_fmaf(x, r, low);
+    }
+    // True when two_step(x, r, l) == RN(x/d) for every x whose quotient neither overflows nor underflows (see above).
+    static bool two_step_proven(f32 d, f32 r, f32 l) {
+        using u64 = unsigned long long; using i64 = long long;
+        int e = 0;
+        const f32 m = __builtin_frexpf(__builtin_fabsf(d), &e);       // |d| = m 2^e, m in [0.5, 1)
+        const u64 Y = u64(__builtin_ldexpf(m, 24));                   // |d| = Y 2^(e-24), Y in [2^23, 2^24)
+        const int v = __builtin_ctzll(Y);
+        const u64 Yo = Y >> v;                                        // odd part
+        if (Yo == 1) return true;                                     // a power of two: the quotient is exact
+        auto inverse = [](u64 a, u64 mod) {                           // a^-1 mod an odd modulus, a odd or even but coprime
+            i64 t = 0, nt = 1, rr = i64(mod), nr = i64(a % mod);
+            while (nr != 0) { const i64 q = rr / nr; i64 k = t - q * nt; t = nt; nt = k; k = rr - q * nr; rr = nr; nr = k; }
+            return u64(t < 0 ? t + i64(mod) : t);
+        };
+        for (int s = 0; s < 2; ++s) {
+            const u64 N = 1ull << (24 + s);
+            const u64 inv = inverse((N >> v) % Yo, Yo);
+            for (int D = -8; D <= 8; ++D) {
+                if (D == 0 || (D % (1 << v)) != 0) continue;          // 2^v divides Y and N, so it must divide D (v <= 3 here)
+                if (v > 3) continue;
+                const i64 Dg = D / (1 << v);
+                const u64 res = u64(((Dg % i64(Yo)) + i64(Yo)) % i64(Yo));
+                const u64 X0 = res * inv % Yo;
+                for (u64 X = X0; X < (1ull << 24); X += Yo) {
+                    if (X < (1ull << 23)) continue;
+                    const f32 x = __builtin_ldexpf(f32(X), e - 24);    // x/|d| = X/Y
+                    const f32 want = f32(double(x) / double(d));       // correctly rounded: double carries 2*24+2 bits
+                    if (two_step(x, r, l) != want || two_step(-x, r, l) != -want) return false;
+                }
+            }
+        }
+        return true;
+    }
     static Params make(const P& v) {
         Params p{};
         p.v = v;
         p.fast = 0;
         if constexpr (kReciprocal) {
-            bool ok = true;
+            bool ok = true, two = true;
             auto one = [&](f32 d) {
                 const f32 a = __builtin_fabsf(d);
                 if (!(a >= 0x1p-40f && a <= 0x1p40f)) { ok = false; return 0.0f; }
                 return exact_reciprocal(d);
             };
             p.rcp = map1<P>(v, one);
-            p.fast = ok ? 1 : 0;
+            if (ok) {
+                p.rcp_lo = map2<P>(v, p.rcp, [](f32 d, f32 r) { return reciprocal_low(d, r); });
+                auto proven = [&](f32 d, f32 r, f32 l) {
+                    const f32 a = __builtin_fabsf(d);
+                    if (!(a >= 0x1p-30f && a <= 0x1p30f) || !two_step_proven(d, r, l)) two = false;
+                };
+                proven(chan_or_scalar<0>(v), chan_or_scalar<0>(p.rcp), chan_or_scalar<0>(p.rcp_lo));
+                if constexpr (cn_v<P> > 1) proven(chan<1>(v), chan<1>(p.rcp), chan<1>(p.rcp_lo));
+                if constexpr (cn_v<P> > 2) proven(chan<2>(v), chan<2>(p.rcp), chan<2>(p.rcp_lo));
+                if constexpr (cn_v<P> > 3) proven(chan<3>(v), chan<3>(p.rcp), chan<3>(p.rcp_lo));
+            }
+            p.fast = ok ? (two ? 2 : 1) : 0;
         }
         return p;
     }
@@ -629,7 +703,8 @@ template <class I, class P, class O> struct Div {
         const f32 e1 = __builtin_fmaf(-y, q1, x);
         return __builtin_fmaf(e1, r, q1);
     }
-    // Straight-line variant: always returns the five-instruction result and clears `ok` when that result may not be
+    FKD_DEV static f32 quick2(f32 x, f32 r, f32 l) { return __builtin_fmaf(x, r, x * l); }
+    // Straight-line variant: always returns the short sequence's result and clears `ok` when that result may not be
     // the correctly rounded quotient for this element; the caller then recomputes the element with exec().
     static constexpr bool kQuick = kReciprocal;
     FKD_DEV static O exec_quick(const I& a, const Params& p, bool& ok) {
@@ -640,6 +715,13 @@ template <class I, class P, class O> struct Div {
         if constexpr (cn_v<I> > 3) { sum += __builtin_fabsf(chan<3>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<3>(a))); }
         ok = ok && p.fast != 0 && sum <= 0x1p60f && least >= 0x1p-60f;
         O o;
+        if (p.fast == 2) {      // launch constant: a scalar branch
+            chan<0>(o) = quick2(chan<0>(a), chan_or_scalar<0>(p.rcp), chan_or_scalar<0>(p.rcp_lo));
+            if constexpr (cn_v<O> > 1) chan<1>(o) = quick2(chan<1>(a), chan_or_scalar<1>(p.rcp), chan_or_scalar<1>(p.rcp_lo));
+            if constexpr (cn_v<O> > 2) chan<2>(o) = quick2(chan<2>(a), chan_or_scalar<2>(p.rcp), chan_or_scalar<2>(p.rcp_lo));
+            if constexpr (cn_v<O> > 3) chan<3>(o) = quick2(chan<3>(a), chan_or_scalar<3>(p.rcp), chan_or_scalar<3>(p.rcp_lo));
+            return o;
+        }
         chan<0>(o) = quick1(chan<0>(a), chan_or_scalar<0>(p.v), chan_or_scalar<0>(p.rcp));
         if constexpr (cn_v<O> > 1) chan<1>(o) = quick1(chan<1>(a), chan_or_scalar<1>(p.v), chan_or_scalar<1>(p.rcp));
         if constexpr (cn_v<O> > 2) chan<2>(o) = quick1(chan<2>(a), chan_or_scalar<2>(p.v), chan_or_scalar<2>(p.rcp));
@@ -1949,10 +2031,10 @@ template <class T> struct TensorSplit {
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
         u32 off = u32(x) * u32(sizeof(B));   // one lane offset, four wave-uniform plane row addresses
         asm volatile("" : "+v"(off));
-        *detail::gmut<B>(reinterpret_cast<char*>(r.p) + off) = chan<0>(v);
-        *detail::gmut<B>(reinterpret_cast<char*>(r.p + r.px) + off) = chan<1>(v);
-        if constexpr (cn_v<T> > 2) *detail::gmut<B>(reinterpret_cast<char*>(r.p + 2 * r.px) + off) = chan<2>(v);
-        if constexpr (cn_v<T> > 3) *detail::gmut<B>(reinterpret_cast<char*>(r.p + 3 * r.px) + off) = chan<3>(v);
+        detail::gstore_through(detail::gmut<B>(reinterpret_cast<char*>(r.p) + off), chan<0>(v));
+        detail::gstore_through(detail::gmut<B>(reinterpret_cast<char*>(r.p + r.px) + off), chan<1>(v));
+        if constexpr (cn_v<T> > 2) detail::gstore_through(detail::gmut<B>(reinterpret_cast<char*>(r.p + 2 * r.px) + off), chan<2>(v));
+        if constexpr (cn_v<T> > 3) detail::gstore_through(detail::gmut<B>(reinterpret_cast<char*>(r.p + 3 * r.px) + off), chan<3>(v));
     }
     template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<T> (&v)[V]) {
         const u32 off = u32(x) * u32(sizeof(B));

@@ -402,6 +402,23 @@ int fklcase_div_f32(void* stream_, const float* in, int w, int h, int pitch, flo
                                           PerThreadWrite<ND::_2D, float>::build(o.ptr()));
     });
 }
+// How the host would divide by d on the device: 0 generic division, 1 five-instruction sequence, 2 two-instruction
+// sequence proven exact for this divisor (fkd::Div).
+int fklcase_div_mode(float d) { return fkd::Div<float, float, float>::make(d).fast; }
+// The same one-operation chain with the sequence chosen by the caller instead of by the host's proof, through the C
+// ABI with a hand-built parameter block: lets a test compare the proof's verdict with what the device really computes.
+int fklcase_div_f32_forced(void* stream_, const float* in, int w, int h, int pitch, float d, int mode, float* out, int out_pitch) {
+    using DivOp = fkd::Div<float, float, float>;
+    using Chain = fkd::Chain<fkd::Read2D<float>, fkd::OpList<DivOp>, fkd::Write2D<float>>;
+    Chain::Params p{};
+    p.active_w = unsigned(w); p.active_h = unsigned(h); p.active_z = 1;
+    p.read = {in, unsigned(w), unsigned(h), unsigned(pitch)};
+    p.ops.head = DivOp::make(d);
+    if (p.ops.head.fast == 0 && mode != 0) return -2;          // the reciprocals were not computed for this divisor
+    p.ops.head.fast = mode;
+    p.write = {out, unsigned(w), unsigned(h), unsigned(out_pitch)};
+    return fklhip_launch(Chain::name().c_str(), &p, sizeof(p), stream_);
+}
 int fklcase_div_f32x3(void* stream_, const float* in, int w, int h, int pitch, const float* d, float* out, int out_pitch) {
     return guarded([&] {
         Stream stream(stream_);

@@ -124,6 +124,64 @@ def test_div_scalar_every_bit_pattern(device, d):
             pytest.fail(f"x bits {int(x[y, xx].view(torch.int32)) & 0xffffffff:#010x} / {d!r}: got {float(out[y, xx])!r}")
 
 
+# ---- the two-instruction quotient and the host's proof that a divisor admits it ------------------------------------
+
+def _random_divisors(n, seed):
+    rng = np.random.RandomState(seed)
+    mant = rng.randint(0, 1 << 23, size=n, dtype=np.int64)
+    expo = rng.randint(127 - 20, 127 + 20, size=n, dtype=np.int64)
+    sign = rng.randint(0, 2, size=n, dtype=np.int64)
+    return [float(_f(int((s << 31) | (e << 23) | m))) for s, e, m in zip(sign, expo, mant)]
+
+
+def _mismatches_forced(torch, device, d, mode):
+    """Number of x (all 2^32) for which the chain with the given sequence differs from IEEE division, and one such x."""
+    out = torch.empty((SIDE, SIDE), dtype=torch.float32, device=device)
+    dt = torch.tensor(d, dtype=torch.float32, device=device)
+    count, first = 0, None
+    for k in range(16):
+        x = _chunk(torch, device, k)
+        cases.div_f32_forced(x, d, mode, out)
+        torch.cuda.synchronize()
+        ok, mask = _same(torch, out, x / dt)
+        if not ok:
+            count += int((~mask).sum())
+            if first is None:
+                y, xx = (~mask).nonzero()[0].tolist()
+                first = int(x[y, xx].view(torch.int32)) & 0xffffffff
+    return count, first
+
+
+def test_two_step_division_where_the_host_proves_it(device):
+    """Random divisors plus the benchmark's: wherever the host's proof admits the two-instruction sequence, every one
+    of the 2^32 numerators must give the IEEE quotient; the proof must also admit most divisors, or it is useless."""
+    import torch
+    divisors = [float(v) for v in wl.C3_STD] + [3.0, 0.1, -7.25, 255.0, float(_f(0x3FFFFFFF)), float(_f(0x3F800001))] + _random_divisors(16, 21)
+    admitted = 0
+    for d in divisors:
+        mode = cases.div_mode(d)
+        assert mode in (1, 2), (d, mode)
+        if mode == 2:
+            admitted += 1
+            count, first = _mismatches_forced(torch, device, d, 2)
+            assert count == 0, f"divisor {d!r} was admitted but x bits {first:#010x} give a wrong quotient ({count} in all)"
+    assert admitted >= len(divisors) // 2, f"only {admitted} of {len(divisors)} divisors admitted"
+
+
+def test_two_step_division_fails_where_the_host_refuses(device):
+    """The other direction, so that the proof is not vacuous: among many divisors find some that the host refuses,
+    force the two-instruction sequence on them anyway, and see wrong quotients on the device."""
+    import torch
+    refused = [d for d in _random_divisors(4000, 22) if cases.div_mode(d) == 1][:3]
+    if not refused:
+        pytest.skip("no divisor among 4000 was refused")
+    for d in refused:
+        count, first = _mismatches_forced(torch, device, d, 2)
+        assert count > 0, f"divisor {d!r} was refused, yet the two-instruction sequence is exact for every numerator"
+        count5, _ = _mismatches_forced(torch, device, d, 1)
+        assert count5 == 0, d
+
+
 def _torch_saturate_u8(torch, x):
     r = torch.round(x)                                   # half to even
     r = torch.where(torch.isnan(x), torch.zeros_like(r), r)
