@@ -112,6 +112,13 @@ def div_f32(src, d, out):
                                 _p(out), out.stride(0) * 4))
 
 
+def normalise_mode(kind, sub, div) -> int:
+    """fkd::Div's mode word for (x - sub) / div behind a bounded read (kind 0), a float image (1), a letterboxed resize (2):
+    low two bits as div_mode, bit 2 set when the chain proves the range and the device skips its per-element test."""
+    return int(cases().fklcase_normalise_mode(int(kind), _host(sub, np.float32).ctypes.data_as(C.POINTER(C.c_float)),
+                                              _host(div, np.float32).ctypes.data_as(C.POINTER(C.c_float))))
+
+
 def div_mode(d) -> int:
     """0 generic division, 1 five-instruction sequence, 2 two-instruction sequence proven exact for this divisor."""
     l = cases()

@@ -314,8 +314,10 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     //             where the zeros of the other three terms decide the sign of the sum, takes all four after all.
     constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3, kPairsPrepared = 4, kWhole = 5;
     const int yend = y0 + YI < ah ? y0 + YI : ah;
-    auto rows = [&](auto mode_tag) {
+    // STATIC: every quick operation of the chain takes its static form (decided once per wave, below).
+    auto rows_with = [&](auto mode_tag, auto static_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
+        constexpr bool STATIC = decltype(static_tag)::value != 0;
         constexpr bool PAIRED = MODE == kPairs || MODE == kPairsSel || MODE == kPairsPrepared;
         detail::PairPrep prep[XI];
         detail::TapImage image;
@@ -398,7 +400,8 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
                         v = RZ::blend(first, Back::finish(b, q.back), Back::finish(c, q.back), Back::finish(d, q.back), tp);
                     }
                     if constexpr (RZ::kAR != IGNORE_AR) { if (!(yin && xin[i])) v = q.bg; }
-                    res[i].v = Chain::compute_checked_ops(v, ops);
+                    if constexpr (STATIC) res[i].v = Chain::compute_static_ops(v, ops);
+                    else res[i].v = Chain::compute_checked_ops(v, ops);
                     continue;
                 }
                 if constexpr (PAIRED) {
@@ -413,7 +416,8 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
                 typename RZ::Out v = RZ::blend(Back::finish(a, q.back), Back::finish(b, q.back),
                                                Back::finish(c, q.back), Back::finish(d, q.back), tp);
                 if constexpr (RZ::kAR != IGNORE_AR) { if (!(yin && xin[i])) v = q.bg; }
-                res[i].v = Chain::compute_checked_ops(v, ops);
+                if constexpr (STATIC) res[i].v = Chain::compute_static_ops(v, ops);
+                else res[i].v = Chain::compute_checked_ops(v, ops);
             }
             if constexpr (FKD_GATHER_ADJ && XI > 1) {
                 if (xof(XI - 1) < aw) {
@@ -453,6 +457,12 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
             }
         }
     };
+    auto rows = [&](auto mode_tag) {
+        if constexpr (Chain::kQuick) {
+            if (Chain::ops_static(ops)) { rows_with(mode_tag, IntTag<1>{}); return; }
+        }
+        rows_with(mode_tag, IntTag<0>{});
+    };
     // Whole-dword reads of 3- and 6-byte elements (and pair reads) touch up to 3 bytes past what they need.  Inside
     // the image that is the next element or row; only in the image's last row it could leave the allocation.
     bool tail = false;
@@ -462,7 +472,7 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
         const int yb = yl + 1 < sh - 1 ? yl + 1 : sh - 1;
         tail = Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back));
     }
-    if constexpr (detail::finite_taps<Back>()) {
+    if constexpr (finite_taps<Back>()) {
         // whole factors, and every source coordinate an exact float
         const bool whole = q.fx >= 1.0f && q.fy >= 1.0f && q.fx == __builtin_floorf(q.fx) && q.fy == __builtin_floorf(q.fy) &&
                            f32(aw) * q.fx <= 16777216.0f && f32(ah) * q.fy <= 16777216.0f;

@@ -30,6 +30,26 @@ inline std::string istr(long long v) { return std::to_string(v); }
 // vectors that the backend can only legalise through scratch or LDS.
 template <class T> struct alignas(sizeof(T) % 4 != 0 ? 4 : alignof(T)) Slot { T v; };
 
+// Facts about values that only types can vouch for, used where an operation may be shortened if its input is tame.
+// finite_taps<B>: the taps of read B, after everything fused into it, are finite numbers whatever the image holds
+// (integer pixels through operations without run-time parameters); a tap with weight zero then contributes a zero and can
+// be left out of a blend.  finite_map<Op>: Op maps finite inputs of moderate size to finite outputs of moderate size and
+// has no run-time parameters.  bounded_out<R>: what read R hands to the chain is finite and below 2^30 in magnitude.
+template <class B> constexpr bool finite_taps() {
+    if constexpr (requires { B::kFiniteTaps; }) return B::kFiniteTaps; else return false;
+}
+template <class Op> constexpr bool finite_map() {
+    if constexpr (requires { Op::kFiniteMap; }) return Op::kFiniteMap; else return false;
+}
+template <class R> constexpr bool bounded_out() {
+    if constexpr (requires { R::kBoundedOut; }) return R::kBoundedOut; else return false;
+}
+template <class T> constexpr bool small_integer_base() {
+    return !(__is_same(base_t<T>, f32) || __is_same(base_t<T>, f64)) && sizeof(base_t<T>) <= 2;
+}
+template <int I, class T, class... Ts> struct TypeAt { using type = typename TypeAt<I - 1, Ts...>::type; };
+template <class T, class... Ts> struct TypeAt<0, T, Ts...> { using type = T; };
+
 #if defined(FKD_DEVICE_CODE)
 namespace detail {
 
@@ -418,15 +438,6 @@ struct PairPrep { u32 off, shift; };
 template <class B> constexpr bool tap_prepared() {
     if constexpr (requires { B::kTapPrepared; }) return B::kTapPrepared; else return false;
 }
-// Reads whose taps, after everything fused into the read, are finite numbers whatever the image holds (integer
-// pixels through operations without run-time parameters): a tap with weight zero then contributes a zero and can be
-// left out of a blend.  Compute operations say so with kFiniteMap.
-template <class B> constexpr bool finite_taps() {
-    if constexpr (requires { B::kFiniteTaps; }) return B::kFiniteTaps; else return false;
-}
-template <class Op> constexpr bool finite_map() {
-    if constexpr (requires { Op::kFiniteMap; }) return Op::kFiniteMap; else return false;
-}
 struct TapImage {
 #if defined(FKD_DEVICE_CODE)
     __amdgpu_buffer_rsrc_t rsrc;
@@ -603,10 +614,18 @@ FKD_BINARY_OP(Mul, x * y)
 // rounded quotient the sequence is exact for that divisor and ALL x (powers of two only shift exponents; the range
 // conditions above, with 2^-30 <= |y| <= 2^30, keep every intermediate normal or harmlessly small), otherwise the divisor
 // keeps the five-instruction form.
+//
+// The per-element range test (7 instructions per pixel) goes away when the chain proves the range, which it can for the
+// usual normalisation (x - mean) / std: see Chain::finalize.  A division with both proofs (fast == 2 | kInputProven) is
+// "static": exec_static is the two instructions and nothing else, and kernels pick the code path built from it once per
+// wave, because a test of `fast` inside the per-element code costs as much as the shorter sequence saves.
 template <class I, class P, class O> struct Div {
     using In = I; using Out = O;
     static constexpr bool kReciprocal = __is_same(base_t<I>, f32) && __is_same(base_t<P>, f32) && __is_same(base_t<O>, f32);
     struct Params { P v; P rcp; P rcp_lo; i32 fast; };
+    // `fast`: low two bits 0 generic division, 1 five instructions, 2 two instructions; kInputProven: the chain has
+    // shown that every element reaching this division is zero or has 2^-60 <= |x| <= 2^60 (Chain::finalize).
+    static constexpr i32 kInputProven = 4;
     FKD_NAME("Div<" + type_name<I>() + "," + type_name<P>() + "," + type_name<O>() + ">")
 
 #if !defined(FKD_DEVICE_CODE)
@@ -704,6 +723,15 @@ template <class I, class P, class O> struct Div {
         return __builtin_fmaf(e1, r, q1);
     }
     FKD_DEV static f32 quick2(f32 x, f32 r, f32 l) { return __builtin_fmaf(x, r, x * l); }
+    FKD_DEV static bool is_static(const Params& p) { return p.fast == (2 | kInputProven); }
+    FKD_DEV static O exec_static(const I& a, const Params& p) {
+        O o;
+        chan<0>(o) = quick2(chan<0>(a), chan_or_scalar<0>(p.rcp), chan_or_scalar<0>(p.rcp_lo));
+        if constexpr (cn_v<O> > 1) chan<1>(o) = quick2(chan<1>(a), chan_or_scalar<1>(p.rcp), chan_or_scalar<1>(p.rcp_lo));
+        if constexpr (cn_v<O> > 2) chan<2>(o) = quick2(chan<2>(a), chan_or_scalar<2>(p.rcp), chan_or_scalar<2>(p.rcp_lo));
+        if constexpr (cn_v<O> > 3) chan<3>(o) = quick2(chan<3>(a), chan_or_scalar<3>(p.rcp), chan_or_scalar<3>(p.rcp_lo));
+        return o;
+    }
     // Straight-line variant: always returns the short sequence's result and clears `ok` when that result may not be
     // the correctly rounded quotient for this element; the caller then recomputes the element with exec().
     static constexpr bool kQuick = kReciprocal;
@@ -713,9 +741,9 @@ template <class I, class P, class O> struct Div {
         if constexpr (cn_v<I> > 1) { sum += __builtin_fabsf(chan<1>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<1>(a))); }
         if constexpr (cn_v<I> > 2) { sum += __builtin_fabsf(chan<2>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<2>(a))); }
         if constexpr (cn_v<I> > 3) { sum += __builtin_fabsf(chan<3>(a)); least = __builtin_fminf(least, __builtin_fabsf(chan<3>(a))); }
-        ok = ok && p.fast != 0 && sum <= 0x1p60f && least >= 0x1p-60f;
+        ok = ok && (p.fast & 3) != 0 && sum <= 0x1p60f && least >= 0x1p-60f;
         O o;
-        if (p.fast == 2) {      // launch constant: a scalar branch
+        if ((p.fast & 3) == 2) {      // launch constant: a scalar branch
             chan<0>(o) = quick2(chan<0>(a), chan_or_scalar<0>(p.rcp), chan_or_scalar<0>(p.rcp_lo));
             if constexpr (cn_v<O> > 1) chan<1>(o) = quick2(chan<1>(a), chan_or_scalar<1>(p.rcp), chan_or_scalar<1>(p.rcp_lo));
             if constexpr (cn_v<O> > 2) chan<2>(o) = quick2(chan<2>(a), chan_or_scalar<2>(p.rcp), chan_or_scalar<2>(p.rcp_lo));
@@ -749,6 +777,7 @@ template <class Op, int N> struct StaticLoop {
 // Cast<I,O>: per-channel static_cast.  FK/algorithms/basic_ops/cast.h:22-33.
 template <class I, class O> struct Cast {
     using In = I; using Out = O; using Params = Empty;
+    static constexpr bool kFiniteMap = __is_same(base_t<O>, f32) && sizeof(base_t<I>) <= 4 && !__is_same(base_t<I>, f64);
     FKD_NAME("Cast<" + type_name<I>() + "," + type_name<O>() + ">")
     FKD_DEV static O exec(const I& a, const Params&) {
         return map1<O>(a, [](auto x) { return static_cast<base_t<O>>(x); });
@@ -1022,18 +1051,40 @@ FKD_DEV auto fold_quick(const V& v, const Tup<typename Op::Params, typename Rest
     else return fold_quick<Rest...>(step(), p.tail, ok);
 }
 
+// The fold with every quick operation in its static form (see Div), and whether the parameters allow it.
+template <class V> FKD_DEV V fold_static(const V& v, const Tup<>&) { return v; }
+template <class Op, class... Rest, class V>
+FKD_DEV auto fold_static(const V& v, const Tup<typename Op::Params, typename Rest::Params...>& p) {
+    auto step = [&] {
+        if constexpr (has_quick<Op>()) return Op::exec_static(v, p.head); else return Op::exec(v, p.head);
+    };
+    if constexpr (sizeof...(Rest) == 0) return step();
+    else return fold_static<Rest...>(step(), p.tail);
+}
+FKD_DEV inline bool all_static(const Tup<>&) { return true; }
+template <class Op, class... Rest>
+FKD_DEV bool all_static_of(const Tup<typename Op::Params, typename Rest::Params...>& p) {
+    bool here = true;
+    if constexpr (has_quick<Op>()) here = Op::is_static(p.head);
+    if constexpr (sizeof...(Rest) == 0) return here;
+    else return here && all_static_of<Rest...>(p.tail);
+}
+
 // The fold over a run of N elements, operation by operation: every element goes through operation k before any
 // goes through operation k+1.  A long chain then needs each operation's parameters (scalar registers) only once and
 // only briefly, instead of all parameters of the chain at the same time for every element.
-template <bool QUICK, int N, class V> FKD_DEV void fold_run(const Slot<V> (&in)[N], Slot<V> (&out)[N], const Tup<>&, bool&) {
+// QUICK: 0 every operation as written, 1 quick forms that report doubtful elements through `ok`, 2 static forms.
+template <int QUICK, int N, class V> FKD_DEV void fold_run(const Slot<V> (&in)[N], Slot<V> (&out)[N], const Tup<>&, bool&) {
 #pragma unroll
     for (int i = 0; i < N; ++i) out[i].v = in[i].v;
 }
-template <bool QUICK, class Op, class... Rest, int N, class V, class O>
+template <int QUICK, class Op, class... Rest, int N, class V, class O>
 FKD_DEV void fold_run(const Slot<V> (&in)[N], Slot<O> (&out)[N], const Tup<typename Op::Params, typename Rest::Params...>& p, bool& ok) {
     static_assert(__is_same(V, typename Op::In), "operation input type does not match the value it receives");
     auto step = [&](const V& v) {
-        if constexpr (QUICK && has_quick<Op>()) return Op::exec_quick(v, p.head, ok); else return Op::exec(v, p.head);
+        if constexpr (QUICK == 2 && has_quick<Op>()) return Op::exec_static(v, p.head);
+        else if constexpr (QUICK == 1 && has_quick<Op>()) return Op::exec_quick(v, p.head, ok);
+        else return Op::exec(v, p.head);
     };
     if constexpr (sizeof...(Rest) == 0) {
 #pragma unroll
@@ -1123,6 +1174,7 @@ template <class T> struct Read2D {
     using Params = RawPtr2D<const T>;
     static constexpr bool kTapCursor = true;
     static constexpr bool kFiniteTaps = !(__is_same(base_t<T>, f32) || __is_same(base_t<T>, f64));
+    static constexpr bool kBoundedOut = small_integer_base<T>();
     FKD_NAME("Read2D<" + type_name<T>() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -1190,6 +1242,7 @@ template <class T> struct Read3D {
     using Out = T;
     using Params = RawPtr3D<const T>;
     static constexpr bool kTapCursor = false;
+    static constexpr bool kBoundedOut = small_integer_base<T>();
     FKD_NAME("Read3D<" + type_name<T>() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -1328,6 +1381,7 @@ template <bool VU> struct ReadNV {
     using Params = RawNV12;
     static constexpr bool kTapCursor = true;
     static constexpr bool kFiniteTaps = true;
+    static constexpr bool kBoundedOut = true;
     FKD_NAME(VU ? "ReadNV21" : "ReadNV12")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
@@ -1464,9 +1518,10 @@ template <class Back> struct Crop {
     using Out = typename Back::Out;
     struct Params { i32 x, y, w, h; typename Back::Params back; };
     static constexpr bool kTapCursor = Back::kTapCursor;
+    static constexpr bool kBoundedOut = bounded_out<Back>();
     FKD_NAME("Crop<" + Back::name() + ">")
 #if defined(FKD_DEVICE_CODE)
-    static constexpr bool kFiniteTaps = detail::finite_taps<Back>();
+    static constexpr bool kFiniteTaps = finite_taps<Back>();
     FKD_DEV static int width(const Params& p) { return p.w; }
     FKD_DEV static int height(const Params& p) { return p.h; }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) { return Back::exec(x + p.x, y + p.y, 0, p.back); }
@@ -1571,9 +1626,10 @@ template <class Back, class... Ops> struct FusedRead {
     using Out = typename FoldOut<typename Back::Out, Ops...>::type;
     struct Params { typename Back::Params back; Tup<typename Ops::Params...> ops; };
     static constexpr bool kTapCursor = Back::kTapCursor;
+    static constexpr bool kBoundedOut = bounded_out<Back>() && (finite_map<Ops>() && ...);
     FKD_NAME("FusedRead<" + Back::name() + OpList<Ops...>::names() + ">")
 #if defined(FKD_DEVICE_CODE)
-    static constexpr bool kFiniteTaps = detail::finite_taps<Back>() && (detail::finite_map<Ops>() && ...);
+    static constexpr bool kFiniteTaps = finite_taps<Back>() && (finite_map<Ops>() && ...);
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
@@ -1639,6 +1695,7 @@ template <int AR, class Back> struct ResizeLinear {
     };
     static constexpr bool kTapCursor = false;
     static constexpr int kAR = AR;
+    static constexpr bool kBoundedOut = AR == IGNORE_AR && bounded_out<Back>();   // a letterbox colour is a run-time value
     using BackOp = Back;
     FKD_NAME("ResizeLinear<" + istr(AR) + "," + Back::name() + ">")
 #if defined(FKD_DEVICE_CODE)
@@ -1848,6 +1905,7 @@ template <int N, class PlaneOp> struct BatchRead {
     static constexpr int kBatch = N;
     struct Params { typename PlaneOp::Params plane[N]; };
     static constexpr bool kTapCursor = false;
+    static constexpr bool kBoundedOut = bounded_out<PlaneOp>();
     FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
 #if defined(FKD_DEVICE_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
@@ -2201,6 +2259,11 @@ template <class W1, class W2> struct TeeWrite {
 // ===================================================================================================
 // A fused chain: one read, a fold of compute operations, one write, over an active grid.
 // ===================================================================================================
+template <class T> struct IsSubOp { static constexpr bool value = false; };
+template <class I, class P, class O> struct IsSubOp<Sub<I, P, O>> { static constexpr bool value = __is_same(base_t<I>, f32) && __is_same(base_t<P>, f32) && __is_same(base_t<O>, f32); };
+template <class T> struct IsDivOp { static constexpr bool value = false; };
+template <class I, class P, class O> struct IsDivOp<Div<I, P, O>> { static constexpr bool value = Div<I, P, O>::kReciprocal; };
+
 template <class R, class Ops, class W> struct Chain;
 template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     using Read = R;
@@ -2213,6 +2276,45 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
         typename W::Params write;
     };
     FKD_NAME("Chain<" + R::name() + ",OpList<" + (sizeof...(Ops) ? OpList<Ops...>::names().substr(1) : std::string()) + ">," + W::name() + ">")
+#if !defined(FKD_DEVICE_CODE)
+    // Host, once the parameter block is filled: what only the whole chain knows about the values an operation receives.
+    //
+    // Normalisation, (x - m) / d with launch constants: when the read hands over finite values below 2^30 (integer pixels,
+    // also bilinearly blended or colour converted) and only parameter-free finite maps sit between it and the
+    // subtraction, then a = the subtraction's input is finite with |a| < 2^30, and for 2^-20 <= |m| <= 2^59 the
+    // difference x = fl(a - m) is zero or has 2^-45 <= |x| < 2^60: if a and m have the same sign and lie within a factor of
+    // two of each other the difference is exact (Sterbenz) and a multiple of the smaller unit in the last place, at least
+    // 2^-24 * |m| / 2; otherwise |a - m| >= |m| / 2.  That is the range the division's short sequences need, so the
+    // device may skip its per-element test.  x = 0 gives the right zero only for a positive divisor (0 * l has the sign of
+    // l, and -0 + +0 is +0), hence d > 0 as well.
+    template <int K> static void finalize_from(Params& p) {
+        if constexpr (K + 1 < int(sizeof...(Ops))) {
+            using A = typename TypeAt<K, Ops...>::type;
+            using B = typename TypeAt<K + 1, Ops...>::type;
+            if constexpr (IsSubOp<A>::value && IsDivOp<B>::value && bounded_out<R>() && prefix_finite<K>()) {
+                const auto& sub = tup_get<K>(p.ops);
+                auto& div = tup_get<K + 1>(p.ops);
+                bool ok = (div.fast & 3) != 0;
+                auto mean_ok = [&](f32 m) { const f32 a = __builtin_fabsf(m); if (!(a >= 0x1p-20f && a <= 0x1p59f)) ok = false; };
+                auto div_ok = [&](f32 d) { if (!(d > 0.0f)) ok = false; };
+                mean_ok(chan_or_scalar<0>(sub.v)); div_ok(chan_or_scalar<0>(div.v));
+                if constexpr (cn_v<decltype(sub.v)> > 1) { mean_ok(chan<1>(sub.v)); }
+                if constexpr (cn_v<decltype(sub.v)> > 2) { mean_ok(chan<2>(sub.v)); }
+                if constexpr (cn_v<decltype(sub.v)> > 3) { mean_ok(chan<3>(sub.v)); }
+                if constexpr (cn_v<decltype(div.v)> > 1) { div_ok(chan<1>(div.v)); }
+                if constexpr (cn_v<decltype(div.v)> > 2) { div_ok(chan<2>(div.v)); }
+                if constexpr (cn_v<decltype(div.v)> > 3) { div_ok(chan<3>(div.v)); }
+                if (ok) div.fast |= B::kInputProven;
+            }
+            finalize_from<K + 1>(p);
+        }
+    }
+    template <int K> static constexpr bool prefix_finite() {
+        if constexpr (K == 0) return true;
+        else return finite_map<typename TypeAt<K - 1, Ops...>::type>() && prefix_finite<K - 1>();
+    }
+    static void finalize(Params& p) { finalize_from<0>(p); }
+#endif
 #if defined(FKD_DEVICE_CODE)
     static_assert(__is_same(Value, typename W::In), "the write operation does not take the type the chain produces");
     FKD_DEV static Value compute(const typename R::Out& v, const Params& p) {
@@ -2224,11 +2326,20 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     using OpParams = Tup<typename Ops::Params...>;
     FKD_DEV static Value compute_checked(const typename R::Out& v, const Params& p) { return compute_checked_ops(v, p.ops); }
     // N elements at once, operation-major (see fold_run); same results as compute() element by element.
+    // Whether every quick operation of the chain can take its static form in this launch (wave uniform), and the
+    // chain computed that way.
+    FKD_DEV static bool ops_static(const OpParams& ops) {
+        if constexpr (!kQuick) return false; else return all_static_of<Ops...>(ops);
+    }
+    FKD_DEV static Value compute_static_ops(const typename R::Out& v, const OpParams& ops) { return fold_static<Ops...>(v, ops); }
     template <int N> FKD_DEV static void compute_run(const Slot<typename R::Out> (&in)[N], Slot<Value> (&out)[N], const OpParams& ops) {
         bool ok = true;
+        if constexpr (kQuick) {
+            if (ops_static(ops)) { fold_run<2, Ops...>(in, out, ops, ok); return; }
+        }
         fold_run<kQuick, Ops...>(in, out, ops, ok);
         if constexpr (kQuick) {
-            if (__builtin_expect(!ok, 0)) fold_run<false, Ops...>(in, out, ops, ok);
+            if (__builtin_expect(!ok, 0)) fold_run<0, Ops...>(in, out, ops, ok);
         }
     }
     // The same for chains with many parameters; `kernarg` is the kernel-argument segment, holding a Params at offset 0.

@@ -75,6 +75,7 @@ template <typename... IOps> struct FusedChain {
             p.active_z = active.z;
             p.read = lower_iop(std::get<0>(all));
             p.ops = make_tup(lower_iop(std::get<Is + 1>(all))...);
+            Chain::finalize(p);
             if constexpr (kTee) {
                 p.write.first = lower_iop(std::get<N - 2>(all));
                 p.write.second = lower_iop(std::get<N - 1>(all));

@@ -402,6 +402,31 @@ int fklcase_div_f32(void* stream_, const float* in, int w, int h, int pitch, flo
                                           PerThreadWrite<ND::_2D, float>::build(o.ptr()));
     });
 }
+// The division mode word (fkd::Div::Params::fast) that the chain-level pass leaves for "(x - sub) / div" behind three
+// kinds of read: 0 a bilinear resize of uchar3 pixels (values bounded by construction), 1 a float image (anything
+// may arrive), 2 a letterboxed resize (the background colour is a run-time value).
+int fklcase_normalise_mode(int kind, const float* sub, const float* div) {
+    using namespace fkd;
+    using F3 = Vec<f32, 3>;
+    using SubOp = fkd::Sub<F3, F3, F3>;
+    using DivOp = fkd::Div<F3, F3, F3>;
+    auto run = [&](auto chain_tag) {
+        using C = typename decltype(chain_tag)::type;
+        typename C::Params p{};
+        constexpr int k = int(sizeof(p.ops) > sizeof(Tup<SubOp::Params, DivOp::Params>));   // a Reorder in front or not
+        tup_get<k>(p.ops).v = F3{sub[0], sub[1], sub[2]};
+        tup_get<k + 1>(p.ops) = DivOp::make(F3{div[0], div[1], div[2]});
+        C::finalize(p);
+        return int(tup_get<k + 1>(p.ops).fast);
+    };
+    using Px = Vec<u8, 3>;
+    switch (kind) {
+    case 0: return run(std::type_identity<Chain<ResizeLinear<1, fkd::Crop<Read2D<Px>>>, OpList<Reorder<F3, 2, 1, 0, 3>, SubOp, DivOp>, fkd::TensorSplit<F3>>>{});
+    case 1: return run(std::type_identity<Chain<Read2D<F3>, OpList<SubOp, DivOp>, Write2D<F3>>>{});
+    case 2: return run(std::type_identity<Chain<ResizeLinear<0, fkd::Crop<Read2D<Px>>>, OpList<SubOp, DivOp>, fkd::TensorSplit<F3>>>{});
+    default: return -1;
+    }
+}
 // How the host would divide by d on the device: 0 generic division, 1 five-instruction sequence, 2 two-instruction
 // sequence proven exact for this divisor (fkd::Div).
 int fklcase_div_mode(float d) { return fkd::Div<float, float, float>::make(d).fast; }
