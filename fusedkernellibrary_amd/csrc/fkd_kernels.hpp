@@ -200,7 +200,16 @@ constexpr int kGatherBY = FKD_GATHER_BY;
 
 struct TileGeom {
     u32 tiles_x, tiles_y, n_tiles;
+    // floor(2^32 / tiles_x) + 1 when (t * magic) >> 32 == t / tiles_x for every tile number t of a plane, else 0: the
+    // division then costs two scalar multiplications instead of a float reciprocal on the vector unit.
+    u32 tiles_x_magic;
 };
+// The magic for dividing numbers below `limit` by d, or 0 when there is none.
+inline u32 division_magic(u32 d, u32 limit) {
+    if (d == 0) return 0;
+    const unsigned long long m = (1ull << 32) / d + 1;        // m * d - 2^32 is in (0, d]; exact while n * d < 2^32
+    return (m < (1ull << 32) && (unsigned long long)limit * d < (1ull << 32)) ? u32(m) : 0u;
+}
 
 // A workgroup owns a (64*XI) x (4*YI) tile of the output of one plane; wave w owns rows w*YI .. w*YI+YI-1 of it, so
 // everything that depends on the row (source rows, vertical weights, row addresses of source and destination) is
@@ -240,9 +249,10 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     const u32 chunk = (per_plane + 7u) / 8u;
     const u32 tin = (blockIdx.x % 8u) * chunk + blockIdx.x / 8u;
     if (tin >= per_plane) return;
-    const int tx0 = int(tin % gg.tiles_x) * TW;
+    const u32 tile_row = gg.tiles_x_magic ? u32(((unsigned long long)tin * gg.tiles_x_magic) >> 32) : tin / gg.tiles_x;
+    const int tx0 = int(tin - tile_row * gg.tiles_x) * TW;
     const int wy = __builtin_amdgcn_readfirstlane(int(threadIdx.y));
-    const int y0 = int(tin / gg.tiles_x) * TH + wy * YI;
+    const int y0 = int(tile_row) * TH + wy * YI;
     if (y0 >= ah) return;
     if constexpr (HasDefaultPlanes<typename Chain::Read>::value) {
         // BatchRead<CONDITIONAL_WITH_DEFAULT>: planes at or beyond `used` read nothing; every element is the default
@@ -473,10 +483,8 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
         tail = Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back));
     }
     if constexpr (finite_taps<Back>()) {
-        // whole factors, and every source coordinate an exact float
-        const bool whole = q.fx >= 1.0f && q.fy >= 1.0f && q.fx == __builtin_floorf(q.fx) && q.fy == __builtin_floorf(q.fy) &&
-                           f32(aw) * q.fx <= 16777216.0f && f32(ah) * q.fy <= 16777216.0f;
-        if (whole) { rows(IntTag<kWhole>{}); return; }
+        // whole factors, and every source coordinate an exact float: decided on the host (ResizeLinear::whole_factors)
+        if (q.whole) { rows(IntTag<kWhole>{}); return; }
     }
     if (tail) {
         rows(IntTag<kSafe>{});

@@ -34,6 +34,7 @@ hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, La
     g.tiles_x = (p.active_w + TW - 1) / TW;
     g.tiles_y = (p.active_h + TH - 1) / TH;
     g.n_tiles = g.tiles_x * g.tiles_y * p.active_z;
+    g.tiles_x_magic = division_magic(g.tiles_x, g.tiles_x * g.tiles_y);
     const unsigned chunk = (g.tiles_x * g.tiles_y + 7u) / 8u;
     const dim3 grid(chunk * 8u, 1, p.active_z), block(kGatherBX, kGatherBY, 1);
     if (info) *info = LaunchInfo{"gather", {grid.x, 1, grid.z}, {block.x, block.y, 1}, 0};

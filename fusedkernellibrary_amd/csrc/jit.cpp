@@ -33,13 +33,19 @@
 namespace fklhip {
 namespace {
 
-// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): eight and three 32-bit words.
+// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): eight and four 32-bit words.
 struct JitMeta {
     unsigned gather, params_bytes, v, rows, xi, yi, by, reserved;
 };
 struct TileGeom {
-    unsigned tiles_x, tiles_y, n_tiles;
+    unsigned tiles_x, tiles_y, n_tiles, tiles_x_magic;
 };
+// As fkd::division_magic: floor(2^32 / d) + 1 when it divides every number below `limit` exactly, else 0.
+unsigned division_magic(unsigned d, unsigned limit) {
+    if (d == 0) return 0;
+    const unsigned long long m = (1ull << 32) / d + 1;
+    return (m < (1ull << 32) && (unsigned long long)limit * d < (1ull << 32)) ? unsigned(m) : 0u;
+}
 
 struct JitKernel {
     std::string signature;
@@ -156,13 +162,14 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
     unsigned active[3];
     memcpy(active, blob, sizeof(active));   // Chain::Params starts with active_w, active_h, active_z
     const JitMeta& m = k->meta;
-    TileGeom g{0, 0, 0};
+    TileGeom g{0, 0, 0, 0};
     unsigned grid[3], block[3] = {64, 4, 1};
     if (m.gather) {
         const unsigned tw = 64 * m.xi, th = m.by * m.yi;
         g.tiles_x = (active[0] + tw - 1) / tw;
         g.tiles_y = (active[1] + th - 1) / th;
         g.n_tiles = g.tiles_x * g.tiles_y * active[2];
+        g.tiles_x_magic = division_magic(g.tiles_x, g.tiles_x * g.tiles_y);
         grid[0] = (g.tiles_x * g.tiles_y + 7u) / 8u * 8u;
         grid[1] = 1;
         grid[2] = active[2];

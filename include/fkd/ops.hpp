@@ -1691,8 +1691,15 @@ template <int AR, class Back> struct ResizeLinear {
         f32 fx, fy;
         i32 x1, y1, x2, y2;
         Out bg;
+        i32 whole;      // whole_factors(dst_w, dst_h, fx, fy), filled by the host
         typename Back::Params back;
     };
+    // Both scale factors are whole numbers and every source coordinate index * factor is an exact float: every source
+    // point is then a pixel and the bilinear weights are exactly 1, 0, 0, 0.
+    FKD_HD static i32 whole_factors(i32 dst_w, i32 dst_h, f32 fx, f32 fy) {
+        return fx >= 1.0f && fy >= 1.0f && fx == __builtin_floorf(fx) && fy == __builtin_floorf(fy) &&
+               f32(dst_w) * fx <= 16777216.0f && f32(dst_h) * fy <= 16777216.0f;
+    }
     static constexpr bool kTapCursor = false;
     static constexpr int kAR = AR;
     static constexpr bool kBoundedOut = AR == IGNORE_AR && bounded_out<Back>();   // a letterbox colour is a run-time value

@@ -200,6 +200,7 @@ struct Lower<ResizeComplete<AR, Ternary<InterpolateComplete<IT, BackIOp>>>> {
         p.dst_h = d.params.dstSize.height;
         p.fx = d.params.src_conv_factors.x;
         p.fy = d.params.src_conv_factors.y;
+        p.whole = type::whole_factors(p.dst_w, p.dst_h, p.fx, p.fy);
         if constexpr (AR == AspectRatio::IGNORE_AR) {
             p.x1 = 0; p.y1 = 0; p.x2 = p.dst_w - 1; p.y2 = p.dst_h - 1;
         } else {
