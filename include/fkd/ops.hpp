@@ -1608,11 +1608,22 @@ template <int BT, class Back> struct Border {
             return Back::exec(fold(x, w), fold(y, h), z, p.back);
         }
     }
+    // A lane whose whole run lies between the image's left and right edge reads it as the image itself would (one wide
+    // access), from the folded row; only lanes that touch an edge go element by element.  The choice differs from lane to
+    // lane, so the wave-cooperative access mode is not handed on.
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        constexpr int kLaneMode = (A & 3) != 0 ? ((A & 4) | 1) : 0;
+        const int w = Back::width(p.back), h = Back::height(p.back);
+        const bool run_inside = x >= 0 && x + V <= w;
+        if constexpr (BT == 0) {
+            if (run_inside && y >= 0 && y < h) { Back::template exec_row<V, kLaneMode>(x, y, z, p.back, out); return; }
+        } else {
+            if (run_inside) { Back::template exec_row<V, kLaneMode>(x, fold(y, h), z, p.back, out); return; }
+        }
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
-    FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // element-wise either way
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
     using Raw = Out;
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
     struct TapRow {}; struct TapBits {}; struct PairBits {};
