@@ -1750,7 +1750,38 @@ template <int AR, class Back> struct ResizeLinear {
         if constexpr (AR == IGNORE_AR) return true;
         else return x >= p.x1 && x <= p.x2 && y >= p.y1 && y <= p.y2;
     }
+    static constexpr bool kPairTaps = [] {
+        if constexpr (requires { Back::kTapPair; }) return Back::kTapCursor && Back::kTapPair; else return false;
+    }();
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
+        if constexpr (kPairTaps) {
+            // The element-wise form of the bilinear read (kernels that keep one element per thread: several chains in
+            // one launch).  Taps x1 and x1 + 1 of a source line come in one access each, issued by every lane (lanes
+            // in the letterbox bars take the taps of pixel (0, 0) and drop them), so that no load waits behind a branch;
+            // a wave that touches the image's last line, where such an access could reach past the allocation, takes
+            // the tap-by-tap path below instead, all lanes together.
+            const int sw = Back::width(p.back), sh = Back::height(p.back);
+            const bool in = inside(x, y, p);
+            int xs = in ? x : 0, ys = in ? y : 0;
+            if constexpr (AR != IGNORE_AR) { if (in) { xs -= p.x1; ys -= p.y1; } }
+            const Taps t = taps(xs, ys, p, sw, sh);
+            const int x1 = t.x1 < 0 ? 0 : (t.x1 < sw - 1 ? t.x1 : sw - 1);      // no-ops wherever the reference is in bounds
+            const int y1 = t.y1 < 0 ? 0 : (t.y1 < sh - 1 ? t.y1 : sh - 1);
+            const int y2 = y1 + 1 < sh - 1 ? y1 + 1 : sh - 1;
+            const auto ra = Back::tap_row(0, y1, z, p.back), rb = Back::tap_row(0, y2, z, p.back);
+            const bool risky = sw < 2 || Back::tap_last(ra) || Back::tap_last(rb);
+            if (__builtin_amdgcn_ballot_w64(risky) == 0) {
+                const bool edge = x1 >= sw - 1;           // x1 + 1 is past the line: both taps are the last pixel
+                const int xp = edge ? sw - 2 : x1;
+                const auto wa = Back::pair_load(ra, xp, p.back), wb = Back::pair_load(rb, xp, p.back);
+                typename Back::Raw a0, a1, b0, b1;
+                Back::pair_values(wa, ra, xp, a0, a1);
+                Back::pair_values(wb, rb, xp, b0, b1);
+                const Out v = blend(Back::finish(edge ? a1 : a0, p.back), Back::finish(a1, p.back),
+                                    Back::finish(edge ? b1 : b0, p.back), Back::finish(b1, p.back), t);
+                if constexpr (AR == IGNORE_AR) return v; else return in ? v : p.bg;
+            }
+        }
         if (!inside(x, y, p)) return p.bg;
         if constexpr (AR != IGNORE_AR) { x -= p.x1; y -= p.y1; }
         const Taps t = taps(x, y, p, Back::width(p.back), Back::height(p.back));
