@@ -516,7 +516,7 @@ template <class Chain> struct RowsConfig {
     static constexpr bool kScattered = ResizeRoot<typename Chain::Read>::value || is_scattered_read<typename Chain::Read>();
     static constexpr int V = kScattered ? 1 : 4;
 #ifndef FKD_ROWS
-#define FKD_ROWS 4
+#define FKD_ROWS 2
 #endif
     static constexpr int ROWS = kScattered ? 1 : FKD_ROWS;
 };
