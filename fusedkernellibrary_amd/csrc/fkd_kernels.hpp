@@ -518,7 +518,10 @@ template <class Chain> struct RowsConfig {
 #ifndef FKD_ROWS
 #define FKD_ROWS 2
 #endif
-    static constexpr int ROWS = kScattered ? 1 : FKD_ROWS;
+    // Two rows per thread; chains long enough to be bound by instruction issue rather than by memory (more than 128
+    // bytes of operation parameters) take four, for the independent work per thread.
+    static constexpr bool kManyOps = sizeof(typename Chain::Params) - sizeof(typename Chain::Read::Params) - sizeof(typename Chain::Write::Params) > 128 + 16;
+    static constexpr int ROWS = kScattered ? 1 : (kManyOps ? 2 * FKD_ROWS : FKD_ROWS);
 };
 
 // ---- divergent batch kernel -------------------------------------------------------------------------------
