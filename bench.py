@@ -244,7 +244,7 @@ def main():
 
 # HBM bytes one launch of configuration 3 moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE scaled by what the
 # same counters read for the plain copy chain of known size (profiles/k_gather_config3_traffic.txt); None until measured.
-TRAFFIC_C3_BYTES = 51197000
+TRAFFIC_C3_BYTES = 51193000
 
 if __name__ == "__main__":
     main()
