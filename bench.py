@@ -232,7 +232,8 @@ def main():
         "dtype": "f32", "data": "synthetic (seeded uniform random pixels and crop rectangles)",
         "config": {"workload": "configs[2]: 64 crops of uchar3 BGR 1920x1080 -> bilinear 224x224 IGNORE_AR -> BGR2RGB -> "
                                "(x-mean)/std -> TensorSplit planar float32 64x3x224x224, one fused launch per step",
-                   "output_pixels_per_step": 64 * 224 * 224, "union_source_pixels": union_px},
+                   "output_pixels_per_step": 64 * 224 * 224, "union_source_pixels": union_px,
+                   "sum_of_crop_areas_bytes": int(sum(int(r[2]) * int(r[3]) for r in c3["rects"])) * 3},
         "roofline": {"bound": "hbm", "achieved": r3["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": r3["frac_of_hbm_peak"], "traffic": TRAFFIC_C3_BYTES,
                      "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"]},
