@@ -527,20 +527,20 @@ template <class Chain> struct RowsConfig {
 // ---- divergent batch kernel -------------------------------------------------------------------------------
 
 // Several chains in one launch of the rows kernel's geometry: plane z runs chain select[z] (wave uniform: the plane is
-// the grid's z index).  Every chain runs through the rows body, bilinear reads included (one element per thread); the
-// grid is laid out for the smallest elements-per-thread of the chains, and workgroups beyond a chain's own extent
-// leave at once.
-template <int A, int... Rest> struct MinOf { static constexpr int value = A; };
-template <int A, int B, int... Rest> struct MinOf<A, B, Rest...> { static constexpr int value = MinOf<(A < B ? A : B), Rest...>::value; };
+// the grid's z index).  Every chain runs through the rows body, bilinear reads included, all with the same elements per
+// thread; workgroups beyond a chain's own extent leave at once.
 template <class... Chains> struct RowsConfig<Divergent<Chains...>> {
-    static constexpr int V = MinOf<RowsConfig<Chains>::V...>::value;
-    static constexpr int ROWS = MinOf<RowsConfig<Chains>::ROWS...>::value;
+    // One geometry for every chain of the launch, gathering reads included (they then take their elements one after
+    // the other): with the grid laid out for the finest chain, the planes of the coarser ones launched up to 16 times
+    // the workgroups they needed, and those empty workgroups cost 4 us of a 31 us launch.
+    static constexpr int V = 4;
+    static constexpr int ROWS = FKD_ROWS;
 };
 template <int I, class First, class... Rest, class P>
 __device__ __forceinline__ void divergent_run(u32 sel, const P& p, const Tup<typename First::Params, typename Rest::Params...>& seq) {
     if (sel == u32(I)) {
         const u32 offset = u32(reinterpret_cast<const char*>(&seq.head) - reinterpret_cast<const char*>(&p));
-        rows_auto_body<First, RowsConfig<First>::V, RowsConfig<First>::ROWS>(seq.head, offset);
+        rows_auto_body<First, 4, FKD_ROWS>(seq.head, offset);
     } else if constexpr (sizeof...(Rest) > 0) {
         divergent_run<I + 1, Rest...>(sel, p, seq.tail);
     }
