@@ -69,6 +69,15 @@ template <class Chain> constexpr bool is_gather_chain() {
         return false;
 }
 
+// Stores of a lane-masking writer (kLaneMasked); other writers never reach these calls, the indirection only keeps their
+// instantiations from looking the members up.
+template <class WP, class Plane> __device__ __forceinline__ u32 masked_row_offset(int y, const Plane& plane) {
+    if constexpr (requires { WP::kLaneMasked; }) return WP::row_offset(y, plane); else return 0u;
+}
+template <class WP, class Plane, class V> __device__ __forceinline__ void masked_put(const Plane& plane, u32 row_off, u32 lane_off, const V& v) {
+    if constexpr (requires { WP::kLaneMasked; }) WP::put_masked(plane, row_off, lane_off, v);
+}
+
 // ---- rows kernel ---------------------------------------------------------------------------------------
 
 constexpr int kRowsBX = 64;   // lanes along x: one wave per row segment
@@ -236,11 +245,18 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     // Everything the wave needs from the kernel-argument segment, fetched in one go.
     const typename RZ::Params* rp;
     if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
-    const TileGeom gg = detail::scalar_copy(g);
-    const typename RZ::Params q = detail::scalar_copy(*rp);
-    const typename Chain::OpParams& ops = p.ops;        // needed only after the taps are on their way
     using WP = typename W::Plane;
-    const typename WP::Params& wpar = W::plane_params(p.write, z);
+    // A scalar load from the kernel-argument segment takes several hundred cycles, and a wave that lives for a few
+    // thousand cannot afford one round trip per first use: geometry, the plane's read parameters, the operations'
+    // parameters and the write's are requested back to back and waited for once.
+    TileGeom gg = g;
+    typename RZ::Params q = *rp;
+    typename Chain::OpParams ops = p.ops;
+    typename WP::Params wpar = W::plane_params(p.write, z);
+    detail::pin_scalars(gg);
+    detail::pin_scalars(q);
+    detail::pin_scalars(ops);
+    detail::pin_scalars(wpar);
     u32 dims[2] = {p.active_w, p.active_h};
     asm volatile("" : "+s"(dims[0]), "+s"(dims[1]));
     const int aw = int(dims[0]), ah = int(dims[1]);
@@ -325,9 +341,18 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     constexpr int kSafe = 0, kSingles = 1, kPairs = 2, kPairsSel = 3, kPairsPrepared = 4, kWhole = 5;
     const int yend = y0 + YI < ah ? y0 + YI : ah;
     // STATIC: every quick operation of the chain takes its static form (decided once per wave, below).
-    auto rows_with = [&](auto mode_tag, auto static_tag) {
+    // Writers that can switch lanes off through their offset (kLaneMasked) store without an execution mask and with
+    // 32-bit scalar row arithmetic; image planes too large for that (plane_maskable) take the plain stores.
+    constexpr bool kCanMask = [] { if constexpr (requires { WP::kLaneMasked; }) return WP::kLaneMasked && !FKD_GATHER_ADJ; else return false; }();
+    auto make_plane = [&] { if constexpr (kCanMask) return WP::plane_ref(z, wpar); else return 0; };
+    const auto oplane = make_plane();
+    u32 lane_off[XI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) { if constexpr (kCanMask) lane_off[i] = WP::lane_offset(xof(i), xof(i) < aw); else lane_off[i] = 0; }
+    auto rows_with = [&](auto mode_tag, auto static_tag, auto masked_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
         constexpr bool STATIC = decltype(static_tag)::value != 0;
+        constexpr bool MASKED = decltype(masked_tag)::value != 0;
         constexpr bool PAIRED = MODE == kPairs || MODE == kPairsSel || MODE == kPairsPrepared;
         detail::PairPrep prep[XI];
         detail::TapImage image;
@@ -381,7 +406,8 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
             if (y >= yend) return;
             bool yin = true;
             if constexpr (RZ::kAR != IGNORE_AR) yin = y >= q.y1 && y <= q.y2;
-            const typename WP::RowRef orow = WP::row(y, z, wpar);
+            typename WP::RowRef orow;
+            if constexpr (!MASKED) orow = WP::row(y, z, wpar);
             Slot<typename Chain::Value> res[XI];
 #pragma unroll
             for (int i = 0; i < XI; ++i) {
@@ -429,7 +455,11 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
                 if constexpr (STATIC) res[i].v = Chain::compute_static_ops(v, ops);
                 else res[i].v = Chain::compute_checked_ops(v, ops);
             }
-            if constexpr (FKD_GATHER_ADJ && XI > 1) {
+            if constexpr (MASKED) {
+                const u32 row_off = masked_row_offset<WP>(y, oplane);
+#pragma unroll
+                for (int i = 0; i < XI; ++i) masked_put<WP>(oplane, row_off, lane_off[i], res[i].v);
+            } else if constexpr (FKD_GATHER_ADJ && XI > 1) {
                 if (xof(XI - 1) < aw) {
                     WP::template put_run<XI>(orow, xof(0), res);
                 } else {
@@ -469,9 +499,9 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
     };
     auto rows = [&](auto mode_tag) {
         if constexpr (Chain::kQuick) {
-            if (Chain::ops_static(ops)) { rows_with(mode_tag, IntTag<1>{}); return; }
+            if (Chain::ops_static(ops)) { rows_with(mode_tag, IntTag<1>{}, IntTag<kCanMask ? 1 : 0>{}); return; }
         }
-        rows_with(mode_tag, IntTag<0>{});
+        rows_with(mode_tag, IntTag<0>{}, IntTag<kCanMask ? 1 : 0>{});
     };
     // Whole-dword reads of 3- and 6-byte elements (and pair reads) touch up to 3 bytes past what they need.  Inside
     // the image that is the next element or row; only in the image's last row it could leave the allocation.
@@ -481,6 +511,13 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
         const int yl = int(__builtin_floorf(f32(ylast - oy) * q.fy));
         const int yb = yl + 1 < sh - 1 ? yl + 1 : sh - 1;
         tail = Back::tap_last(Back::tap_row(0, yb < 0 ? 0 : yb, z, q.back));
+    }
+    if constexpr (kCanMask) {
+        if (!WP::plane_maskable(wpar)) {
+            if (tail) rows_with(IntTag<kSafe>{}, IntTag<0>{}, IntTag<0>{});
+            else rows_with(IntTag<kSingles>{}, IntTag<0>{}, IntTag<0>{});
+            return;
+        }
     }
     if constexpr (finite_taps<Back>()) {
         // whole factors, and every source coordinate an exact float: decided on the host (ResizeLinear::whole_factors)

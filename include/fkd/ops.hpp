@@ -557,6 +557,19 @@ template <class T> FKD_DEV T scalar_copy(const T& src) {
     }
 }
 
+// Pins an object that is wave uniform into scalar registers where it stands (objects whose size is not a whole number
+// of dwords, or that are larger than 256 bytes, are left to the compiler).
+template <class T> FKD_DEV void pin_scalars(T& v) {
+    if constexpr (sizeof(T) % 4 == 0 && sizeof(T) <= 256 && __is_trivially_copyable(T)) {
+        constexpr int N = int(sizeof(T)) / 4;
+        u32 w[N];
+        __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+        for (int i = 0; i < N; ++i) asm volatile("" : "+s"(w[i]));
+        __builtin_memcpy(&v, w, sizeof(T));
+    }
+}
+
 FKD_HD bool dword_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 template <class T> FKD_DEV const T* row_ptr(const T* data, u32 pitch, int x, int y) {
@@ -2133,6 +2146,34 @@ template <class T> struct TensorSplit {
     // The part of the parameters one plane needs (all of them here).
     using Plane = TensorSplit;
     FKD_DEV static const Params& plane_params(const Params& p, int) { return p; }
+    // Stores through a buffer resource, for kernels whose lanes keep their column while their wave walks down rows:
+    // image plane z with all its channel planes is one resource, a row and a channel plane are a scalar offset, the
+    // column is the lane's offset, and a lane outside the image carries an offset beyond the resource's extent, so the
+    // address check drops its store and the wave needs no execution mask around the stores.  Scalar work per row: one
+    // multiplication and one addition per channel, in 32 bits.  For image planes smaller than 2 GB (plane_maskable).
+    static constexpr bool kLaneMasked = sizeof(B) == 4;
+    static constexpr u32 kMaskedExtent = 0x7fffffffu, kMaskedOut = 0x80000000u;
+    struct PlaneRef { __amdgpu_buffer_rsrc_t rsrc; u32 chan_bytes, pitch; };
+    FKD_DEV static bool plane_maskable(const Params& p) {
+        return size_t(p.width) * p.height * sizeof(B) * cn_v<T> < size_t(kMaskedExtent) && size_t(p.pitch) * p.height < size_t(kMaskedExtent);
+    }
+    FKD_DEV static PlaneRef plane_ref(int z, const Params& p) {
+        char* base = reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z;
+        PlaneRef r;
+        r.rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, kMaskedExtent, 0x00020000);   // raw 32-bit data, as detail::make_tap_image
+        r.chan_bytes = p.width * p.height * u32(sizeof(B));
+        r.pitch = p.pitch;
+        return r;
+    }
+    FKD_DEV static u32 lane_offset(int x, bool valid) { return valid ? u32(x) * u32(sizeof(B)) : kMaskedOut; }
+    FKD_DEV static u32 row_offset(int y, const PlaneRef& r) { return u32(y) * r.pitch; }
+    FKD_DEV static void put_masked(const PlaneRef& r, u32 row_off, u32 lane_off, const T& v) {
+        constexpr int kThrough = 1 | 16;     // sc0 sc1: written through the L2, as gstore_through
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<0>(v)), r.rsrc, lane_off, row_off, kThrough);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<1>(v)), r.rsrc, lane_off, row_off + r.chan_bytes, kThrough);
+        if constexpr (cn_v<T> > 2) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<2>(v)), r.rsrc, lane_off, row_off + 2u * r.chan_bytes, kThrough);
+        if constexpr (cn_v<T> > 3) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<3>(v)), r.rsrc, lane_off, row_off + 3u * r.chan_bytes, kThrough);
+    }
     struct RowRef { B* p; size_t px; };
     FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), size_t(p.width) * p.height}; }
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
