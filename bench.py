@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--list-compiled", action="store_true",
                     help="print to stderr the kernel symbol and signature of every chain compiled at run time")
+    ap.add_argument("--issue-rate", action="store_true",
+                    help="run the stand-alone instruction-issue measurement (fusedkernellibrary_amd/probe_issue_rate) and exit")
     ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
@@ -71,6 +73,13 @@ class Timer:
 
 def main():
     args = parse()
+    if args.issue_rate:
+        import subprocess
+        probe = os.path.join(ROOT, "fusedkernellibrary_amd", "probe_issue_rate")
+        if not os.path.exists(probe):
+            print(f"bench.py: {probe} is missing: build it with `python -m fusedkernellibrary_amd.build`", file=sys.stderr)
+            sys.exit(1)
+        sys.exit(subprocess.run([probe]).returncode)
     if args.gpus != 1:
         print(f"bench.py: this path runs on ONE GPU (asked for {args.gpus}); every output pixel is independent, "
               "so more GPUs would only split the batch. Run with --gpus 1.", file=sys.stderr)
@@ -80,7 +89,8 @@ def main():
     import torch
 
     import fusedkernellibrary_amd as fkl
-    from fusedkernellibrary_amd import cases, workloads as wl
+    import fkl_cases as cases
+    import workloads as wl
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)

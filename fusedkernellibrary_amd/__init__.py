@@ -2,7 +2,7 @@
 
 The product is native: `libfklhip.so` (C ABI declared in include/fklhip.h, hand-written HIP kernels) and the
 C++20 host headers under include/fused_kernel/.  This Python package only locates and loads the library for
-tests and benchmarks, and defines the synthetic workloads.  There is no CPU fallback: if the library is missing
+tests and benchmarks (their case drivers and synthetic workloads live under tests/).  There is no CPU fallback: if the library is missing
 or cannot be loaded, importing `lib()` raises.
 """
 from __future__ import annotations

@@ -607,11 +607,11 @@ struct JitMeta {
     u32 params_bytes;    // sizeof(Chain::Params)
     u32 v, rows;         // rows kernel: elements per thread along x, rows per thread
     u32 xi, yi, by;      // gather kernel: pixels per lane along x, rows per wave, waves per workgroup
-    u32 reserved;
+    u32 max_planes;      // most planes (grid z) a launch may have, 0: no limit of the kernel's own
 };
 template <class Chain> constexpr JitMeta jit_meta() {
     if constexpr (IsDivergent<Chain>::value)
-        return JitMeta{0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V), u32(RowsConfig<Chain>::ROWS), 0u, 0u, 0u, 0u};
+        return JitMeta{0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V), u32(RowsConfig<Chain>::ROWS), 0u, 0u, 0u, u32(Chain::kMaxPlanes)};
     else
         return JitMeta{is_gather_chain<Chain>() ? 1u : 0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V),
                        u32(RowsConfig<Chain>::ROWS), u32(FKD_GATHER_XI), u32(FKD_GATHER_YI), u32(kGatherBY), 0u};

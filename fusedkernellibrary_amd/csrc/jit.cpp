@@ -20,9 +20,11 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <fcntl.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/stat.h>
 #include <unistd.h>
 
 #include <mutex>
@@ -35,7 +37,7 @@ namespace {
 
 // Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): eight and four 32-bit words.
 struct JitMeta {
-    unsigned gather, params_bytes, v, rows, xi, yi, by, reserved;
+    unsigned gather, params_bytes, v, rows, xi, yi, by, max_planes;
 };
 struct TileGeom {
     unsigned tiles_x, tiles_y, n_tiles, tiles_x_magic;
@@ -115,28 +117,51 @@ std::string kernel_symbol(const std::string& signature) {
     snprintf(name, sizeof(name), "fkd_jit_%016llx", fnv1a(14695981039346656037ull, signature));
     return name;
 }
+// A cache file is a 24-byte header (magic, payload length, FNV-1a of the payload) followed by the code object: a file
+// that was cut short, damaged or put there by something else fails the check and is recompiled, instead of being handed
+// to the module loader, which takes a bare pointer and would run whatever loads.
+constexpr char kCacheMagic[8] = {'F', 'K', 'L', 'H', 'I', 'P', 'C', '1'};
+struct CacheHeader { char magic[8]; unsigned long long bytes, hash; };
+
 bool read_file(const std::string& path, std::vector<char>* out) {
-    FILE* f = fopen(path.c_str(), "rb");
-    if (!f) return false;
+    const int fd = open(path.c_str(), O_RDONLY | O_NOFOLLOW | O_CLOEXEC);
+    if (fd < 0) return false;
     bool ok = false;
-    if (fseek(f, 0, SEEK_END) == 0) {
-        const long n = ftell(f);
-        if (n > 0 && fseek(f, 0, SEEK_SET) == 0) {
-            out->resize(size_t(n));
-            ok = fread(out->data(), 1, size_t(n), f) == size_t(n);
+    struct stat st;
+    CacheHeader h;
+    if (fstat(fd, &st) == 0 && S_ISREG(st.st_mode) && size_t(st.st_size) > sizeof(h) &&
+        read(fd, &h, sizeof(h)) == ssize_t(sizeof(h)) && memcmp(h.magic, kCacheMagic, sizeof(kCacheMagic)) == 0 &&
+        h.bytes == size_t(st.st_size) - sizeof(h)) {
+        out->resize(size_t(h.bytes));
+        size_t got = 0;
+        while (got < out->size()) {
+            const ssize_t n = read(fd, out->data() + got, out->size() - got);
+            if (n <= 0) break;
+            got += size_t(n);
         }
+        ok = got == out->size() && fnv1a(14695981039346656037ull, out->data(), out->size()) == h.hash;
     }
-    fclose(f);
+    close(fd);
+    if (!ok) out->clear();
     return ok;
 }
-// Written under a private name and renamed into place, so a reader never sees half a file; failures are silent
-// (the cache is an optimisation).
+// Written under a private name (created exclusively, owner-only, never through a symbolic link) and renamed into
+// place, so a reader never sees half a file; failures are silent (the cache is an optimisation).
 void write_file(const std::string& path, const std::vector<char>& data) {
     const std::string tmp = path + ".tmp" + std::to_string(long(getpid()));
-    FILE* f = fopen(tmp.c_str(), "wb");
-    if (!f) return;
-    const bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
-    if (fclose(f) != 0 || !ok || rename(tmp.c_str(), path.c_str()) != 0) remove(tmp.c_str());
+    const int fd = open(tmp.c_str(), O_WRONLY | O_CREAT | O_EXCL | O_NOFOLLOW | O_CLOEXEC, 0600);
+    if (fd < 0) return;
+    CacheHeader h;
+    memcpy(h.magic, kCacheMagic, sizeof(kCacheMagic));
+    h.bytes = data.size();
+    h.hash = fnv1a(14695981039346656037ull, data.data(), data.size());
+    bool ok = write(fd, &h, sizeof(h)) == ssize_t(sizeof(h));
+    size_t put = 0;
+    while (ok && put < data.size()) {
+        const ssize_t n = write(fd, data.data() + put, data.size() - put);
+        if (n <= 0) ok = false; else put += size_t(n);
+    }
+    if (close(fd) != 0 || !ok || rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());
 }
 
 int get_function(JitKernel* k, hipFunction_t* fn) {
@@ -182,6 +207,7 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
     if (info) *info = fkd::LaunchInfo{m.gather ? "gather_jit" : "rows_jit", {grid[0], grid[1], grid[2]}, {block[0], block[1], 1}, 0};
     if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return FKLHIP_OK;
     if (grid[1] > 65535u || grid[2] > 65535u) return int(hipErrorInvalidConfiguration);
+    if (m.max_planes != 0 && grid[2] > m.max_planes) return int(hipErrorInvalidConfiguration);   // as launch_divergent
     hipFunction_t fn = nullptr;
     const int rc = get_function(k, &fn);
     if (rc != FKLHIP_OK) return rc;
@@ -263,8 +289,25 @@ static int build_and_register(const char* signature, bool may_read_cache) {
         g_log = std::string("loading the compiled chain failed: ") + hipGetErrorString(e);
         return int(e);
     }
-    if (from_cache) g_log = "loaded from " + cached;
-    else if (!cached.empty()) write_file(cached, k->code);
+    // The ahead-of-time build refuses kernels that need scratch memory (a private array the optimiser could not keep in
+    // registers, or spills: a silent slowdown of an order of magnitude).  A chain compiled here still runs, the note goes
+    // into the log; with FKLHIP_JIT_STRICT=1 it is refused like there.
+    int scratch_bytes = 0;
+    if (hipFuncGetAttribute(&scratch_bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, fn) != hipSuccess) scratch_bytes = 0;
+    if (scratch_bytes > 0) {
+        const char* strict = getenv("FKLHIP_JIT_STRICT");
+        const std::string note = "the compiled chain needs " + std::to_string(scratch_bytes) + " bytes of scratch memory per lane";
+        if (strict && strict[0] == '1') {
+            hipModuleUnload(mod);
+            delete k;
+            g_log = note + " (refused: FKLHIP_JIT_STRICT=1)";
+            return FKLHIP_EUNKNOWN_SIGNATURE;
+        }
+        g_log = note;
+    } else if (from_cache) {
+        g_log = "loaded from " + cached;
+    }
+    if (!from_cache && !cached.empty()) write_file(cached, k->code);
     int dev = 0;
     hipGetDevice(&dev);
     k->per_device.emplace(dev, fn);

@@ -1074,7 +1074,7 @@ FKD_DEV auto fold_static(const V& v, const Tup<typename Op::Params, typename Res
     if constexpr (sizeof...(Rest) == 0) return step();
     else return fold_static<Rest...>(step(), p.tail);
 }
-FKD_DEV inline bool all_static(const Tup<>&) { return true; }
+FKD_DEV bool all_static(const Tup<>&) { return true; }
 template <class Op, class... Rest>
 FKD_DEV bool all_static_of(const Tup<typename Op::Params, typename Rest::Params...>& p) {
     bool here = true;

@@ -10,7 +10,7 @@ import os
 
 import numpy as np
 
-from . import ROOT_DIR, lib
+from fusedkernellibrary_amd import ROOT_DIR, lib
 
 CASES_SO = os.path.join(ROOT_DIR, "tests", "cases", "libfkl_cases.so")
 _cases = None

@@ -20,7 +20,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 import oracle_lib as ol  # noqa: E402
-from fusedkernellibrary_amd import workloads as wl  # noqa: E402
+import workloads as wl  # noqa: E402
 
 
 def sha(a) -> str:

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
-from fusedkernellibrary_amd import cases
+import fkl_cases as cases
 
 pytestmark = pytest.mark.gpu
 TYPES = [ol.BORDER_CONSTANT, ol.BORDER_REPLICATE, ol.BORDER_REFLECT, ol.BORDER_WRAP, ol.BORDER_REFLECT_101]

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
-from fusedkernellibrary_amd import cases
+import fkl_cases as cases
 
 pytestmark = pytest.mark.gpu
 

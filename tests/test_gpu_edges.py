@@ -5,7 +5,9 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
-from fusedkernellibrary_amd import cases, last_launch, workloads as wl
+from fusedkernellibrary_amd import last_launch
+import fkl_cases as cases
+import workloads as wl
 
 pytestmark = pytest.mark.gpu
 

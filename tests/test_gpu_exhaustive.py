@@ -9,7 +9,8 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
-from fusedkernellibrary_amd import cases, workloads as wl
+import fkl_cases as cases
+import workloads as wl
 
 pytestmark = pytest.mark.gpu
 

@@ -4,7 +4,7 @@ values are closed forms: N float additions of `add` starting from `init`, each r
 import numpy as np
 import pytest
 
-from fusedkernellibrary_amd import cases
+import fkl_cases as cases
 
 pytestmark = pytest.mark.gpu
 

@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
-from fusedkernellibrary_amd import cases, last_launch
+from fusedkernellibrary_amd import last_launch
+import fkl_cases as cases
 
 pytestmark = pytest.mark.gpu
 
