@@ -47,11 +47,46 @@ template <class R> constexpr bool bounded_out() {
 template <class T> constexpr bool small_integer_base() {
     return !(__is_same(base_t<T>, f32) || __is_same(base_t<T>, f64)) && sizeof(base_t<T>) <= 2;
 }
+// Type classes without the standard library (run-time compilation has no headers) and without compiler-specific builtins.
+template <class T> constexpr bool is_float_v = __is_same(T, f32) || __is_same(T, f64);
+template <class T> constexpr bool is_integer_v =
+    __is_same(T, bool) || __is_same(T, char) || __is_same(T, signed char) || __is_same(T, unsigned char) || __is_same(T, short) ||
+    __is_same(T, unsigned short) || __is_same(T, int) || __is_same(T, unsigned int) || __is_same(T, long) ||
+    __is_same(T, unsigned long) || __is_same(T, long long) || __is_same(T, unsigned long long);
 template <int I, class T, class... Ts> struct TypeAt { using type = typename TypeAt<I - 1, Ts...>::type; };
 template <class T, class... Ts> struct TypeAt<0, T, Ts...> { using type = T; };
 
+// FKD_EXEC_CODE: the element-wise bodies of the operations (exec, width, height) are compiled: always in device code, and
+// in host code that defines FKD_HOST_EXEC (the host headers' CPU executor, which runs a chain element by element with
+// exactly these bodies).  Everything that moves runs of elements, gathers taps or uses a gfx950 instruction stays under
+// FKD_DEVICE_CODE.
+#if defined(FKD_DEVICE_CODE) || defined(FKD_HOST_EXEC)
+#define FKD_EXEC_CODE 1
+#endif
+
+#if defined(FKD_HOST_EXEC) && !defined(FKD_DEVICE_CODE)
+namespace detail {
+#define FKD_GLOBAL
+template <class T> inline const T* gconst(const void* p) { return static_cast<const T*>(p); }
+template <class T> inline T* gmut(void* p) { return static_cast<T*>(p); }
+template <class T> inline T load_elem(const T* p) { return *p; }
+template <class T> inline void store_elem(T* p, const T& v) { *p = v; }
+template <class T> inline const T* row_ptr(const T* data, u32 pitch, int x, int y) {
+    return reinterpret_cast<const T*>(reinterpret_cast<const char*>(data) + size_t(y) * pitch) + x;
+}
+template <class T> inline T* row_ptr(T* data, u32 pitch, int x, int y) {
+    return reinterpret_cast<T*>(reinterpret_cast<char*>(data) + size_t(y) * pitch) + x;
+}
+inline bool dword_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+inline bool none_in_wave(bool) { return false; }     // never reached: host code has no paired-tap paths
+} // namespace detail
+#endif
+
 #if defined(FKD_DEVICE_CODE)
 namespace detail {
+
+// True when no lane of the wave holds `flag`.
+FKD_DEV bool none_in_wave(bool flag) { return __builtin_amdgcn_ballot_w64(flag) == 0; }
 
 // Every pointer this library dereferences on the device is device (global) memory.  Saying so at the access keeps
 // the accesses global_load/global_store (scalar base + lane offset addressing, vmcnt only) even where the pointer
@@ -819,7 +854,7 @@ template <class T, int I0, int I1, int I2 = 2, int I3 = 3> struct Reorder {
 template <class I, class O> struct SaturateCast {
     using In = I; using Out = O; using Params = Empty;
     FKD_NAME("SaturateCast<" + type_name<I>() + "," + type_name<O>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     template <class D> struct Lim {
         static constexpr bool is_signed = D(-1) < D(0);
         static constexpr long long hi = is_signed ? (long long)((1ull << (8 * sizeof(D) - 1)) - 1)
@@ -829,11 +864,13 @@ template <class I, class O> struct SaturateCast {
     template <class S, class D> FKD_DEV static D sat(S s) {
         if constexpr (__is_same(S, D)) {
             return s;
+#if defined(FKD_DEVICE_CODE)
         } else if constexpr (__is_same(S, f32) && __is_same(D, u8)) {
             // v_cvt_pk_u8_f32: round half to even, clamp to [0, 255], NaN -> 0 in one instruction.  Checked against
             // the reference rule for all 2^32 float bit patterns (tests/test_gpu_exhaustive.py).
             return u8(__builtin_amdgcn_cvt_pk_u8_f32(s, 0u, 0u));
-        } else if constexpr (__is_floating_point(S) && __is_integral(D)) {
+#endif
+        } else if constexpr (is_float_v<S> && is_integer_v<D>) {
             // Branch free.  Round half to even under the default rounding mode (v_rndne_f32 / v_rndne_f64), then
             // clamp: fmax/fmin return the non-NaN operand, so NaN leaves the clamp as lo; for destination types whose
             // bounds are exact in S (8/16-bit) the clamp alone is the saturation.
@@ -850,7 +887,7 @@ template <class I, class O> struct SaturateCast {
                 const D v = static_cast<D>(safe);
                 return nan ? D(0) : (over ? D(Lim<D>::hi) : (under ? D(Lim<D>::lo) : v));
             }
-        } else if constexpr (__is_integral(S) && __is_integral(D)) {
+        } else if constexpr (is_integer_v<S> && is_integer_v<D>) {
             const long long v = (long long)s;
             return v > Lim<D>::hi ? D(Lim<D>::hi) : (v < Lim<D>::lo ? D(Lim<D>::lo) : D(s));
         } else {
@@ -859,7 +896,7 @@ template <class I, class O> struct SaturateCast {
     }
 #endif
     FKD_DEV static O exec(const I& a, const Params&) {
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
         return map1<O>(a, [](auto x) { return sat<decltype(x), base_t<O>>(x); });
 #else
         (void)a; return O{};
@@ -1039,7 +1076,7 @@ template <class In, class Op, class... Rest> struct FoldOut<In, Op, Rest...> {
     using type = typename FoldOut<typename Op::Out, Rest...>::type;
     using first_in = typename Op::In;
 };
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
 template <class V> FKD_DEV V fold(const V& v, const Tup<>&) { return v; }
 template <class Op, class... Rest, class V>
 FKD_DEV auto fold(const V& v, const Tup<typename Op::Params, typename Rest::Params...>& p) {
@@ -1047,6 +1084,8 @@ FKD_DEV auto fold(const V& v, const Tup<typename Op::Params, typename Rest::Para
     if constexpr (sizeof...(Rest) == 0) return Op::exec(v, p.head);
     else return fold<Rest...>(Op::exec(v, p.head), p.tail);
 }
+#endif
+#if defined(FKD_DEVICE_CODE)
 
 // The same fold through each operation's straight-line variant where it has one (see Div).  `ok` comes back false
 // when some operation could not vouch for its quick result; the value must then be recomputed with fold().
@@ -1172,7 +1211,7 @@ template <class... Ops> struct FusedCompute {
     using Out = typename FoldOut<In, Ops...>::type;
     using Params = Tup<typename Ops::Params...>;
     FKD_NAME("FusedCompute<" + OpList<Ops...>::names().substr(1) + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static Out exec(const In& a, const Params& p) { return fold<Ops...>(a, p); }
 #endif
 };
@@ -1189,12 +1228,14 @@ template <class T> struct Read2D {
     static constexpr bool kFiniteTaps = !(__is_same(base_t<T>, f32) || __is_same(base_t<T>, f64));
     static constexpr bool kBoundedOut = small_integer_base<T>();
     FKD_NAME("Read2D<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static T exec(int x, int y, int, const Params& p) {
         return detail::load_elem(detail::row_ptr(p.data, p.pitch, x, y));
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<T> (&out)[V]) {
         detail::load_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), out);
     }
@@ -1257,7 +1298,7 @@ template <class T> struct Read3D {
     static constexpr bool kTapCursor = false;
     static constexpr bool kBoundedOut = small_integer_base<T>();
     FKD_NAME("Read3D<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static const T* plane(const Params& p, int z) {
@@ -1266,6 +1307,8 @@ template <class T> struct Read3D {
     FKD_DEV static T exec(int x, int y, int z, const Params& p) {
         return detail::load_elem(detail::row_ptr(plane(p, z), p.pitch, x, y));
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
         detail::load_run<T, V, A>(detail::row_ptr(plane(p, z), p.pitch, x, y), out);
     }
@@ -1285,7 +1328,7 @@ template <class T> struct TensorPack {
     using Params = RawPtr3D<const B>;
     static constexpr bool kTapCursor = false;
     FKD_NAME("TensorPack<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static const B* at(const Params& p, int x, int y, int z) {
@@ -1302,6 +1345,8 @@ template <class T> struct TensorPack {
         if constexpr (cn_v<T> > 3) chan<3>(o) = g[3 * px];
         return o;
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
         const B* r = at(p, x, y, z);
         const size_t px = size_t(p.width) * p.height;
@@ -1343,10 +1388,12 @@ template <int DIR, int BATCH, class Back> struct CircularRead {
     struct Params { i32 first; typename Back::Params back; };
     static constexpr bool kTapCursor = false;
     FKD_NAME("CircularRead<" + istr(DIR) + "," + istr(BATCH) + "," + Back::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return Back::exec(x, y, circular_plane<DIR, BATCH>(z, p.first), p.back); }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         Back::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), p.back, out);
     }
@@ -1365,13 +1412,15 @@ template <int DIR, int BATCH, class PlaneOp> struct CircularBatchRead {
     struct Params { i32 first; typename PlaneOp::Params plane[BATCH]; };
     static constexpr bool kTapCursor = false;
     FKD_NAME("CircularBatchRead<" + istr(DIR) + "," + istr(BATCH) + "," + PlaneOp::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return PlaneOp::width(p.plane[0]); }
     FKD_DEV static int height(const Params& p) { return PlaneOp::height(p.plane[0]); }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         return PlaneOp::exec(x, y, c, p.plane[c]);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         PlaneOp::template exec_row<V, A>(x, y, c, p.plane[c], out);
@@ -1396,7 +1445,7 @@ template <bool VU> struct ReadNV {
     static constexpr bool kFiniteTaps = true;
     static constexpr bool kBoundedOut = true;
     FKD_NAME(VU ? "ReadNV21" : "ReadNV12")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) {
@@ -1407,6 +1456,8 @@ template <bool VU> struct ReadNV {
         o.z = c[VU ? 0 : 1];
         return o;
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
@@ -1491,7 +1542,7 @@ template <int PF> struct ReadYUV {
     using Params = RawYUV;
     static constexpr bool kTapCursor = false;
     FKD_NAME("ReadYUV<" + istr(PF) + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) {
@@ -1511,6 +1562,8 @@ template <int PF> struct ReadYUV {
         }
         return o;
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
@@ -1527,34 +1580,54 @@ template <int PF> struct ReadYUV {
 
 // Crop<BackIOp>: FK/algorithms/image_processing/crop.h:36-39.  Shifts by the rectangle origin, drops z,
 // clips nothing.
+// The tap interface of a read that wraps another one: the inner read's, or placeholders when the inner read has none
+// (a bilinear resize, a warp: their elements are computed, not fetched), so that the wrapper's declarations still name
+// types; nothing calls them then, because kTapCursor is false.
+namespace detail {
+template <class B> constexpr bool has_tap_types() {
+    if constexpr (requires { typename B::TapRow; typename B::Raw; }) return true; else return false;
+}
+struct NoTapRaw {}; struct NoTapRow {}; struct NoTapBits {}; struct NoPairBits {};
+template <class B, bool = has_tap_types<B>()> struct TapTypesOf {
+    using Raw = typename B::Raw; using TapRow = typename B::TapRow; using TapBits = typename B::TapBits; using PairBits = typename B::PairBits;
+    static constexpr bool kTapOverread = B::kTapOverread, kTapPair = B::kTapPair;
+};
+template <class B> struct TapTypesOf<B, false> {
+    using Raw = NoTapRaw; using TapRow = NoTapRow; using TapBits = NoTapBits; using PairBits = NoPairBits;
+    static constexpr bool kTapOverread = false, kTapPair = false;
+};
+} // namespace detail
+
 template <class Back> struct Crop {
     using Out = typename Back::Out;
     struct Params { i32 x, y, w, h; typename Back::Params back; };
     static constexpr bool kTapCursor = Back::kTapCursor;
     static constexpr bool kBoundedOut = bounded_out<Back>();
     FKD_NAME("Crop<" + Back::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     static constexpr bool kFiniteTaps = finite_taps<Back>();
     FKD_DEV static int width(const Params& p) { return p.w; }
     FKD_DEV static int height(const Params& p) { return p.h; }
     FKD_DEV static Out exec(int x, int y, int, const Params& p) { return Back::exec(x + p.x, y + p.y, 0, p.back); }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Params& p, Slot<Out> (&out)[V]) {
         Back::template exec_row<V, A>(x + p.x, y + p.y, 0, p.back, out);
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff + p.x); }
-    using Raw = typename Back::Raw;
+    using Raw = typename detail::TapTypesOf<Back>::Raw;
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return Back::finish(r, p.back); }
-    static constexpr bool kTapOverread = Back::kTapOverread;
-    using TapRow = typename Back::TapRow;
+    static constexpr bool kTapOverread = detail::TapTypesOf<Back>::kTapOverread;
+    using TapRow = typename detail::TapTypesOf<Back>::TapRow;
     FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) { return Back::tap_row(x0 + p.x, y + p.y, 0, p.back); }
     FKD_DEV static bool tap_last(const TapRow& r) { return Back::tap_last(r); }
-    using TapBits = typename Back::TapBits;
+    using TapBits = typename detail::TapTypesOf<Back>::TapBits;
     template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params& p) {
         return Back::template tap_load<OVER>(r, x, p.back);
     }
     FKD_DEV static Raw tap_value(const TapBits& b) { return Back::tap_value(b); }
-    static constexpr bool kTapPair = Back::kTapPair;
-    using PairBits = typename Back::PairBits;
+    static constexpr bool kTapPair = detail::TapTypesOf<Back>::kTapPair;
+    using PairBits = typename detail::TapTypesOf<Back>::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
     static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
@@ -1589,7 +1662,7 @@ template <int BT, class Back> struct Border {
     struct Params { Out value; typename Back::Params back; };     // value: CONSTANT only
     static constexpr bool kTapCursor = false;
     FKD_NAME("Border<" + istr(BT) + "," + Back::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static int iabs(int v) { return v < 0 ? -v : v; }
@@ -1636,6 +1709,8 @@ template <int BT, class Back> struct Border {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
     using Raw = Out;
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
@@ -1652,13 +1727,15 @@ template <class Back, class... Ops> struct FusedRead {
     static constexpr bool kTapCursor = Back::kTapCursor;
     static constexpr bool kBoundedOut = bounded_out<Back>() && (finite_map<Ops>() && ...);
     FKD_NAME("FusedRead<" + Back::name() + OpList<Ops...>::names() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     static constexpr bool kFiniteTaps = finite_taps<Back>() && (finite_map<Ops>() && ...);
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
         return fold<Ops...>(Back::exec(x, y, z, p.back), p.ops);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         Slot<typename Back::Out> t[V];
         Back::template exec_row<V, A>(x, y, z, p.back, t);
@@ -1666,19 +1743,19 @@ template <class Back, class... Ops> struct FusedRead {
         for (int i = 0; i < V; ++i) out[i].v = fold<Ops...>(t[i].v, p.ops);
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) { return Back::rows_aligned(p.back, xoff); }
-    using Raw = typename Back::Raw;
+    using Raw = typename detail::TapTypesOf<Back>::Raw;
     FKD_DEV static Out finish(const Raw& r, const Params& p) { return fold<Ops...>(Back::finish(r, p.back), p.ops); }
-    static constexpr bool kTapOverread = Back::kTapOverread;
-    using TapRow = typename Back::TapRow;
+    static constexpr bool kTapOverread = detail::TapTypesOf<Back>::kTapOverread;
+    using TapRow = typename detail::TapTypesOf<Back>::TapRow;
     FKD_DEV static TapRow tap_row(int x0, int y, int z, const Params& p) { return Back::tap_row(x0, y, z, p.back); }
     FKD_DEV static bool tap_last(const TapRow& r) { return Back::tap_last(r); }
-    using TapBits = typename Back::TapBits;
+    using TapBits = typename detail::TapTypesOf<Back>::TapBits;
     template <bool OVER> FKD_DEV static TapBits tap_load(const TapRow& r, int x, const Params& p) {
         return Back::template tap_load<OVER>(r, x, p.back);
     }
     FKD_DEV static Raw tap_value(const TapBits& b) { return Back::tap_value(b); }
-    static constexpr bool kTapPair = Back::kTapPair;
-    using PairBits = typename Back::PairBits;
+    static constexpr bool kTapPair = detail::TapTypesOf<Back>::kTapPair;
+    using PairBits = typename detail::TapTypesOf<Back>::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
     static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
@@ -1729,7 +1806,7 @@ template <int AR, class Back> struct ResizeLinear {
     static constexpr bool kBoundedOut = AR == IGNORE_AR && bounded_out<Back>();   // a letterbox colour is a run-time value
     using BackOp = Back;
     FKD_NAME("ResizeLinear<" + istr(AR) + "," + Back::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return p.dst_w; }
     FKD_DEV static int height(const Params& p) { return p.dst_h; }
 
@@ -1783,7 +1860,7 @@ template <int AR, class Back> struct ResizeLinear {
             const int y2 = y1 + 1 < sh - 1 ? y1 + 1 : sh - 1;
             const auto ra = Back::tap_row(0, y1, z, p.back), rb = Back::tap_row(0, y2, z, p.back);
             const bool risky = sw < 2 || Back::tap_last(ra) || Back::tap_last(rb);
-            if (__builtin_amdgcn_ballot_w64(risky) == 0) {
+            if (detail::none_in_wave(risky)) {
                 const bool edge = x1 >= sw - 1;           // x1 + 1 is past the line: both taps are the last pixel
                 const int xp = edge ? sw - 2 : x1;
                 const auto wa = Back::pair_load(ra, xp, p.back), wb = Back::pair_load(rb, xp, p.back);
@@ -1804,6 +1881,8 @@ template <int AR, class Back> struct ResizeLinear {
         const Src d = Back::exec(t.x2r, t.y2r, z, p.back);
         return blend(a, b, c, d, t);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
@@ -1822,7 +1901,7 @@ template <int DT, class Back> struct Deinterlace {
     struct Params { i32 use_even; typename Back::Params back; };
     static constexpr bool kTapCursor = false;
     FKD_NAME("Deinterlace<" + istr(DT) + "," + Back::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     // which lines take part for output line y: first, second, and whether they are averaged
@@ -1848,6 +1927,8 @@ template <int DT, class Back> struct Deinterlace {
         lines(y, p, ya, yb, average);
         return mix(Back::exec(x, ya, z, p.back), Back::exec(x, yb, z, p.back), average);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         int ya, yb; bool average;
         lines(y, p, ya, yb, average);
@@ -1880,7 +1961,7 @@ template <int WT, class Back> struct Warp {
         if constexpr (requires { Back::kTapPair; }) return Back::kTapCursor && Back::kTapPair; else return false;
     }();
     FKD_NAME("Warp<" + istr(WT) + "," + Back::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return p.dst_w; }
     FKD_DEV static int height(const Params& p) { return p.dst_h; }
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
@@ -1905,7 +1986,7 @@ template <int WT, class Back> struct Warp {
             const int y2r = y1 + 1 < sh - 1 ? y1 + 1 : sh - 1;
             const auto ra = Back::tap_row(0, y1, z, p.back), rb = Back::tap_row(0, y2r, z, p.back);
             const bool risky = sw < 2 || Back::tap_last(ra) || Back::tap_last(rb);
-            if (__builtin_amdgcn_ballot_w64(risky) == 0) {
+            if (detail::none_in_wave(risky)) {
                 const bool edge = x1 >= sw - 1;           // x1 + 1 is past the line: both taps are the last pixel
                 const int xp = edge ? sw - 2 : x1;
                 const auto wa = Back::pair_load(ra, xp, p.back), wb = Back::pair_load(rb, xp, p.back);
@@ -1951,6 +2032,8 @@ template <int WT, class Back> struct Warp {
         }
         return o;
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
@@ -1969,8 +2052,10 @@ template <int N, class PlaneOp> struct BatchRead {
     static constexpr bool kTapCursor = false;
     static constexpr bool kBoundedOut = bounded_out<PlaneOp>();
     FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         PlaneOp::template exec_row<V, A>(x, y, z, p.plane[z], out);
     }
@@ -1990,11 +2075,13 @@ template <int N, class PlaneOp> struct BatchReadDefault {
     struct Params { typename PlaneOp::Params plane[N]; i32 used; Out def; };
     static constexpr bool kTapCursor = false;
     FKD_NAME("BatchReadDefault<" + istr(N) + "," + PlaneOp::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) {
         if (p.used <= z) return p.def;
         return PlaneOp::exec(x, y, z, p.plane[z]);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
         if (p.used <= z) {
 #pragma unroll
@@ -2019,10 +2106,12 @@ template <class T> struct ReadSet {
     struct Params { T value; u32 width, height, planes; };
     static constexpr bool kTapCursor = false;
     FKD_NAME("ReadSet<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static T exec(int, int, int, const Params& p) { return p.value; }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int, int, int, const Params& p, Slot<T> (&out)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = p.value;
@@ -2040,10 +2129,12 @@ template <class T> struct Write2D {
     using In = T;
     using Params = RawPtr2D<T>;
     FKD_NAME("Write2D<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static void exec(int x, int y, int, const T& v, const Params& p) {
         detail::store_elem(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Slot<T> (&v)[V], const Params& p) {
         detail::store_run<T, V, A>(detail::row_ptr(p.data, p.pitch, x, y), v);
     }
@@ -2070,13 +2161,15 @@ template <class T> struct TensorWrite {
     using In = T;
     using Params = RawPtr3D<T>;
     FKD_NAME("TensorWrite<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static T* plane(const Params& p, int z) {
         return reinterpret_cast<T*>(reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z);
     }
     FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
         detail::store_elem(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         detail::store_run<T, V, A>(detail::row_ptr(plane(p, z), p.pitch, x, y), v);
     }
@@ -2104,7 +2197,7 @@ template <class T> struct TensorSplit {
     using B = base_t<T>;
     using Params = RawPtr3D<B>;
     FKD_NAME("TensorSplit<" + type_name<T>() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static B* at(const Params& p, int x, int y, int z) {
         return reinterpret_cast<B*>(reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z +
                                     size_t(y) * p.pitch) + x;
@@ -2118,6 +2211,8 @@ template <class T> struct TensorSplit {
         if constexpr (cn_v<T> > 2) gw[2 * px] = chan<2>(v);
         if constexpr (cn_v<T> > 3) gw[3 * px] = chan<3>(v);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         B* w = at(p, x, y, z);
         const size_t px = size_t(p.width) * p.height;
@@ -2220,7 +2315,7 @@ template <int PF> struct WriteYUV {
     using In = Vec<B, 3>;
     using Params = RawYUVOut;
     FKD_NAME("WriteYUV<" + istr(PF) + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     struct RowRef { char* row; char* crow; bool chroma_row; int last_x; };
     FKD_DEV static RowRef row(int y, int, const Params& p) {
         RowRef r;
@@ -2252,11 +2347,13 @@ template <int PF> struct WriteYUV {
             }
         }
     }
+    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { put(row(y, z, p), x, v); }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<In> (&v)[V]) {
 #pragma unroll
         for (int i = 0; i < V; ++i) put(r, x + i, v[i].v);
     }
-    FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { put(row(y, z, p), x, v); }
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         put_run<V>(row(y, z, p), x, v);
     }
@@ -2271,8 +2368,10 @@ template <int N, class W> struct BatchWrite {
     using In = typename W::In;
     struct Params { typename W::Params plane[N]; };
     FKD_NAME("BatchWrite<" + istr(N) + "," + W::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, z, v, p.plane[z]); }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         W::template exec_row<V, A>(x, y, z, v, p.plane[z]);
     }
@@ -2295,8 +2394,10 @@ template <int DIR, int BATCH, class W> struct CircularWrite {
     using In = typename W::In;
     struct Params { i32 first; typename W::Params w; };
     FKD_NAME("CircularWrite<" + istr(DIR) + "," + istr(BATCH) + "," + W::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) { W::exec(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w); }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         W::template exec_row<V, A>(x, y, circular_plane<DIR, BATCH>(z, p.first), v, p.w);
     }
@@ -2309,11 +2410,13 @@ template <int DIR, int BATCH, class W> struct CircularBatchWrite {
     using In = typename W::In;
     struct Params { i32 first; typename W::Params plane[BATCH]; };
     FKD_NAME("CircularBatchWrite<" + istr(DIR) + "," + istr(BATCH) + "," + W::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         W::exec(x, y, c, v, p.plane[c]);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         const int c = circular_plane<DIR, BATCH>(z, p.first);
         W::template exec_row<V, A>(x, y, c, v, p.plane[c]);
@@ -2333,11 +2436,13 @@ template <class W1, class W2> struct TeeWrite {
     using In = typename W2::In;
     struct Params { typename W1::Params first; typename W2::Params second; };
     FKD_NAME("TeeWrite<" + W1::name() + "," + W2::name() + ">")
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     FKD_DEV static void exec(int x, int y, int z, const In& v, const Params& p) {
         W1::exec(x, y, z, v, p.first);
         W2::exec(x, y, z, v, p.second);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
         W1::template exec_row<V, A>(x, y, z, v, p.first);
         W2::template exec_row<V, A>(x, y, z, v, p.second);
@@ -2405,11 +2510,13 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
     }
     static void finalize(Params& p) { finalize_from<0>(p); }
 #endif
-#if defined(FKD_DEVICE_CODE)
+#if defined(FKD_EXEC_CODE)
     static_assert(__is_same(Value, typename W::In), "the write operation does not take the type the chain produces");
     FKD_DEV static Value compute(const typename R::Out& v, const Params& p) {
         if constexpr (sizeof...(Ops) == 0) return v; else return fold<Ops...>(v, p.ops);
     }
+#endif
+#if defined(FKD_DEVICE_CODE)
     // compute() through the operations' straight-line variants, falling back to compute() for the (rare) elements
     // they cannot vouch for.  Same result as compute(), fewer instructions on the common path.
     static constexpr bool kQuick = any_quick<Ops...>();

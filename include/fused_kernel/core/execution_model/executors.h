@@ -1,4 +1,5 @@
 // Executor<TransformDPP<ParArch::GPU_AMD, TF>>: turns an argument list of IOps into one launch of a gfx950 kernel.
+// (Executor<TransformDPP<ParArch::CPU, TF>>, further down, runs the same lowered chain on the calling thread.)
 //
 //   1. BackFuser::fuse_back collapses the Read + ReadBack... prefix into one Read IOp (backwards vertical fusion).
 //   2. Every IOp is lowered to its device counterpart; together they spell the type fkd::Chain<Read, OpList<...>,
@@ -125,6 +126,41 @@ template <typename... IOps> struct LoweredSequence {
     typename Fused::Chain::Params params;
 };
 
+// ---- ParArch::CPU: the same lowered chain, run element by element on the calling thread ------------------------------
+// Reference loop: FK/core/execution_model/data_parallel_patterns.h:271-283 (one pass over z, y, x; synchronous).  The
+// element bodies are the device operations' own (fkd::...::exec, compiled for the host), so both architectures compute
+// every element with the same source code; with floating-point contraction off on the host (-ffp-contract=off, and no
+// -ffast-math) the results are the same bits.  Nothing on the GPU path ever comes here: the architecture is part of the
+// DPP's type, chosen by the caller.
+template <typename Chain> void run_plane_on_host(const typename Chain::Params& p, int z) {
+    const int w = int(p.active_w), h = int(p.active_h);
+    for (int y = 0; y < h; ++y)
+        for (int x = 0; x < w; ++x)
+            Chain::Write::exec(x, y, z, Chain::compute(Chain::Read::exec(x, y, z, p.read), p), p.write);
+}
+template <typename... IOps> void run_fused_on_host(const IOps&... iOps) {
+    using F = FusedChain<IOps...>;
+    const typename F::Chain::Params p = F::params(iOps...);
+    for (int z = 0; z < int(p.active_z); ++z) run_plane_on_host<typename F::Chain>(p, z);
+}
+template <size_t I, typename First, typename... Rest> void run_selected_on_host(size_t sel, int z, const First& first, const Rest&... rest) {
+    if (sel == I) run_plane_on_host<typename First::Fused::Chain>(first.params, z);
+    else if constexpr (sizeof...(Rest) > 0) run_selected_on_host<I + 1>(sel, z, rest...);
+}
+template <typename SequenceSelector, typename... Seqs> void run_divergent_on_host(const Seqs&... seqs) {
+    uint planes = 0;
+    ((planes += seqs.params.active_z), ...);
+    // plane z runs sequence SequenceSelector::at(z), with z handed on unchanged; a plane no sequence claims runs nothing
+    for (uint z = 0; z < planes; ++z) run_selected_on_host<0>(size_t(SequenceSelector::at(z)), int(z), seqs...);
+}
+
+template <typename... IOps> auto lower_sequence(const IOpSequence<IOps...>& seq) {
+    const auto fused = std::apply([](const auto&... iOps) { return BackFuser::fuse_back(iOps...); }, seq.iOps);
+    return std::apply([](const auto&... f) {
+        return LoweredSequence<std::decay_t<decltype(f)>...>{FusedChain<std::decay_t<decltype(f)>...>::params(f...)};
+    }, fused);
+}
+
 } // namespace amd
 
 template <typename Child> struct BaseExecutor {
@@ -163,8 +199,8 @@ template <typename Child> struct BaseExecutor {
 };
 
 template <typename DataParallelPattern> struct Executor {
-    static_assert(DataParallelPattern::PAR_ARCH == ParArch::GPU_AMD,
-                  "this build of the library provides the GPU_AMD (MI355X) backend only");
+    static_assert(DataParallelPattern::PAR_ARCH == ParArch::GPU_AMD || DataParallelPattern::PAR_ARCH == ParArch::CPU,
+                  "this build of the library provides the GPU_AMD (MI355X) and CPU architectures");
 };
 
 template <TF TFEN> struct Executor<TransformDPP<ParArch::GPU_AMD, TFEN, void>> : BaseExecutor<Executor<TransformDPP<ParArch::GPU_AMD, TFEN, void>>> {
@@ -179,6 +215,19 @@ private:
 };
 
 
+// TransformDPP<ParArch::CPU>: FK/core/execution_model/executors.h:163-189.  Synchronous; the stream is the reference's
+// no-op Stream_<ParArch::CPU>.  Thread fusion changes nothing here either.
+template <TF TFEN> struct Executor<TransformDPP<ParArch::CPU, TFEN, void>> : BaseExecutor<Executor<TransformDPP<ParArch::CPU, TFEN, void>>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::CPU; }
+
+private:
+    friend struct BaseExecutor<Executor<TransformDPP<ParArch::CPU, TFEN, void>>>;
+    template <typename... IOps> static void executeOperations_helper(Stream_<ParArch::CPU>&, const IOps&... iOps) {
+        amd::run_fused_on_host(iOps...);
+    }
+};
+
 // Executor of DivergentBatchTransformDPP: every sequence is back-fused like a TransformDPP chain, then all of them go
 // into one launch.  Interface counterpart: FK/core/execution_model/executors.h:360-411.
 template <typename SequenceSelector> struct Executor<DivergentBatchTransformDPP<ParArch::GPU_AMD, SequenceSelector>> {
@@ -190,11 +239,15 @@ template <typename SequenceSelector> struct Executor<DivergentBatchTransformDPP<
     }
 
 private:
-    template <typename... IOps> static auto lower(const IOpSequence<IOps...>& seq) {
-        const auto fused = std::apply([](const auto&... iOps) { return BackFuser::fuse_back(iOps...); }, seq.iOps);
-        return std::apply([](const auto&... f) {
-            return amd::LoweredSequence<std::decay_t<decltype(f)>...>{amd::FusedChain<std::decay_t<decltype(f)>...>::params(f...)};
-        }, fused);
+    template <typename... IOps> static auto lower(const IOpSequence<IOps...>& seq) { return amd::lower_sequence(seq); }
+};
+
+template <typename SequenceSelector> struct Executor<DivergentBatchTransformDPP<ParArch::CPU, SequenceSelector>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::CPU; }
+    template <typename... IOpSequenceTypes>
+    static void executeOperations(Stream_<ParArch::CPU>&, const IOpSequenceTypes&... iOpSequences) {
+        amd::run_divergent_on_host<SequenceSelector>(amd::lower_sequence(iOpSequences)...);
     }
 };
 

@@ -21,6 +21,11 @@
 #include <type_traits>
 #include <utility>
 
+// The element-wise bodies of the device operations are compiled for the host as well: they are what
+// Executor<TransformDPP<ParArch::CPU>> runs (core/execution_model/executors.h).
+#ifndef FKD_HOST_EXEC
+#define FKD_HOST_EXEC 1
+#endif
 #include <fkd/ops.hpp>
 
 #include <fused_kernel/core/utils/utils.h>

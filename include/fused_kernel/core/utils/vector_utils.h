@@ -59,11 +59,16 @@ template <int I, typename V> constexpr auto vectorAt(const V& v) {
     else return v.w;
 }
 
-// make_<float3>(a, b, c)
+// make_<float3>(a, b, c); fewer values than channels leave the remaining channels zero (aggregate initialisation, as
+// in the reference, FK/core/utils/vector_utils.h:251-277)
 template <typename V, typename... Args> constexpr V make_(const Args&... args) {
-    static_assert(sizeof...(Args) == cn<V>, "make_<V> needs exactly cn<V> values");
-    if constexpr (isVector<V>) return V{static_cast<VBase<V>>(args)...};
-    else return (static_cast<V>(args), ...);
+    if constexpr (isVector<V>) {
+        static_assert(sizeof...(Args) >= 1 && sizeof...(Args) <= cn<V>, "make_<V> takes at most cn<V> values");
+        return V{static_cast<VBase<V>>(args)...};
+    } else {
+        static_assert(sizeof...(Args) == 1, "passing more than one argument for a non vector type");
+        return (static_cast<V>(args), ...);
+    }
 }
 // make_set<float3>(v): every channel = v
 template <typename V, typename S> constexpr V make_set(const S& s) {

@@ -1,5 +1,9 @@
 // ref_chains.cpp -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
 //
+// (Compiled a second time with -DFKL_HARNESS_PUBLIC_API_ONLY against THIS repository's headers -- oracle/Makefile,
+// target hostexec -- the same chain text runs on this repository's own TransformDPP<ParArch::CPU> executor; tests then
+// hold that executor against the oracle.  The few probes of reference internals are left out of that build.)
+//
 // A thin C-ABI harness around the REFERENCE library's own CPU backend.  It is compiled against the
 // reference's headers where they lie on disk (see oracle/Makefile: -I$(FKL_REFERENCE)), never copied,
 // and the resulting shared object goes to oracle/_ref/ (git-ignored).  Each entry point spells one fused
@@ -307,6 +311,7 @@ int fklref_crop_swap_u8_b4(const uint8_t* src, int w, int h, int pitch, const in
     return crop_swap_u8<4>(src, w, h, pitch, rects, out);
 }
 
+#ifndef FKL_HARNESS_PUBLIC_API_ONLY   // probes of reference internals (static exec, the constexpr matrix)
 // SaturateCast<float, uchar> over an array, one element at a time.
 int fklref_saturate_cast_u8(const float* in, int n, uint8_t* out) {
     for (int i = 0; i < n; ++i) out[i] = SaturateCast<float, uchar>::exec(in[i]);
@@ -321,6 +326,8 @@ int fklref_yuv2rgb_709_full_matrix(float* m9) {
     m9[6] = m.z.x; m9[7] = m.z.y; m9[8] = m.z.z;
     return 0;
 }
+
+#endif
 
 // Letterbox geometry and factors the reference computes for one crop size (PRESERVE_AR), read back from the
 // built IOp: out = {x1, y1, x2, y2}, f = {fx, fy}.
@@ -338,6 +345,7 @@ int fklref_resize_params_par(int sw, int sh, int dw, int dh, int32_t* out4, floa
 // ---- pixel formats and colour conversions (tests/cases/color_chains.h on the reference's CPU backend) ----------
 namespace {
 using RefColor = color_chains::Chains<CpuDPP, CpuStream>;
+#ifndef FKL_HARNESS_PUBLIC_API_ONLY
 template <int CD, int CR, int CP, int DIR> void color_matrix_of(float* m9) {
     constexpr M3x3Float m = ccMatrix<ColorRange(CR), ColorPrimitives(CP), ColorConversionDir(DIR), ColorDepth(CD)>;
     m9[0] = m.x.x; m9[1] = m.x.y; m9[2] = m.x.z;
@@ -349,6 +357,7 @@ template <size_t... I> MatrixFn matrix_fn(size_t i, std::index_sequence<I...>) {
     static constexpr MatrixFn table[] = {&color_matrix_of<int(I / 12), int((I / 6) % 2), int((I / 2) % 3), int(I % 2)>...};
     return table[i];
 }
+#endif
 } // namespace
 
 extern "C" {
@@ -389,6 +398,7 @@ int fklref_normalize(int which, const void* src, int w, int h, int pitch, float*
     s.sync();
     return rc;
 }
+#ifndef FKL_HARNESS_PUBLIC_API_ONLY
 // ccMatrix<range, primaries, direction, depth> as the reference computes it at compile time, row major.
 // to_rgb = 1 selects YCbCr2RGB.
 int fklref_color_matrix(int cd, int cr, int cp, int to_rgb, float* m9) {
@@ -397,6 +407,7 @@ int fklref_color_matrix(int cd, int cr, int cp, int to_rgb, float* m9) {
     matrix_fn(((size_t(cd) * 2 + size_t(cr)) * 3 + size_t(cp)) * 2 + dir, std::make_index_sequence<72>{})(m9);
     return 0;
 }
+#endif
 
 } // extern "C"
 

@@ -60,7 +60,8 @@ template <ParArch PA> struct Chains {
     template <int BATCH, CircularTensorOrder ORDER>
     static void circular_one(StreamT& s, const uint8_t* const* images, int iters, int w, int h, int pitch, MemType mem, float fill, float* states) {
         const uint width = uint(w), height = uint(h);
-        CircularTensor<float, 3, BATCH, ORDER, ColorPlanes::Standard> window(width, height);
+        // the window lives where the caller's images do (a host build of the reference has no other memory anyway)
+        CircularTensor<float, 3, BATCH, ORDER, ColorPlanes::Standard> window(width, height, mem == MemType::Host ? MemType::Host : defaultMemType);
         setTo(fill, window, s);
         const size_t plane = size_t(w) * size_t(h) * 3;
         for (int i = 0; i < iters; ++i) {

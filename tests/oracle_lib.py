@@ -138,6 +138,28 @@ def ref():
     return _ref
 
 
+# The same harness compiled against THIS repository's headers (oracle/Makefile, target hostexec): the chains then run on
+# this repository's TransformDPP<ParArch::CPU> executor.  `with host_executor():` makes the ref_* wrappers below call it.
+HOSTEXEC_SO = os.path.join(ROOT, "oracle", "libfkl_hostexec.so")
+
+
+def have_hostexec() -> bool:
+    return os.path.exists(HOSTEXEC_SO)
+
+
+class host_executor:
+    def __enter__(self):
+        global _ref
+        self.saved = _ref
+        _ref = C.CDLL(HOSTEXEC_SO)
+        return _ref
+
+    def __exit__(self, *exc):
+        global _ref
+        _ref = self.saved
+        return False
+
+
 # ---- helpers to describe chains to the oracle -----------------------------------------------------------
 
 def op(code, p=(0, 0, 0, 0), idx=(0, 0, 0, 0)) -> Op:

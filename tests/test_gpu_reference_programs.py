@@ -16,7 +16,9 @@ TESTS = ["tests_algorithm_test_crop", "tests_algorithm_test_batchresize_build", 
          "tests_algorithm_test_warp", "tests_algorithm_test_border_reader", "tests_data_test_ptr_nd", "tests_data_test_rect",
          "tests_data_test_circular_tensor", "tests_data_parallel_patterns_test_divergent_batch",
          "tests_examples_compiler_explorer_example", "tests_buildAPI_batch_build_compilation_time",
-         "tests_operation_test_cricular_batch", "utests_core_execution_model_utest_executors"]
+         "tests_operation_test_cricular_batch", "tests_examples_readme_test_code", "utests_core_execution_model_utest_executors"]
+# host-only logic (no device call): also run where there is no GPU
+HOST_TESTS = ["tests_thread_fusion_test_thread_fusion"]
 BENCHMARKS = ["benchmarks_fusion_benchmark_horizontal_fusion", "benchmarks_fusion_benchmark_thread_fusion",
               "benchmarks_latencyhiding_benchmark_latency_hiding", "benchmarks_numinstructions_benchmark_numinstructions_x_operation"]
 
@@ -46,8 +48,14 @@ def test_reference_benchmark_program_runs_and_checks_out(device, name, tmp_path)
     assert any(f.endswith("_GPU_AMD.csv") for f in os.listdir(tmp_path))
 
 
+@pytest.mark.parametrize("name", HOST_TESTS)
+def test_reference_host_test_program_passes(name, tmp_path):
+    out = run_program(name, tmp_path)
+    assert "Failed" not in out
+
+
 def test_reference_programs_are_built_where_the_reference_tree_is():
     if not os.path.isdir("/root/reference/tests"):
         pytest.skip("no reference tree here")
-    missing = [n for n in TESTS + BENCHMARKS if not os.path.exists(os.path.join(PROGRAMS, n))]
+    missing = [n for n in TESTS + HOST_TESTS + BENCHMARKS if not os.path.exists(os.path.join(PROGRAMS, n))]
     assert not missing, f"run __graft_entry__.build(): not built: {missing}"
