@@ -237,7 +237,13 @@ template <typename Operation, typename Enabler = void> struct Lower {
 template <typename Operation, typename = void> struct has_lowering : std::true_type {};
 template <typename Operation> struct has_lowering<Operation, std::enable_if_t<!Lower<Operation>::available>> : std::false_type {};
 
-template <typename IOp> using device_op_t = typename Lower<typename IOp::Operation>::type;
+template <typename Operation, bool = has_lowering<Operation>::value> struct DeviceOperationOf { using type = typename Lower<Operation>::type; };
+template <typename Operation> struct DeviceOperationOf<Operation, false> {
+    static_assert(has_lowering<Operation>::value,
+                  "this Operation has no MI355X lowering: specialise fk::amd::Lower<Operation> (device type + parameter conversion)");
+    using type = void;
+};
+template <typename IOp> using device_op_t = typename DeviceOperationOf<typename IOp::Operation>::type;
 template <typename IOp> auto lower_iop(const IOp& iop) {
     using Op = typename IOp::Operation;
     static_assert(has_lowering<Op>::value,

@@ -206,3 +206,54 @@ static_assert(std::is_same_v<decltype(fk::ReadYUV<fk::PixelFormat::UYVY>::build(
 static_assert(std::is_same_v<decltype(fk::WriteYUV<fk::PixelFormat::P010>::build(fk::RawImage<fk::PixelFormat::P010>{})),
                              fk::Write<fk::WriteYUV<fk::PixelFormat::P010>>>);
 static_assert(fk::maxDepthValue<fk::ColorDepth::p10bit> == 1023 && fk::maxDepthValue<fk::ColorDepth::fn12bit> == 1.f);
+
+// ---- A user-defined Operation, declared the way the reference documents it (Parent + DECLARE_*_PARENT + exec):
+// it builds, fuses and type-checks on the host; launching it needs fk::amd::Lower<> (checked by tests/test_abi.py, which
+// compiles this file a second time with FK_API_COMPAT_LAUNCH_USER_OP and expects the explanatory static_assert) --------
+#include <fused_kernel/core/execution_model/operation_model/parent_operations.h>
+#include <fused_kernel/core/execution_model/thread_fusion.h>
+#include <fused_kernel/core/utils/vlimits.h>
+namespace user_ops {
+template <typename I, typename O> struct Twice {
+private:
+    using SelfType = Twice<I, O>;
+public:
+    FK_STATIC_STRUCT(Twice, SelfType)
+    using Parent = fk::UnaryOperation<I, O, Twice<I, O>>;
+    DECLARE_UNARY_PARENT
+    FK_HOST_DEVICE_FUSE OutputType exec(const InputType& input) { return static_cast<O>(input * 2); }
+};
+template <typename I, typename P = I, typename O = I> struct AddThrice {
+private:
+    using SelfType = AddThrice<I, P, O>;
+public:
+    FK_STATIC_STRUCT(AddThrice, SelfType)
+    using Parent = fk::BinaryOperation<I, P, O, AddThrice<I, P, O>>;
+    DECLARE_BINARY_PARENT
+    FK_HOST_DEVICE_FUSE OutputType exec(const InputType& input, const ParamsType& params) { return input + params * 3; }
+};
+} // namespace user_ops
+static_assert(user_ops::Twice<int, float>::exec(4) == 8.f);
+constexpr auto userBinary = user_ops::AddThrice<float>::build(2.f);
+static_assert(user_ops::AddThrice<float>::exec(1.f, userBinary) == 7.f);
+static_assert(fk::opIs<fk::UnaryType, decltype(user_ops::Twice<int, float>::build())> && fk::opIs<fk::BinaryType, decltype(userBinary)>);
+constexpr auto userFused = fk::PerThreadRead<fk::ND::_2D, float>::build(fk::RawPtr<fk::ND::_2D, float>{nullptr, {8, 8, 32}}).then(userBinary);
+static_assert(fk::opIs<fk::ReadType, decltype(userFused)>, "a user-defined Operation fuses onto a read like any other");
+#ifdef FK_API_COMPAT_LAUNCH_USER_OP
+inline void launch_user_op(fk::Stream& s, const fk::Ptr2D<float>& a, const fk::Ptr2D<float>& b) {
+    fk::executeOperations<fk::TransformDPP<>>(s, fk::PerThreadRead<fk::ND::_2D, float>::build(a), userBinary,
+                                              fk::PerThreadWrite<fk::ND::_2D, float>::build(b));
+}
+#endif
+
+// ---- Thread-fusion type arithmetic and numeric limits, the reference's answers --------------------------------------
+static_assert(fk::ThreadFusionInfo<uchar, uchar, true>::elems_per_thread == 4 && fk::ThreadFusionInfo<float, float, true>::elems_per_thread == 2);
+static_assert(fk::ThreadFusionInfo<uchar3, uchar3, true>::elems_per_thread == 1 && fk::ThreadFusionInfo<double, double, true>::elems_per_thread == 1);
+static_assert(std::is_same_v<fk::ThreadFusionInfo<float, float, true>::BiggerReadType, float2> &&
+              std::is_same_v<fk::ThreadFusionInfo<uchar2, uchar2, true>::BiggerWriteType, uchar4>);
+static_assert(!fk::ThreadFusionInfo<uchar, float3, true>::ENABLED && fk::ThreadFusionInfo<uchar, float3, true>::elems_per_thread == 1,
+              "four fused reads times three channels is no vector type: fusion is off");
+static_assert(fk::isThreadFusionEnabled<true, fk::Read<fk::PerThreadRead<fk::ND::_2D, float>>, fk::Write<fk::PerThreadWrite<fk::ND::_2D, float>>>());
+static_assert(!fk::isThreadFusionEnabled<true, fk::Read<fk::PerThreadRead<fk::ND::_2D, float3>>, fk::Write<fk::TensorSplit<float3>>>(),
+              "a planar split never fuses threads");
+static_assert(fk::maxValue<uchar> == 255 && fk::minValue<float3>.y == -3.402823466e+38f);

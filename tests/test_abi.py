@@ -66,3 +66,13 @@ def test_host_api_translation_unit_compiles_and_resolves_signatures():
     r = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), src],
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_launching_a_user_defined_operation_without_a_lowering_is_a_compile_time_message():
+    """A reference-style user Operation (Parent + DECLARE_*_PARENT + exec) compiles and fuses; asking the GPU executor to
+    launch it stops the build with the sentence that says what is missing, not with a template error."""
+    src = os.path.join(ROOT, "tests", "cases", "api_compat.cpp")
+    r = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-DFK_API_COMPAT_LAUNCH_USER_OP", "-I", os.path.join(ROOT, "include"), src],
+                       capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "this Operation has no MI355X lowering: specialise fk::amd::Lower<Operation>" in r.stderr
