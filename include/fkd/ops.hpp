@@ -1065,6 +1065,56 @@ template <class I, class O> struct Discard {
 };
 
 // Fold of compute operations over a value, left to right.  FK/core/execution_model/data_parallel_patterns.h:75-78.
+// Saturate<T>: every channel clamped to [lo, hi] with the comparisons of cxp::clamp, (v < lo) ? lo : ((hi < v) ? hi : v),
+// so a NaN channel stays NaN.  FK/algorithms/image_processing/saturate.h:38-49, FK/core/constexpr_libs/
+// constexpr_cmath.h:60-62.  SaturateDepth<T, CD> is this with lo = 0 and hi = the depth's largest value
+// (FK/algorithms/image_processing/color_conversion.h:96-107).
+template <class T> struct Saturate {
+    using In = T; using Out = T;
+    struct Params { base_t<T> lo, hi; };
+    FKD_NAME("Saturate<" + type_name<T>() + ">")
+    FKD_DEV static T exec(const T& a, const Params& p) {
+        return map1<T>(a, [&](auto v) { return (v < p.lo) ? p.lo : ((p.hi < v) ? p.hi : v); });
+    }
+};
+
+// SaturateFloat<T>: every float channel through fmaxf(0, fminf(s, 1)), spelled with comparisons so that the special cases
+// come out as on the reference's CPU backend (x86-64, glibc): NaN -> 1 (fminf returns its other operand), -0 stays -0
+// (of two zeros fmaxf returns its second operand there), everything else clamped to [0, 1].
+// FK/algorithms/image_processing/saturate.h:51-64, FK/core/constexpr_libs/constexpr_saturate.h:152-168.
+template <class T> struct SaturateFloat {
+    static_assert(__is_same(base_t<T>, f32), "Saturate float only works with float base types.");
+    using In = T; using Out = T; using Params = Empty;
+    FKD_NAME("SaturateFloat<" + type_name<T>() + ">")
+    FKD_DEV static f32 unit(f32 s) {
+        const f32 t = (s < 1.f) ? s : 1.f;
+        return (t < 0.f) ? 0.f : t;
+    }
+    FKD_DEV static T exec(const T& a, const Params&) { return map1<T>(a, [](f32 v) { return unit(v); }); }
+};
+
+// DenormalizePixel<O, CD>: float channels times the depth's largest value, converted to O's channel type like a C cast
+// (truncation toward zero; the product must be representable, which it is for inputs in [0, 1]).
+// FK/algorithms/image_processing/color_conversion.h:109-121.
+template <class O, int CD> struct DenormalizePixel {
+    using In = vec_t<f32, cn_v<O>>; using Out = O; using Params = Empty;
+    FKD_NAME("DenormalizePixel<" + type_name<O>() + "," + istr(CD) + ">")
+    FKD_DEV static O exec(const In& a, const Params&) {
+        return map1<O>(a, [](f32 v) { return static_cast<base_t<O>>(v * DepthConsts<CD>::max_v); });
+    }
+};
+
+// SaturateDenormalizePixel<I, O, CD>: SaturateFloat, then DenormalizePixel.
+// FK/algorithms/image_processing/color_conversion.h:136-148.
+template <class I, class O, int CD> struct SaturateDenormalizePixel {
+    static_assert(__is_same(base_t<I>, f32) && cn_v<I> == cn_v<O>, "SaturateDenormalizePixel only works with float base types.");
+    using In = I; using Out = O; using Params = Empty;
+    FKD_NAME("SaturateDenormalizePixel<" + type_name<I>() + "," + type_name<O>() + "," + istr(CD) + ">")
+    FKD_DEV static O exec(const I& a, const Params&) {
+        return map1<O>(a, [](f32 v) { return static_cast<base_t<O>>(SaturateFloat<f32>::unit(v) * DepthConsts<CD>::max_v); });
+    }
+};
+
 template <class... Ops> struct OpList {
     using Params = Tup<typename Ops::Params...>;
 #if defined(FKD_HOST_NAMES)
@@ -1319,25 +1369,44 @@ template <class T> struct Read3D {
 #endif
 };
 
-// TensorPack<T>: FK/algorithms/basic_ops/memory_operations.h:243-290.  The planar layout TensorSplit writes, read back
-// as a vector: channel c of pixel (x, y, z) sits c * width * height base elements after the position of channel 0.
-template <class T> struct TensorPack {
+// Where the channel planes of a planar tensor lie.  Standard (TensorSplit / TensorPack, FK/core/data/rawptr.h:215-227):
+// image z starts z * plane_pitch * color_planes bytes into the tensor and channel c of a pixel sits c * width * height
+// elements after channel 0.  Transposed (TensorTSplit / TensorTPack, FK/core/data/rawptr.h:229-240): image z starts
+// z * plane_pitch bytes in and channel c sits c * color_planes_pitch bytes after channel 0 (a multiple of the element
+// size: rows are whole elements).
+namespace detail {
+template <class B, bool TRANSPOSED> struct PlanarGeometry;
+template <class B> struct PlanarGeometry<B, false> {
+    template <class E> using View = RawPtr3D<E>;
+    template <class P> FKD_HD static size_t image_bytes(const P& p) { return size_t(p.plane_pitch) * p.color_planes; }
+    template <class P> FKD_HD static size_t channel_elements(const P& p) { return size_t(p.width) * p.height; }
+};
+template <class B> struct PlanarGeometry<B, true> {
+    template <class E> using View = RawPtrT3D<E>;
+    template <class P> FKD_HD static size_t image_bytes(const P& p) { return size_t(p.plane_pitch); }
+    template <class P> FKD_HD static size_t channel_elements(const P& p) { return size_t(p.color_planes_pitch) / sizeof(B); }
+};
+} // namespace detail
+
+// TensorPack<T>: FK/algorithms/basic_ops/memory_operations.h:243-290, and TensorTPack<T> (TRANSPOSED), :292-327.  The
+// planar layout TensorSplit / TensorTSplit writes, read back as a vector.
+template <class T, bool TRANSPOSED = false> struct TensorPack {
     static_assert(cn_v<T> >= 2, "Wrong type for split tensor read. It must be one of <type>2, <type>3 or <type>4.");
     using Out = T;
     using B = base_t<T>;
-    using Params = RawPtr3D<const B>;
+    using G = detail::PlanarGeometry<B, TRANSPOSED>;
+    using Params = typename G::template View<const B>;
     static constexpr bool kTapCursor = false;
-    FKD_NAME("TensorPack<" + type_name<T>() + ">")
+    FKD_NAME((TRANSPOSED ? "TensorTPack<" : "TensorPack<") + type_name<T>() + ">")
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
     FKD_DEV static const B* at(const Params& p, int x, int y, int z) {
-        return reinterpret_cast<const B*>(reinterpret_cast<const char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z +
-                                          size_t(y) * p.pitch) + x;
+        return reinterpret_cast<const B*>(reinterpret_cast<const char*>(p.data) + G::image_bytes(p) * z + size_t(y) * p.pitch) + x;
     }
     FKD_DEV static T exec(int x, int y, int z, const Params& p) {
         const FKD_GLOBAL B* g = detail::gconst<B>(at(p, x, y, z));
-        const size_t px = size_t(p.width) * p.height;
+        const size_t px = G::channel_elements(p);
         T o;
         chan<0>(o) = g[0];
         chan<1>(o) = g[px];
@@ -1349,7 +1418,7 @@ template <class T> struct TensorPack {
 #if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<T> (&out)[V]) {
         const B* r = at(p, x, y, z);
-        const size_t px = size_t(p.width) * p.height;
+        const size_t px = G::channel_elements(p);
         Slot<B> c[4][V];
         detail::load_run<B, V, A>(r, c[0]);
         detail::load_run<B, V, A>(r + px, c[1]);
@@ -1365,7 +1434,7 @@ template <class T> struct TensorPack {
     }
     FKD_HD static bool rows_aligned(const Params& p, int xoff) {
         return detail::dword_aligned(reinterpret_cast<const char*>(p.data) + ptrdiff_t(xoff) * ptrdiff_t(sizeof(B))) && p.pitch % 4 == 0 &&
-               (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 && (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
+               G::image_bytes(p) % 4 == 0 && (G::channel_elements(p) * sizeof(B)) % 4 == 0;
     }
     using Raw = Out;
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
@@ -1373,6 +1442,8 @@ template <class T> struct TensorPack {
     static constexpr bool kTapOverread = false, kTapPair = false;
 #endif
 };
+
+template <class T> using TensorTPack = TensorPack<T, true>;
 
 // Plane index of a circular buffer of BATCH planes whose logical plane 0 is stored at `first`:
 // computeCircularThreadIdx, FK/algorithms/basic_ops/memory_operations.h:422-432.  DIR 0 (Ascendent) walks forward from
@@ -2190,21 +2261,22 @@ template <class T> struct TensorWrite {
 #endif
 };
 
-// TensorSplit<T>: FK/algorithms/basic_ops/memory_operations.h:181-212.  Planar store: channel c of pixel
-// (x,y) of plane z goes to the 3-D address of (x,y,z) plus c*width*height base elements.
-template <class T> struct TensorSplit {
+// TensorSplit<T>: FK/algorithms/basic_ops/memory_operations.h:181-212, and TensorTSplit<T> (TRANSPOSED), :214-241.
+// Planar store: channel c of pixel (x,y) of image z goes to the address of (x,y,z) plus c channel planes
+// (detail::PlanarGeometry).
+template <class T, bool TRANSPOSED = false> struct TensorSplit {
     using In = T;
     using B = base_t<T>;
-    using Params = RawPtr3D<B>;
-    FKD_NAME("TensorSplit<" + type_name<T>() + ">")
+    using G = detail::PlanarGeometry<B, TRANSPOSED>;
+    using Params = typename G::template View<B>;
+    FKD_NAME((TRANSPOSED ? "TensorTSplit<" : "TensorSplit<") + type_name<T>() + ">")
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static B* at(const Params& p, int x, int y, int z) {
-        return reinterpret_cast<B*>(reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z +
-                                    size_t(y) * p.pitch) + x;
+        return reinterpret_cast<B*>(reinterpret_cast<char*>(p.data) + G::image_bytes(p) * z + size_t(y) * p.pitch) + x;
     }
     FKD_DEV static void exec(int x, int y, int z, const T& v, const Params& p) {
         B* w = at(p, x, y, z);
-        const size_t px = size_t(p.width) * p.height;
+        const size_t px = G::channel_elements(p);
         FKD_GLOBAL B* gw = detail::gmut<B>(w);
         gw[0] = chan<0>(v);
         gw[px] = chan<1>(v);
@@ -2215,7 +2287,7 @@ template <class T> struct TensorSplit {
 #if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         B* w = at(p, x, y, z);
-        const size_t px = size_t(p.width) * p.height;
+        const size_t px = G::channel_elements(p);
         Slot<B> c0[V], c1[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) { c0[i].v = chan<0>(v[i].v); c1[i].v = chan<1>(v[i].v); }
@@ -2235,8 +2307,7 @@ template <class T> struct TensorSplit {
         }
     }
     FKD_HD static bool rows_aligned(const Params& p) {
-        return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && (size_t(p.plane_pitch) * p.color_planes) % 4 == 0 &&
-               (size_t(p.width) * p.height * sizeof(B)) % 4 == 0;
+        return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && G::image_bytes(p) % 4 == 0 && (G::channel_elements(p) * sizeof(B)) % 4 == 0;
     }
     // The part of the parameters one plane needs (all of them here).
     using Plane = TensorSplit;
@@ -2250,13 +2321,14 @@ template <class T> struct TensorSplit {
     static constexpr u32 kMaskedExtent = 0x7fffffffu, kMaskedOut = 0x80000000u;
     struct PlaneRef { __amdgpu_buffer_rsrc_t rsrc; u32 chan_bytes, pitch; };
     FKD_DEV static bool plane_maskable(const Params& p) {
-        return size_t(p.width) * p.height * sizeof(B) * cn_v<T> < size_t(kMaskedExtent) && size_t(p.pitch) * p.height < size_t(kMaskedExtent);
+        return G::channel_elements(p) * sizeof(B) * cn_v<T> < size_t(kMaskedExtent) &&
+               G::channel_elements(p) * sizeof(B) * (cn_v<T> - 1) + size_t(p.pitch) * p.height < size_t(kMaskedExtent);
     }
     FKD_DEV static PlaneRef plane_ref(int z, const Params& p) {
-        char* base = reinterpret_cast<char*>(p.data) + size_t(p.plane_pitch) * p.color_planes * z;
+        char* base = reinterpret_cast<char*>(p.data) + G::image_bytes(p) * z;
         PlaneRef r;
         r.rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, kMaskedExtent, 0x00020000);   // raw 32-bit data, as detail::make_tap_image
-        r.chan_bytes = p.width * p.height * u32(sizeof(B));
+        r.chan_bytes = u32(G::channel_elements(p) * sizeof(B));
         r.pitch = p.pitch;
         return r;
     }
@@ -2270,7 +2342,7 @@ template <class T> struct TensorSplit {
         if constexpr (cn_v<T> > 3) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<3>(v)), r.rsrc, lane_off, row_off + 3u * r.chan_bytes, kThrough);
     }
     struct RowRef { B* p; size_t px; };
-    FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), size_t(p.width) * p.height}; }
+    FKD_DEV static RowRef row(int y, int z, const Params& p) { return RowRef{at(p, 0, y, z), G::channel_elements(p)}; }
     FKD_DEV static void put(const RowRef& r, int x, const T& v) {
         u32 off = u32(x) * u32(sizeof(B));   // one lane offset, four wave-uniform plane row addresses
         asm volatile("" : "+v"(off));
@@ -2301,6 +2373,8 @@ template <class T> struct TensorSplit {
     }
 #endif
 };
+
+template <class T> using TensorTSplit = TensorSplit<T, true>;
 
 // WriteYUV<NV12 | NV21 | P010 | P210 | Y210 | UYVY>: FK/algorithms/image_processing/color_conversion.h:298-389.  The value
 // is (Y, U, V).  Semi-planar formats store Y at (x, y) and the chroma pair of a 2x2 (4:2:0) or 2x1 (4:2:2) block from

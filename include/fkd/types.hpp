@@ -120,6 +120,13 @@ template <class T> struct RawPtr3D {
     T* data;
     u32 width, height, planes, color_planes, pitch, plane_pitch;
 };
+// Batched 3-D view with the channel planes outermost ("transposed": all R planes, then all G planes, ...): channel
+// plane c of image z starts at data + c*color_planes_pitch + z*plane_pitch, plane_pitch = pitch*height,
+// color_planes_pitch = plane_pitch*planes.
+template <class T> struct RawPtrT3D {
+    T* data;
+    u32 width, height, planes, color_planes, pitch, plane_pitch, color_planes_pitch;
+};
 // NV12 frame: luma rows 0..height-1, then height/2 rows of interleaved (U,V) pairs, all with one pitch.
 struct RawNV12 {
     const u8* data;

@@ -1,7 +1,7 @@
 // Per-element memory operations: PerThreadRead / PerThreadWrite (pitched 1-D/2-D/3-D), TensorRead / TensorWrite,
 // TensorSplit (planar writer) and TensorPack (its reader), and the circular-buffer views CircularTensorRead /
 // CircularTensorWrite.  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:26-212, 243-290, 413-432,
-// 505-587.  CircularBatchRead / CircularBatchWrite (434-503) too.  The transposed-plane forms (TensorTSplit / TensorTPack) are not built.
+// 505-587.  CircularBatchRead / CircularBatchWrite (434-503) and the transposed-plane forms TensorTSplit / TensorTPack (214-241, 292-327) too.
 #ifndef FK_AMD_MEMORY_OPERATIONS_H
 #define FK_AMD_MEMORY_OPERATIONS_H
 
@@ -105,6 +105,31 @@ template <typename T> struct TensorPack : ReadOperation<VBase<T>, RawPtr<ND::_3D
     }
 };
 
+// Planar writer and reader of a transposed tensor (RawPtr<ND::T3D>): channel c of pixel (x, y, z) lies in colour plane c,
+// c * color_planes_pitch bytes after channel 0.  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:214-241
+// (TensorTSplit) and :292-327 (TensorTPack).
+template <typename T> struct TensorTSplit : WriteOperation<T, RawPtr<ND::T3D, VBase<T>>, VBase<T>, TF::DISABLED, TensorTSplit<T>> {
+    using Parent = WriteOperation<T, RawPtr<ND::T3D, VBase<T>>, VBase<T>, TF::DISABLED, TensorTSplit<T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(TensorTSplit, TensorTSplit)
+    static_assert(cn<T> >= 2, "Wrong type for split tensor write. It must be one of <type>2, <type>3 or <type>4.");
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+};
+template <typename T> struct TensorTPack : ReadOperation<T, RawPtr<ND::T3D, VBase<T>>, T, TF::DISABLED, TensorTPack<T>> {
+    using Parent = ReadOperation<T, RawPtr<ND::T3D, VBase<T>>, T, TF::DISABLED, TensorTPack<T>>;
+    using typename Parent::OperationDataType;
+    FK_STATIC_STRUCT(TensorTPack, TensorTPack)
+    static_assert(cn<T> >= 2, "Wrong type for split tensor read. It must be one of <type>2, <type>3 or <type>4.");
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
+    static constexpr uint num_elems_y(const Point, const OperationDataType& opData) { return opData.params.dims.height; }
+    static constexpr uint num_elems_z(const Point, const OperationDataType& opData) { return opData.params.dims.planes; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {opData.params.dims.width, opData.params.dims.height, opData.params.dims.planes};
+    }
+};
+
 // A tensor of BATCH planes used as a circular buffer: logical plane z lives at (first + z) mod BATCH (Ascendent) or
 // (first - z) mod BATCH (Descendent).
 enum class CircularDirection { Ascendent, Descendent };
@@ -180,6 +205,13 @@ template <typename T> struct Lower<TensorPack<T>> {
     using type = fkd::TensorPack<dev_t<T>>;
     static typename type::Params params(const OperationData<TensorPack<T>>& d) {
         return to_dev3<VBase<T>, const typename DevType<VBase<T>>::type>(d.params);
+    }
+};
+template <typename T> struct Lower<TensorTPack<T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorTPack<dev_t<T>>;
+    static typename type::Params params(const OperationData<TensorTPack<T>>& d) {
+        return to_devT3<VBase<T>, const typename DevType<VBase<T>>::type>(d.params);
     }
 };
 template <CircularDirection direction, typename Operation, int BATCH> struct Lower<CircularBatchRead<direction, Operation, BATCH>> {
@@ -266,6 +298,25 @@ template <typename T> struct Lower<TensorSplit<T>> {
     static typename type::Params params(const OperationData<TensorSplit<T>>& d) {
         return to_dev3<VBase<T>, typename DevType<VBase<T>>::type>(d.params);
     }
+};
+template <typename T> struct Lower<TensorTSplit<T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorTSplit<dev_t<T>>;
+    static typename type::Params params(const OperationData<TensorTSplit<T>>& d) {
+        return to_devT3<VBase<T>, typename DevType<VBase<T>>::type>(d.params);
+    }
+};
+// PerThreadRead / PerThreadWrite on a transposed tensor address colour plane 0 only (the accessor's default), as in the
+// reference (FK/core/data/rawptr.h:229-240).
+template <typename T> struct Lower<PerThreadRead<ND::T3D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::Read3D<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadRead<ND::T3D, T>>& d) { return first_color_plane<T, const dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<PerThreadWrite<ND::T3D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::TensorWrite<dev_t<T>>;
+    static typename type::Params params(const OperationData<PerThreadWrite<ND::T3D, T>>& d) { return first_color_plane<T, dev_t<T>>(d.params); }
 };
 } // namespace amd
 

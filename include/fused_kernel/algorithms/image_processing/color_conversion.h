@@ -1,10 +1,9 @@
 // Colour operations of the fused path: channel swaps, alpha insertion/removal and gray (ColorConversion<code, ...>),
 // the pixel-format readers and writers ReadYUV<PF> / WriteYUV<PF>, the YCbCr<->RGB conversions for every depth, range
-// and set of primaries, and NormalizePixel.
-// Interface counterpart: FK/algorithms/image_processing/color_conversion.h:28-93, 121-132, 150-201, 206-389, 391-505.
+// and set of primaries, NormalizePixel, SaturateDepth, DenormalizePixel and SaturateDenormalizePixel.
+// Interface counterpart: FK/algorithms/image_processing/color_conversion.h:28-201, 206-389, 391-505.
 // Pixel formats the reference declares but gives no reader/writer (YV12, P016, P216, Y216), or whose reader does not
 // compile there (Y416: four values into a three-channel pixel), fail at compile time here with a message that says so.
-// SaturateDepth, DenormalizePixel and SaturateDenormalizePixel are not built.
 #ifndef FK_AMD_COLOR_CONVERSION_H
 #define FK_AMD_COLOR_CONVERSION_H
 
@@ -45,6 +44,27 @@ template <typename I, ColorDepth CD> struct AddOpaqueAlpha : UnaryOperation<I, V
 template <typename I, ColorDepth CD> struct NormalizePixel : UnaryOperation<I, VectorType_t<float, cn<I>>, NormalizePixel<I, CD>> {
     using Parent = UnaryOperation<I, VectorType_t<float, cn<I>>, NormalizePixel<I, CD>>;
     FK_STATIC_STRUCT(NormalizePixel, NormalizePixel)
+};
+
+// Every channel clamped to [0, largest value of the depth].  The reference spells this for T = float only (its body calls
+// Saturate<float>); vectors of float work the same way here.
+template <typename T, ColorDepth CD> struct SaturateDepth : UnaryOperation<T, T, SaturateDepth<T, CD>> {
+    using Parent = UnaryOperation<T, T, SaturateDepth<T, CD>>;
+    FK_STATIC_STRUCT(SaturateDepth, SaturateDepth)
+    static_assert(std::is_same_v<VBase<T>, float>, "SaturateDepth works on float channels");
+};
+
+// float channels * largest value of the depth, converted to O's channel type like a C cast (towards zero).
+template <typename O, ColorDepth CD> struct DenormalizePixel : UnaryOperation<VectorType_t<float, cn<O>>, O, DenormalizePixel<O, CD>> {
+    using Parent = UnaryOperation<VectorType_t<float, cn<O>>, O, DenormalizePixel<O, CD>>;
+    FK_STATIC_STRUCT(DenormalizePixel, DenormalizePixel)
+};
+
+// SaturateFloat (clamp to [0, 1], NaN -> 1), then DenormalizePixel.
+template <typename I, typename O, ColorDepth CD> struct SaturateDenormalizePixel : UnaryOperation<I, O, SaturateDenormalizePixel<I, O, CD>> {
+    using Parent = UnaryOperation<I, O, SaturateDenormalizePixel<I, O, CD>>;
+    FK_STATIC_STRUCT(SaturateDenormalizePixel, SaturateDenormalizePixel)
+    static_assert(std::is_same_v<VBase<I>, float>, "SaturateDenormalizePixel only works with float base types.");
 };
 
 // (Y, Cb, Cr) -> float3 (R, G, B); no clamp.
@@ -200,6 +220,23 @@ template <typename I, ColorDepth CD> struct Lower<NormalizePixel<I, CD>> {
     static constexpr bool available = true;
     using type = fkd::Div<dev_t<I>, fkd::f32, dev_t<VectorType_t<float, cn<I>>>>;
     static typename type::Params params(const OperationData<NormalizePixel<I, CD>>&) { return type::make(static_cast<float>(maxDepthValue<CD>)); }
+};
+template <typename T, ColorDepth CD> struct Lower<SaturateDepth<T, CD>> {
+    static constexpr bool available = true;
+    using type = fkd::Saturate<dev_t<T>>;
+    static typename type::Params params(const OperationData<SaturateDepth<T, CD>>&) {
+        return typename type::Params{0.f, static_cast<float>(maxDepthValue<CD>)};
+    }
+};
+template <typename O, ColorDepth CD> struct Lower<DenormalizePixel<O, CD>> {
+    static constexpr bool available = true;
+    using type = fkd::DenormalizePixel<dev_t<O>, int(CD)>;
+    static typename type::Params params(const OperationData<DenormalizePixel<O, CD>>&) { return {}; }
+};
+template <typename I, typename O, ColorDepth CD> struct Lower<SaturateDenormalizePixel<I, O, CD>> {
+    static constexpr bool available = true;
+    using type = fkd::SaturateDenormalizePixel<dev_t<I>, dev_t<O>, int(CD)>;
+    static typename type::Params params(const OperationData<SaturateDenormalizePixel<I, O, CD>>&) { return {}; }
 };
 } // namespace amd
 

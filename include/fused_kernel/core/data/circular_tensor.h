@@ -3,7 +3,8 @@
 // new image and shifts the others by one plane in ONE launch: a DivergentBatchTransformDPP of two sequences, the
 // caller's chain with a store into a hidden circular copy put before its write, and a copy of the other BATCH - 1
 // planes out of that hidden copy.
-// Interface counterpart: FK/core/data/circular_tensor.h:24-168.  ColorPlanes::Transposed is not built.
+// Interface counterpart: FK/core/data/circular_tensor.h:24-168.  With ColorPlanes::Transposed the window is a TensorT
+// (all first channel planes, then all second ones, ...) and the chain must end in Write<TensorTSplit<StoreT>>.
 #ifndef FK_AMD_CIRCULAR_TENSOR_H
 #define FK_AMD_CIRCULAR_TENSOR_H
 
@@ -33,6 +34,11 @@ template <CircularTensorOrder CT_ORDER> static constexpr CircularDirection CTRea
 
 enum class ColorPlanes { Standard, Transposed };
 
+template <typename T, ColorPlanes CP_MODE> struct CoreType;
+template <typename T> struct CoreType<T, ColorPlanes::Standard> { using type = Tensor<T>; };
+template <typename T> struct CoreType<T, ColorPlanes::Transposed> { using type = TensorT<T>; };
+template <typename T, ColorPlanes CP_MODE> using CoreType_t = typename CoreType<T, CP_MODE>::type;
+
 template <typename T, int COLOR_PLANES, typename Enabler = void> struct CircularTensorStoreType {};
 template <typename T, int COLOR_PLANES> struct CircularTensorStoreType<T, COLOR_PLANES, std::enable_if_t<std::is_aggregate_v<T> && COLOR_PLANES == 1>> {
     using type = T;
@@ -41,13 +47,13 @@ template <typename T, int COLOR_PLANES> struct CircularTensorStoreType<T, COLOR_
     using type = VectorType_t<T, COLOR_PLANES>;
 };
 
-template <typename T, int COLOR_PLANES, int BATCH, CircularTensorOrder CT_ORDER, ColorPlanes CP_MODE> class CircularTensor : public Tensor<T> {
-    static_assert(CP_MODE == ColorPlanes::Standard, "ColorPlanes::Transposed (TensorT / TensorTSplit) is not built in this library");
-    using ParentType = Tensor<T>;
+template <typename T, int COLOR_PLANES, int BATCH, CircularTensorOrder CT_ORDER, ColorPlanes CP_MODE> class CircularTensor : public CoreType_t<T, CP_MODE> {
+    using ParentType = CoreType_t<T, CP_MODE>;
     using StoreT = typename CircularTensorStoreType<T, COLOR_PLANES>::type;
-    using WriteInstantiableOperations = TypeList<Write<TensorWrite<StoreT>>, Write<TensorSplit<StoreT>>>;
+    using WriteInstantiableOperations = TypeList<Write<TensorWrite<StoreT>>, Write<TensorSplit<StoreT>>, Write<TensorTSplit<StoreT>>>;
     using ReadInstantiableOperations = TypeList<Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorRead<StoreT>, BATCH>>,
-                                                Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorPack<StoreT>, BATCH>>>;
+                                                Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorPack<StoreT>, BATCH>>,
+                                                Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorTPack<StoreT>, BATCH>>>;
 
 public:
     CircularTensor() {}
@@ -64,8 +70,13 @@ public:
         const auto writeInstantiableOperation = ppLast(instantiableOperationInstances...);
         using writeDFType = std::decay_t<decltype(writeInstantiableOperation)>;
         using writeOpType = typename writeDFType::Operation;
-        static_assert(one_of_v<writeDFType, WriteInstantiableOperations>,
-                      "the chain given to CircularTensor::update must end in Write<TensorWrite<StoreT>> or Write<TensorSplit<StoreT>>");
+        if constexpr (CP_MODE == ColorPlanes::Transposed) {
+            static_assert(std::is_same_v<writeDFType, Write<TensorTSplit<StoreT>>>,
+                          "Need to use TensorTSplitWrite as write function because you are using a transposed CircularTensor (CP_MODE = Transposed)");
+        } else {
+            static_assert(one_of_v<writeDFType, TypeList<Write<TensorWrite<StoreT>>, Write<TensorSplit<StoreT>>>>,
+                          "the chain given to CircularTensor::update must end in Write<TensorWrite<StoreT>> or Write<TensorSplit<StoreT>>");
+        }
         using equivalentReadDFType = EquivalentType_t<writeDFType, WriteInstantiableOperations, ReadInstantiableOperations>;
 
         // The launch's planes are the planes of both sequences together: one for the new image, BATCH - 1 copied.
@@ -91,7 +102,7 @@ public:
     }
 
 private:
-    Tensor<T> m_tempTensor;
+    CoreType_t<T, CP_MODE> m_tempTensor;
     int m_nextUpdateIdx{0};
 };
 

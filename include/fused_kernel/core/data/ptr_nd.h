@@ -364,6 +364,18 @@ public:
     Ptr3D<T> crop3D(const Point p, const PtrDims<ND::_3D>& newDims) { return Ptr<ND::_3D, T>::crop(p, newDims); }
 };
 
+// A 3-D pointer with the colour planes outermost (every image's first channel plane, then every second one, ...).
+template <typename T> class PtrT3D : public Ptr<ND::T3D, T> {
+public:
+    PtrT3D(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+           const MemType& type_ = defaultMemType, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(PtrDims<ND::T3D>(width_, height_, planes_, color_planes_), type_, deviceID_) {}
+    PtrT3D(const Ptr<ND::T3D, T>& other) : Ptr<ND::T3D, T>(other) {}
+    PtrT3D(T* data_, const PtrDims<ND::T3D>& dims_, const MemType& type_ = defaultMemType, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(data_, dims_, type_, deviceID_) {}
+    PtrT3D<T> crop3D(const Point p, const PtrDims<ND::T3D>& newDims) { return Ptr<ND::T3D, T>::crop(p, newDims); }
+};
+
 // Contiguous batch of planes: rows are always tightly packed (pitch = sizeof(T) * width).
 template <typename T> class Tensor : public Ptr<ND::_3D, T> {
 public:
@@ -380,6 +392,32 @@ public:
                      const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
         this->freePtr();
         this->allocPtr(PtrDims<ND::_3D>(width_, height_, planes_, color_planes_, uint(sizeof(T)) * width_), type_, deviceID_);
+    }
+};
+
+// The same batch with the colour planes outermost (the layout TensorTSplit writes and TensorTPack reads).  A view over
+// caller-owned memory gets the tight pitches the allocating constructor would have chosen.
+template <typename T> class TensorT : public Ptr<ND::T3D, T> {
+    static PtrDims<ND::T3D> tightDims(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_) {
+        PtrDims<ND::T3D> d(width_, height_, planes_, color_planes_);
+        ptr_detail::Layout<ND::T3D, T>::tight(d);
+        return d;
+    }
+
+public:
+    TensorT() {}
+    TensorT(const TensorT<T>& other) : Ptr<ND::T3D, T>(other) {}
+    TensorT& operator=(const TensorT<T>& other) { Ptr<ND::T3D, T>::operator=(other); return *this; }
+    TensorT(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+            const MemType& type_ = defaultMemType, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(PtrDims<ND::T3D>(width_, height_, planes_, color_planes_), type_, deviceID_) {}
+    TensorT(T* data, const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+            const MemType& type_ = defaultMemType, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(data, tightDims(width_, height_, planes_, color_planes_), type_, deviceID_) {}
+    void allocTensor(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+                     const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
+        this->freePtr();
+        this->allocPtr(PtrDims<ND::T3D>(width_, height_, planes_, color_planes_), type_, deviceID_);
     }
 };
 

@@ -15,8 +15,17 @@ namespace fk {
 // filled, on the host and right away (the reference does this with its CPU executor, which this backend does not
 // have; a fill is plain data movement, not a computation of the fused path).
 template <ParArch PA, ND D, typename T> inline void setTo(const T& value, Ptr<D, T>& outputPtr, Stream_<PA>& stream) {
-    Executor<TransformDPP<PA>>::executeOperations(stream, ReadSet<T>::build(value, outputPtr.dims()),
-                                                  PerThreadWrite<D, T>::build(outputPtr.ptr()));
+    if constexpr (D == ND::T3D) {
+        // Every colour plane is filled: the planes of a transposed tensor follow each other at plane_pitch, so the whole
+        // of it is one batch of planes * color_planes planes.  (The reference's PerThreadWrite<T3D> addresses colour
+        // plane 0 only and leaves the others as they were.)
+        const auto t = outputPtr.ptr();
+        const RawPtr<ND::_3D, T> all{t.data, PtrDims<ND::_3D>(t.dims.width, t.dims.height, t.dims.planes * t.dims.color_planes, 1, t.dims.pitch)};
+        Executor<TransformDPP<PA>>::executeOperations(stream, ReadSet<T>::build(value, all.dims), PerThreadWrite<ND::_3D, T>::build(all));
+    } else {
+        Executor<TransformDPP<PA>>::executeOperations(stream, ReadSet<T>::build(value, outputPtr.dims()),
+                                                      PerThreadWrite<D, T>::build(outputPtr.ptr()));
+    }
     if (outputPtr.getMemType() == MemType::DeviceAndPinned) {
         const auto host = outputPtr.ptrPinned();
         const auto dims = host.dims;      // the mirror has its own (tight) pitch

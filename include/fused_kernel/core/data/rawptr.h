@@ -93,6 +93,20 @@ template <> struct PtrAccessor<ND::_3D> {
     }
 };
 
+// Channel planes outermost: channel plane c of image z starts c * color_planes_pitch + z * plane_pitch bytes in.
+template <> struct PtrAccessor<ND::T3D> {
+    template <typename T, typename BiggerType = T>
+    static const BiggerType* cr_point(const Point p, const RawPtr<ND::T3D, T>& ptr, const uint color_plane = 0) {
+        return (const BiggerType*)((const char*)ptr.data + (size_t(color_plane) * ptr.dims.color_planes_pitch) +
+                                   (size_t(ptr.dims.plane_pitch) * p.z) + (size_t(p.y) * ptr.dims.pitch)) + p.x;
+    }
+    template <typename T, typename BiggerType = T>
+    static BiggerType* point(const Point p, const RawPtr<ND::T3D, T>& ptr, const uint color_plane = 0) {
+        return (BiggerType*)((char*)ptr.data + (size_t(color_plane) * ptr.dims.color_planes_pitch) +
+                             (size_t(ptr.dims.plane_pitch) * p.z) + (size_t(p.y) * ptr.dims.pitch)) + p.x;
+    }
+};
+
 // Small arrays with compile-time extents held by value (transform matrices and the like).
 // Interface counterpart: FK/core/data/rawptr.h:105-185.
 template <int W> struct StaticPtrDims1D { static constexpr uint width{W}; };

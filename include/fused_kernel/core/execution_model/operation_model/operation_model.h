@@ -230,6 +230,15 @@ template <typename T, typename Q = T> fkd::RawPtr3D<Q> to_dev3(const RawPtr<ND::
                             p.dims.color_planes, p.dims.pitch, p.dims.plane_pitch};
 }
 
+template <typename T, typename Q = T> fkd::RawPtrT3D<Q> to_devT3(const RawPtr<ND::T3D, T>& p) {
+    return fkd::RawPtrT3D<Q>{reinterpret_cast<Q*>(p.data), p.dims.width, p.dims.height, p.dims.planes,
+                             p.dims.color_planes, p.dims.pitch, p.dims.plane_pitch, p.dims.color_planes_pitch};
+}
+// Colour plane 0 of a transposed tensor is an ordinary batch of planes (what PerThreadRead/Write<T3D> address).
+template <typename T, typename Q = T> fkd::RawPtr3D<Q> first_color_plane(const RawPtr<ND::T3D, T>& p) {
+    return fkd::RawPtr3D<Q>{reinterpret_cast<Q*>(p.data), p.dims.width, p.dims.height, p.dims.planes, 1u, p.dims.pitch, p.dims.plane_pitch};
+}
+
 // Primary: an Operation without a specialisation cannot run on this backend.
 template <typename Operation, typename Enabler = void> struct Lower {
     static constexpr bool available = false;

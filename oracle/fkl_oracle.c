@@ -306,6 +306,40 @@ static int apply_op(const fklo_op *op, fklo_val *v) {
         v->elem = FKLO_U8;
         return FKLO_OK;
     }
+    /* Saturate<T>::exec, FK/algorithms/image_processing/saturate.h:38-49 -> cxp::clamp, FK/core/constexpr_libs/
+     * constexpr_cmath.h:60-62: the two comparisons below, so NaN stays NaN.  SaturateDepth<T, CD>
+     * (color_conversion.h:96-107) is this with p = {0, maxDepthValue<CD>}. */
+    case FKLO_CLAMP: {
+        if (v->elem != FKLO_F32) return FKLO_ETYPE;
+        for (int c = 0; c < v->cn; ++c) {
+            const float a = v->f[c];
+            v->f[c] = (a < op->p[0]) ? op->p[0] : ((op->p[1] < a) ? op->p[1] : a);
+        }
+        return FKLO_OK;
+    }
+    /* SaturateFloat<T>::exec, saturate.h:51-64 -> cxp::saturate_float, FK/core/constexpr_libs/constexpr_saturate.h:152-168:
+     * fmaxf(0.f, fminf(s, 1.f)) on the host, written out with comparisons so the result does not depend on the C
+     * library at hand: fminf(NaN, 1) = 1, and of two zeros fmaxf returns its second operand on x86-64 (glibc's
+     * fmaxf ends in maxss), so -0 stays -0 while every other negative value becomes +0. */
+    case FKLO_SATURATE_FLOAT: {
+        if (v->elem != FKLO_F32) return FKLO_ETYPE;
+        for (int c = 0; c < v->cn; ++c) {
+            const float s = v->f[c];
+            const float t = (s < 1.0f) ? s : 1.0f;
+            v->f[c] = (t < 0.0f) ? 0.0f : t;
+        }
+        return FKLO_OK;
+    }
+    /* cxp::cast<O>::f, FK/core/constexpr_libs/constexpr_cmath.h:648-662: static_cast per channel; DenormalizePixel<O, CD>
+     * (color_conversion.h:109-121) is FKLO_MUL by maxDepthValue<CD> and then this. */
+    case FKLO_CAST_TRUNC: {
+        if (v->elem != FKLO_F32) return FKLO_ETYPE;
+        if (op->idx[0] == FKLO_U8) { for (int c = 0; c < v->cn; ++c) v->u[c] = (uint8_t)v->f[c]; }
+        else if (op->idx[0] == FKLO_U16) { for (int c = 0; c < v->cn; ++c) v->h[c] = (uint16_t)v->f[c]; }
+        else if (op->idx[0] != FKLO_F32) return FKLO_ETYPE;
+        v->elem = op->idx[0];
+        return FKLO_OK;
+    }
     case FKLO_CAST_F32: {
         if (v->elem != FKLO_F32) {
             for (int c = 0; c < v->cn; ++c) v->f[c] = chan_as_float(v, c);
@@ -331,7 +365,7 @@ static int apply_op(const fklo_op *op, fklo_val *v) {
  * ReadYUV<NV12>::exec, FK/algorithms/image_processing/color_conversion.h:219-238: Y at (x,y) of the
  * luma plane; (U,V) at element x>>1 of chroma row y>>1, chroma base = data + pitch*height. */
 static uint16_t load_u16(const uint8_t *p) { uint16_t v; memcpy(&v, p, 2); return v; }
-static int read_is_pixel_format(const fklo_read *r) { return r->kind != FKLO_READ_2D; }
+static int read_is_pixel_format(const fklo_read *r) { return r->kind != FKLO_READ_2D && r->kind != FKLO_READ_PLANAR; }
 static int pixel_format_elem(int kind) {
     return (kind == FKLO_READ_P010 || kind == FKLO_READ_P210 || kind == FKLO_READ_Y210) ? FKLO_U16 : FKLO_U8;
 }
@@ -382,6 +416,19 @@ static void read_source(const fklo_read *r, int x, int y, fklo_val *out) {
     out->elem = r->elem;
     out->cn = r->cn;
     const uint8_t *row = base + (int64_t)y * r->pitch;
+    if (r->kind == FKLO_READ_PLANAR) {
+        /* TensorPack<T>::exec, FK/algorithms/basic_ops/memory_operations.h:243-290 (channel_stride = width*height elements)
+         * and TensorTPack<T>::exec, :292-327 with PtrAccessor<T3D>::cr_point, FK/core/data/rawptr.h:229-235
+         * (channel_stride = color_planes_pitch). */
+        const int64_t esz = r->elem == FKLO_U8 ? 1 : (r->elem == FKLO_U16 ? 2 : 4);
+        for (int c = 0; c < r->cn; ++c) {
+            const uint8_t *p = row + (int64_t)x * esz + (int64_t)c * r->channel_stride;
+            if (r->elem == FKLO_U8) out->u[c] = *p;
+            else if (r->elem == FKLO_U16) out->h[c] = load_u16(p);
+            else memcpy(&out->f[c], p, 4);
+        }
+        return;
+    }
     if (r->elem == FKLO_U8) {
         const uint8_t *p = row + (int64_t)x * r->cn;
         for (int c = 0; c < r->cn; ++c) out->u[c] = p[c];
@@ -544,6 +591,15 @@ static int write_value(const fklo_write *w, int x, int y, int z, const fklo_val 
         return FKLO_OK;
     }
     const int64_t plane_pitch = (int64_t)w->pitch * w->height;
+    if (w->kind == FKLO_TENSOR_TSPLIT) {
+        /* TensorTSplit<T>::exec, FK/algorithms/basic_ops/memory_operations.h:214-241 with PtrAccessor<T3D>::point,
+         * FK/core/data/rawptr.h:236-239: data + c*color_planes_pitch + z*plane_pitch + y*pitch, then x elements;
+         * color_planes_pitch = plane_pitch * planes (ptr_nd.h:119-125). */
+        for (int c = 0; c < w->cn; ++c)
+            memcpy(base + (int64_t)c * plane_pitch * w->planes + plane_pitch * z + (int64_t)y * w->pitch + (int64_t)x * esz,
+                   val_chan(v, c), (size_t)esz);
+        return FKLO_OK;
+    }
     uint8_t *row = base + plane_pitch * w->color_planes * z + (int64_t)y * w->pitch;
     if (w->kind == FKLO_TENSOR_WRITE) {
         uint8_t *p = row + (int64_t)x * esz * w->cn;

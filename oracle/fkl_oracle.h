@@ -44,7 +44,9 @@ enum fklo_read_kind {
     FKLO_READ_P010 = 3, /* ReadYUV<P010>: NV12 layout with 16-bit samples             */
     FKLO_READ_P210 = 4, /* ReadYUV<P210>: 16-bit samples, chroma rows at full height  */
     FKLO_READ_Y210 = 5, /* ReadYUV<Y210>: packed 16-bit Y0 U Y1 V                     */
-    FKLO_READ_UYVY = 6  /* ReadYUV<UYVY>: packed 8-bit U Y0 V Y1                      */
+    FKLO_READ_UYVY = 6, /* ReadYUV<UYVY>: packed 8-bit U Y0 V Y1                      */
+    FKLO_READ_PLANAR = 7 /* TensorPack<T> / TensorTPack<T>: cn channel planes of elem, channel_stride bytes apart;
+                            data = channel 0 of this image plane                        */
 };
 
 enum fklo_aspect { FKLO_PRESERVE_AR = 0, FKLO_IGNORE_AR = 1 };
@@ -63,14 +65,18 @@ enum fklo_opcode {
     FKLO_RGB2GRAY = 11,        /* RGB2Gray<I, O>: idx[0] = element type of O           */
     FKLO_ADD_LAST = 12,        /* one more channel holding p[0] (AddOpaqueAlpha)       */
     FKLO_DISCARD = 13,         /* keep the first idx[0] channels                       */
-    FKLO_SATCAST_U16 = 14      /* float -> ushort: NaN->0, round-half-even, clamp      */
+    FKLO_SATCAST_U16 = 14,     /* float -> ushort: NaN->0, round-half-even, clamp      */
+    FKLO_CLAMP = 15,           /* Saturate<T> / SaturateDepth: (v<p[0]) ? p[0] : ((p[1]<v) ? p[1] : v)       */
+    FKLO_SATURATE_FLOAT = 16,  /* SaturateFloat<T>: fmaxf(0, fminf(v, 1)); NaN -> 1, -0 stays -0            */
+    FKLO_CAST_TRUNC = 17       /* float -> element type idx[0] like a C cast (DenormalizePixel after FKLO_MUL) */
 };
 
 enum fklo_write_kind {
     FKLO_WRITE_2D = 0,      /* PerThreadWrite<_2D,T>; one fklo_write per plane when batched */
     FKLO_TENSOR_WRITE = 1,  /* TensorWrite<T>: AoS, plane z at z*plane_pitch*color_planes   */
     FKLO_TENSOR_SPLIT = 2,  /* TensorSplit<T>: planar, channel c at +c*width*height elems   */
-    FKLO_WRITE_YUV = 3      /* WriteYUV<PF>: yuv_format names the layout (a fklo_read_kind) */
+    FKLO_WRITE_YUV = 3,     /* WriteYUV<PF>: yuv_format names the layout (a fklo_read_kind) */
+    FKLO_TENSOR_TSPLIT = 4  /* TensorTSplit<T>: channel c at +c*pitch*height*planes bytes, plane z at +z*pitch*height */
 };
 
 /* Values of fk::ColorDepth, fk::ColorRange, fk::ColorPrimitives (FK/algorithms/image_processing/itu_color.h:26-29). */
@@ -107,6 +113,7 @@ typedef struct {
     int32_t border;          /* BorderReader between the source and the crop: 0 none, else 1 + fk::BorderType       */
     float border_value[4];   /* (1 CONSTANT, 2 REPLICATE, 3 REFLECT, 4 WRAP, 5 REFLECT_101); CONSTANT's value, typed  */
                              /* like the source element                                                             */
+    int64_t channel_stride;  /* FKLO_READ_PLANAR: bytes from one channel plane to the next                                  */
 } fklo_read;
 
 typedef struct {

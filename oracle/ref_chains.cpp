@@ -398,6 +398,12 @@ int fklref_normalize(int which, const void* src, int w, int h, int pitch, float*
     s.sync();
     return rc;
 }
+int fklref_depth_ops(int which, const void* src, int w, int h, int pitch, void* out, int out_pitch, float lo, float hi) {
+    CpuStream s;
+    const int rc = RefColor::depth_ops(s, MemType::Host, which, src, w, h, pitch, out, out_pitch, lo, hi);
+    s.sync();
+    return rc;
+}
 #ifndef FKL_HARNESS_PUBLIC_API_ONLY
 // ccMatrix<range, primaries, direction, depth> as the reference computes it at compile time, row major.
 // to_rgb = 1 selects YCbCr2RGB.
@@ -434,6 +440,18 @@ int fklref_divergent_mixed(const float* tensor4, int w, int h, float mul, const 
     circular_chains::Chains<ParArch::CPU>::divergent_mixed(s, MemType::Host, tensor4, w, h, mul, img, iw, ih, ipitch, out);
     s.sync();
     return 0;
+}
+int fklref_transposed_round_trip(const uint8_t* const* images, int planes, int w, int h, int pitch, float mul, float* tensor_t, float mul2,
+                                 float* packed) {
+    CpuStream s;
+    circular_chains::Chains<ParArch::CPU>::transposed_round_trip(s, MemType::Host, images, planes, w, h, pitch, mul, tensor_t, mul2, packed);
+    s.sync();
+    return 0;
+}
+int fklref_circular_transposed(int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch, float fill,
+                               float* states) {
+    CpuStream s;
+    return circular_chains::Chains<ParArch::CPU>::circular_transposed(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Host, fill, states);
 }
 int fklref_circular(int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch, float fill, float* states) {
     CpuStream s;

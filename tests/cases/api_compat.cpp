@@ -14,6 +14,7 @@
 #include <fused_kernel/fused_kernel.h>
 #include <fused_kernel/core/execution_model/execution_model.h>
 #include <fused_kernel/algorithms/algorithms.h>
+#include <fused_kernel/core/data/circular_tensor.h>
 
 #include <type_traits>
 
@@ -257,3 +258,14 @@ static_assert(fk::isThreadFusionEnabled<true, fk::Read<fk::PerThreadRead<fk::ND:
 static_assert(!fk::isThreadFusionEnabled<true, fk::Read<fk::PerThreadRead<fk::ND::_2D, float3>>, fk::Write<fk::TensorSplit<float3>>>(),
               "a planar split never fuses threads");
 static_assert(fk::maxValue<uchar> == 255 && fk::minValue<float3>.y == -3.402823466e+38f);
+
+// ---- Depth operations and transposed tensors: the reference's types ---------------------------------------------------
+static_assert(std::is_same_v<fk::DenormalizePixel<uchar3, fk::ColorDepth::p8bit>::InputType, float3> &&
+              std::is_same_v<fk::DenormalizePixel<uchar3, fk::ColorDepth::p8bit>::OutputType, uchar3>);
+static_assert(std::is_same_v<fk::SaturateDenormalizePixel<float4, ushort4, fk::ColorDepth::p10bit>::OutputType, ushort4>);
+static_assert(std::is_same_v<fk::Saturate<float3>::ParamsType, float2> && fk::opIs<fk::BinaryType, decltype(fk::Saturate<float>::build(float2{0.f, 1.f}))>);
+static_assert(fk::opIs<fk::UnaryType, decltype(fk::SaturateDepth<float, fk::ColorDepth::p12bit>::build())>);
+static_assert(std::is_same_v<fk::TensorTSplit<float3>::ParamsType, fk::RawPtr<fk::ND::T3D, float>> &&
+              std::is_same_v<fk::TensorTPack<float3>::OutputType, float3> && !fk::TensorTSplit<float3>::THREAD_FUSION);
+static_assert(std::is_base_of_v<fk::TensorT<float>, fk::CircularTensor<float, 3, 4, fk::CircularTensorOrder::NewestFirst, fk::ColorPlanes::Transposed>> &&
+              std::is_base_of_v<fk::Tensor<float>, fk::CircularTensor<float, 3, 4, fk::CircularTensorOrder::NewestFirst, fk::ColorPlanes::Standard>>);

@@ -57,6 +57,67 @@ template <ParArch PA> struct Chains {
     // The reference's CircularTensor test scenario on caller-supplied images: the tensor starts at `fill`, then every
     // image goes through update(read -> SaturateCast<uchar3, float3> -> TensorSplit); after each update the whole
     // tensor is copied to `states` (iters x BATCH x 3 x h x w floats, host memory).
+    // A transposed tensor over caller-owned memory: planes * 3 channel planes of w x h floats, tightly packed, all first
+    // channel planes first.
+    static PtrT3D<float> wrap_t(const float* data, int w, int h, int planes, MemType mem) {
+        PtrDims<ND::T3D> d(uint(w), uint(h), uint(planes), 3);
+        d.pitch = uint(w) * uint(sizeof(float));
+        d.plane_pitch = d.pitch * uint(h);
+        d.color_planes_pitch = d.plane_pitch * uint(planes);
+        return PtrT3D<float>(const_cast<float*>(data), d, mem, 0);
+    }
+    // uchar3 images -> Cast -> Mul -> TensorTSplit<float3>: image z into plane z of a transposed tensor of `planes` planes
+    // (one launch per image, each through a view of one plane), then the tensor back as float3 pixels * mul2 through
+    // TensorTPack<float3> into an ordinary tensor.
+    static void transposed_round_trip(StreamT& s, MemType mem, const uint8_t* const* images, int planes, int w, int h, int pitch, float mul,
+                                      float* tensor_t, float mul2, float* packed) {
+        const auto t = wrap_t(tensor_t, w, h, planes, mem);
+        for (int z = 0; z < planes; ++z) {
+            const auto in = wrap<uchar3>(images[z], w, h, pitch, mem);
+            auto view = t.ptr();
+            view.data = PtrAccessor<ND::T3D>::point(Point{0, 0, z}, t.ptr());    // plane z; the channel planes keep their distance
+            executeOperations<TransformDPP<PA>>(s, PerThreadRead<ND::_2D, uchar3>::build(in.ptr()), Cast<uchar3, float3>::build(),
+                                                Binary<Mul<float3, float>>{mul}, Write<TensorTSplit<float3>>{view});
+        }
+        Tensor<float3> o(reinterpret_cast<float3*>(packed), uint(w), uint(h), uint(planes), 1, mem, 0);
+        executeOperations<TransformDPP<PA>>(s, Read<TensorTPack<float3>>{t.ptr()}, Binary<Mul<float3, float>>{mul2}, Write<TensorWrite<float3>>{o.ptr()});
+    }
+
+    // circular_one with ColorPlanes::Transposed: update(read -> SaturateCast -> TensorTSplit); `states` has the layout of
+    // circular_one's (iters x BATCH x 3 x h x w), gathered from the transposed window.  Only colour plane 0 is filled
+    // before the first update (the reference's setTo reaches no other plane of a transposed tensor).
+    template <int BATCH, CircularTensorOrder ORDER>
+    static void circular_transposed_one(StreamT& s, const uint8_t* const* images, int iters, int w, int h, int pitch, MemType mem, float fill, float* states) {
+        const uint width = uint(w), height = uint(h);
+        CircularTensor<float, 3, BATCH, ORDER, ColorPlanes::Transposed> window(width, height, mem == MemType::Host ? MemType::Host : defaultMemType);
+        setTo(fill, window, s);
+        const size_t plane = size_t(w) * size_t(h) * 3;
+        for (int i = 0; i < iters; ++i) {
+            const auto in = wrap<uchar3>(images[i], w, h, pitch, mem);
+            window.update(s, Read<PerThreadRead<ND::_2D, uchar3>>{in.ptr()}, Unary<SaturateCast<uchar3, float3>>{},
+                          Write<TensorTSplit<float3>>{window.ptr()});
+            window.download(s);
+            s.sync();
+            const RawPtr<ND::T3D, float> host = mem == MemType::Host ? window.ptr() : window.ptrPinned();
+            for (int z = 0; z < BATCH; ++z)
+                for (int c = 0; c < 3; ++c)
+                    for (int y = 0; y < h; ++y)
+                        std::memcpy(states + (size_t(i) * BATCH + z) * plane + (size_t(c) * h + y) * w,
+                                    PtrAccessor<ND::T3D>::cr_point(Point{0, y, z}, host, uint(c)), size_t(w) * sizeof(float));
+        }
+    }
+    static int circular_transposed(StreamT& s, int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch,
+                                   MemType mem, float fill, float* states) {
+        constexpr auto NF = CircularTensorOrder::NewestFirst, OF = CircularTensorOrder::OldestFirst;
+#define CIRCULAR_CASE(B) case B: if (oldest_first) circular_transposed_one<B, OF>(s, images, iters, w, h, pitch, mem, fill, states); \
+                                 else circular_transposed_one<B, NF>(s, images, iters, w, h, pitch, mem, fill, states); return 0;
+        switch (batch) {
+            CIRCULAR_CASE(2) CIRCULAR_CASE(3) CIRCULAR_CASE(5)
+        default: return 2;
+        }
+#undef CIRCULAR_CASE
+    }
+
     template <int BATCH, CircularTensorOrder ORDER>
     static void circular_one(StreamT& s, const uint8_t* const* images, int iters, int w, int h, int pitch, MemType mem, float fill, float* states) {
         const uint width = uint(w), height = uint(h);

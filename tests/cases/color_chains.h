@@ -184,6 +184,34 @@ template <class DPP, class StreamT> struct Chains {
         }
         return 2;
     }
+
+    // ---- float image -> SaturateDepth / DenormalizePixel / SaturateDenormalizePixel / Saturate / SaturateFloat -> image ----
+    template <class I, class O, class IOp>
+    static void depth_one(StreamT& s, MemType mem, const IOp& iop, const void* src, int w, int h, int pitch, void* out, int out_pitch) {
+        const auto in = wrap<I>(src, w, h, pitch, mem);
+        const auto o = wrap<O>(out, w, h, out_pitch, mem);
+        executeOperations<DPP>(s, PerThreadRead<ND::_2D, I>::build(in.ptr()), iop, PerThreadWrite<ND::_2D, O>::build(o.ptr()));
+    }
+    // which: 0 SaturateDepth<float, p8bit>, 1 SaturateDepth<float, p10bit>, 2 DenormalizePixel<uchar3, p8bit>,
+    // 3 DenormalizePixel<float3, p8bit>, 4 SaturateDenormalizePixel<float3, uchar3, p8bit>,
+    // 5 SaturateDenormalizePixel<float3, ushort3, p10bit>, 6 SaturateFloat<float4>, 7 Saturate<float3>{lo, hi},
+    // 8 DenormalizePixel<ushort3, p12bit>, 9 SaturateDenormalizePixel<float4, uchar4, p8bit>
+    static int depth_ops(StreamT& s, MemType mem, int which, const void* src, int w, int h, int pitch, void* out, int out_pitch, float lo, float hi) {
+        constexpr auto p8 = ColorDepth::p8bit, p10 = ColorDepth::p10bit, p12 = ColorDepth::p12bit;
+        switch (which) {
+        case 0: depth_one<float, float>(s, mem, SaturateDepth<float, p8>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 1: depth_one<float, float>(s, mem, SaturateDepth<float, p10>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 2: depth_one<float3, uchar3>(s, mem, DenormalizePixel<uchar3, p8>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 3: depth_one<float3, float3>(s, mem, DenormalizePixel<float3, p8>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 4: depth_one<float3, uchar3>(s, mem, SaturateDenormalizePixel<float3, uchar3, p8>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 5: depth_one<float3, ushort3>(s, mem, SaturateDenormalizePixel<float3, ushort3, p10>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 6: depth_one<float4, float4>(s, mem, SaturateFloat<float4>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 7: depth_one<float3, float3>(s, mem, Saturate<float3>::build(make_<float2>(lo, hi)), src, w, h, pitch, out, out_pitch); return 0;
+        case 8: depth_one<float3, ushort3>(s, mem, DenormalizePixel<ushort3, p12>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        case 9: depth_one<float4, uchar4>(s, mem, SaturateDenormalizePixel<float4, uchar4, p8>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        default: return 2;
+        }
+    }
 };
 
 } // namespace color_chains

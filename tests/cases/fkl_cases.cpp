@@ -502,6 +502,9 @@ int fklcase_convert_code(void* stream_, int which, const void* src, int w, int h
 int fklcase_normalize(void* stream_, int which, const void* src, int w, int h, int pitch, float* out, int out_pitch) {
     return guarded_rc([&] { Stream s(stream_); return GpuColor::normalize(s, MemType::Device, which, src, w, h, pitch, out, out_pitch); });
 }
+int fklcase_depth_ops(void* stream_, int which, const void* src, int w, int h, int pitch, void* out, int out_pitch, float lo, float hi) {
+    return guarded_rc([&] { Stream s(stream_); return GpuColor::depth_ops(s, MemType::Device, which, src, w, h, pitch, out, out_pitch, lo, hi); });
+}
 
 } // extern "C"
 
@@ -530,6 +533,24 @@ int fklcase_circular(void* stream_, int batch, int oldest_first, const uint8_t* 
     const int g = guarded([&] {
         Stream s(stream_);
         rc = circular_chains::Chains<ParArch::GPU_AMD>::circular(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Device, fill, states);
+    });
+    return g ? g : rc;
+}
+// images: `planes` device pointers to uchar3 images; tensor_t (planes x 3 channel planes, transposed) and packed
+// (planes x h x w float3) are device memory
+int fklcase_transposed_round_trip(void* stream_, const uint8_t* const* images, int planes, int w, int h, int pitch, float mul, float* tensor_t,
+                                  float mul2, float* packed) {
+    return guarded([&] {
+        Stream s(stream_);
+        circular_chains::Chains<ParArch::GPU_AMD>::transposed_round_trip(s, MemType::Device, images, planes, w, h, pitch, mul, tensor_t, mul2, packed);
+    });
+}
+int fklcase_circular_transposed(void* stream_, int batch, int oldest_first, const uint8_t* const* images, int iters, int w, int h, int pitch,
+                                float fill, float* states) {
+    int rc = 0;
+    const int g = guarded([&] {
+        Stream s(stream_);
+        rc = circular_chains::Chains<ParArch::GPU_AMD>::circular_transposed(s, batch, oldest_first, images, iters, w, h, pitch, MemType::Device, fill, states);
     });
     return g ? g : rc;
 }

@@ -257,6 +257,12 @@ def normalize(which, src, out):
     _ok(cases().fklcase_normalize(_stream(), int(which), _p(src), src.shape[1], src.shape[0], _pitch(src), _p(out), _pitch(out)))
 
 
+def depth_ops(which, src, out, lo=0.0, hi=1.0):
+    """Operation number `which` of depth_ops in tests/cases/color_chains.h on src (H,W[,cn]) f32 cuda -> out cuda."""
+    _ok(cases().fklcase_depth_ops(_stream(), int(which), _p(src), src.shape[1], src.shape[0], _pitch(src), _p(out), _pitch(out),
+                                  C.c_float(float(lo)), C.c_float(float(hi))))
+
+
 def pad(src, border_type, left, top, out, value=(0, 0, 0)):
     """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out."""
     v = np.zeros(4, np.float32)
@@ -286,6 +292,24 @@ def circular(batch, oldest_first, images, fill):
     ptrs = (C.c_void_p * len(images))(*[i.data_ptr() for i in images])
     _ok(cases().fklcase_circular(_stream(), int(batch), int(bool(oldest_first)), ptrs, len(images), w, h, _pitch(images[0]), C.c_float(float(fill)),
                                  states.ctypes.data_as(C.c_void_p)))
+    return states
+
+
+def transposed_round_trip(images, mul, tensor_t, mul2, packed):
+    """images: list of (H,W,3) u8 cuda; tensor_t (3, planes, H, W) f32 cuda; packed (planes, H, W, 3) f32 cuda."""
+    h, w = images[0].shape[:2]
+    ptrs = (C.c_void_p * len(images))(*[i.data_ptr() for i in images])
+    _ok(cases().fklcase_transposed_round_trip(_stream(), ptrs, len(images), w, h, _pitch(images[0]), C.c_float(float(mul)), _p(tensor_t),
+                                              C.c_float(float(mul2)), _p(packed)))
+
+
+def circular_transposed(batch, oldest_first, images, fill):
+    """circular() with ColorPlanes::Transposed and TensorTSplit; same result layout."""
+    h, w = images[0].shape[:2]
+    states = np.zeros((len(images), batch, 3, h, w), np.float32)
+    ptrs = (C.c_void_p * len(images))(*[i.data_ptr() for i in images])
+    _ok(cases().fklcase_circular_transposed(_stream(), int(batch), int(bool(oldest_first)), ptrs, len(images), w, h, _pitch(images[0]),
+                                            C.c_float(float(fill)), states.ctypes.data_as(C.c_void_p)))
     return states
 
 

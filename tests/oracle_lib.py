@@ -15,11 +15,11 @@ ORACLE_SO = os.path.join(ROOT, "oracle", "libfkl_oracle.so")
 REF_SO = os.path.join(ROOT, "oracle", "_ref", "libfkl_ref.so")
 
 U8, F32, U16 = 0, 1, 2
-READ_2D, READ_NV12, READ_NV21, READ_P010, READ_P210, READ_Y210, READ_UYVY = 0, 1, 2, 3, 4, 5, 6
+READ_2D, READ_NV12, READ_NV21, READ_P010, READ_P210, READ_Y210, READ_UYVY, READ_PLANAR = 0, 1, 2, 3, 4, 5, 6, 7
 PRESERVE_AR, IGNORE_AR = 0, 1
 MUL, ADD, SUB, DIV, REORDER, SATCAST_U8, CAST_F32, YUV2RGB_709_FULL = 1, 2, 3, 4, 5, 6, 7, 8
-YUV2RGB, RGB2YUV, RGB2GRAY, ADD_LAST, DISCARD, SATCAST_U16 = 9, 10, 11, 12, 13, 14
-WRITE_2D, TENSOR_WRITE, TENSOR_SPLIT, WRITE_YUV = 0, 1, 2, 3
+YUV2RGB, RGB2YUV, RGB2GRAY, ADD_LAST, DISCARD, SATCAST_U16, CLAMP, SATURATE_FLOAT, CAST_TRUNC = 9, 10, 11, 12, 13, 14, 15, 16, 17
+WRITE_2D, TENSOR_WRITE, TENSOR_SPLIT, WRITE_YUV, TENSOR_TSPLIT = 0, 1, 2, 3, 4
 
 # fk::PixelFormat / ColorDepth / ColorRange / ColorPrimitives enumerator values, and what the oracle calls each format
 PF_NV12, PF_NV21, PF_P010, PF_P210, PF_Y210, PF_UYVY = 0, 1, 3, 6, 8, 10
@@ -58,6 +58,7 @@ class Read(C.Structure):
         ("warp", C.c_int32), ("warp_m", C.c_float * 9),
         ("deinterlace", C.c_int32),
         ("border", C.c_int32), ("border_value", C.c_float * 4),
+        ("channel_stride", C.c_int64),
     ]
 
 
@@ -264,7 +265,7 @@ def write(kind, a: np.ndarray, cn: int, width: int, height: int, planes: int = 1
     w.width, w.height, w.planes, w.color_planes = width, height, planes, color_planes
     esz = a.dtype.itemsize
     if pitch is None:
-        pitch = width * esz * (1 if kind == TENSOR_SPLIT else cn)
+        pitch = width * esz * (1 if kind in (TENSOR_SPLIT, TENSOR_TSPLIT) else cn)
     w.pitch = int(pitch)
     return w
 
@@ -643,6 +644,90 @@ def ref_normalize(which, src):
     rc = ref().fklref_normalize(which, C.c_void_p(_ptr(src)), w, h, src.strides[0], C.c_void_p(_ptr(out)), out.strides[0])
     assert rc == 0, rc
     return out
+
+
+# ---- SaturateDepth / DenormalizePixel / SaturateDenormalizePixel / SaturateFloat / Saturate -----------------------------
+# which -> (input channels, output dtype, oracle operations given (lo, hi)); the list of tests/cases/color_chains.h
+DEPTH_OPS = {
+    0: (1, np.float32, lambda lo, hi: [op(CLAMP, [0.0, 255.0])]),
+    1: (1, np.float32, lambda lo, hi: [op(CLAMP, [0.0, 1023.0])]),
+    2: (3, np.uint8, lambda lo, hi: [op(MUL, [255.0]), op(CAST_TRUNC, idx=(U8, 0, 0, 0))]),
+    3: (3, np.float32, lambda lo, hi: [op(MUL, [255.0]), op(CAST_TRUNC, idx=(F32, 0, 0, 0))]),
+    4: (3, np.uint8, lambda lo, hi: [op(SATURATE_FLOAT), op(MUL, [255.0]), op(CAST_TRUNC, idx=(U8, 0, 0, 0))]),
+    5: (3, np.uint16, lambda lo, hi: [op(SATURATE_FLOAT), op(MUL, [1023.0]), op(CAST_TRUNC, idx=(U16, 0, 0, 0))]),
+    6: (4, np.float32, lambda lo, hi: [op(SATURATE_FLOAT)]),
+    7: (3, np.float32, lambda lo, hi: [op(CLAMP, [lo, hi])]),
+    8: (3, np.uint16, lambda lo, hi: [op(MUL, [4095.0]), op(CAST_TRUNC, idx=(U16, 0, 0, 0))]),
+    9: (4, np.uint8, lambda lo, hi: [op(SATURATE_FLOAT), op(MUL, [255.0]), op(CAST_TRUNC, idx=(U8, 0, 0, 0))]),
+}
+
+
+def _depth_out(which, src):
+    cn, dt, _ = DEPTH_OPS[which]
+    h, w = src.shape[:2]
+    return np.zeros((h, w, cn) if cn > 1 else (h, w), dt)
+
+
+def oracle_depth_ops(which, src, lo=0.0, hi=1.0):
+    """src (H,W,cn) or (H,W) float32."""
+    cn, _, make = DEPTH_OPS[which]
+    out = _depth_out(which, src)
+    execute([read_2d(src, cn)], make(lo, hi), [write(WRITE_2D, out, cn, src.shape[1], src.shape[0])])
+    return out
+
+
+def ref_depth_ops(which, src, lo=0.0, hi=1.0):
+    out = _depth_out(which, src)
+    rc = ref().fklref_depth_ops(which, C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], C.c_void_p(_ptr(out)), out.strides[0],
+                                C.c_float(lo), C.c_float(hi))
+    assert rc == 0, rc
+    return out
+
+
+# ---- transposed tensors: TensorTSplit / TensorTPack --------------------------------------------------------------------
+
+def oracle_transposed_round_trip(images, mul, mul2):
+    """images: list of (H,W,3) u8.  Returns (tensor_t (3, planes, H, W) f32, packed (planes, H, W, 3) f32): image z -> Cast ->
+    Mul -> TensorTSplit into plane z, then TensorTPack -> Mul -> TensorWrite."""
+    planes = len(images)
+    h, w = images[0].shape[:2]
+    tensor_t = np.zeros((3, planes, h, w), np.float32)
+    for z, img in enumerate(images):
+        view = tensor_t[:, z:]                       # plane z first; channel planes stay planes * h * w elements apart
+        wr = write(TENSOR_TSPLIT, view, 3, w, h, planes, 3)
+        execute([read_2d(img, 3)], [op(CAST_F32), op(MUL, [mul])], [wr])
+    packed = np.zeros((planes, h, w, 3), np.float32)
+    reads = []
+    for z in range(planes):
+        r = Read()
+        r.kind, r.elem, r.cn, r.width, r.height, r.pitch = READ_PLANAR, F32, 3, w, h, w * 4
+        r.data = _ptr(tensor_t[0, z])
+        r.channel_stride = tensor_t.strides[0]
+        reads.append(r)
+    execute(reads, [op(MUL, [mul2])], [write(TENSOR_WRITE, packed, 3, w, h, planes, 1)])
+    return tensor_t, packed
+
+
+def ref_transposed_round_trip(images, mul, mul2):
+    planes = len(images)
+    h, w = images[0].shape[:2]
+    tensor_t = np.zeros((3, planes, h, w), np.float32)
+    packed = np.zeros((planes, h, w, 3), np.float32)
+    ptrs = (C.c_void_p * planes)(*[_ptr(i) for i in images])
+    rc = ref().fklref_transposed_round_trip(ptrs, planes, w, h, images[0].strides[0], C.c_float(mul), C.c_void_p(_ptr(tensor_t)), C.c_float(mul2),
+                                            C.c_void_p(_ptr(packed)))
+    assert rc == 0, rc
+    return tensor_t, packed
+
+
+def ref_circular_transposed(batch, oldest_first, images, fill):
+    h, w = images[0].shape[:2]
+    states = np.zeros((len(images), batch, 3, h, w), np.float32)
+    ptrs = (C.c_void_p * len(images))(*[_ptr(i) for i in images])
+    rc = ref().fklref_circular_transposed(batch, int(bool(oldest_first)), ptrs, len(images), w, h, images[0].strides[0], C.c_float(fill),
+                                          C.c_void_p(_ptr(states)))
+    assert rc == 0, rc
+    return states
 
 
 # ---- padding through BorderReader ---------------------------------------------------------------------------

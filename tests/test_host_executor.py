@@ -13,6 +13,7 @@ import oracle_lib as ol
 import test_oracle as t_core
 import test_oracle_border as t_border
 import test_oracle_color as t_color
+import test_oracle_depth_and_transposed as t_depth
 import test_oracle_window as t_window
 
 pytestmark = pytest.mark.skipif(not ol.have_hostexec(), reason="oracle/libfkl_hostexec.so not built (make -C oracle hostexec)")
@@ -97,3 +98,19 @@ def test_circular_window(batch, oldest_first):
 
 def test_divergent_launches():
     on_host_executor(t_window.test_divergent_launches_match_reference_backend)
+
+
+@pytest.mark.parametrize("which", sorted(ol.DEPTH_OPS))
+def test_depth_operations(which):
+    on_host_executor(t_depth.test_depth_operations_match_reference_backend, which)
+
+
+def test_transposed_tensor():
+    on_host_executor(t_depth.test_transposed_tensor_matches_reference_backend, 3, 10, 6)
+    on_host_executor(t_depth.test_transposed_tensor_matches_reference_backend, 4, 33, 5)
+
+
+@pytest.mark.parametrize("batch", [2, 5])
+@pytest.mark.parametrize("oldest_first", [False, True])
+def test_transposed_window(batch, oldest_first):
+    on_host_executor(t_depth.test_transposed_window_matches_reference_backend, batch, oldest_first)
