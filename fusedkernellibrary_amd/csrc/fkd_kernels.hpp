@@ -228,45 +228,18 @@ inline u32 division_magic(u32 d, u32 limit) {
 // ignored); neighbouring lanes and rows hit the same cache lines, so HBM sees each source line about once.
 // All loads of a lane are issued before the first use and are unconditional (coordinates are clamped into the
 // source); only stores are predicated.
-template <class Chain, int XI, int YI>
-__device__ __forceinline__ void gather_body(const typename Chain::Params& p, const TileGeom& g) {
+// The tile's work once the plane's parameters are in registers: q (the plane's read), ops, wpar (the plane's write), the
+// output extent aw x ah, the plane z, the tile's first column tx0 and its row of tiles.
+template <class Chain, int XI, int YI, class Q, class OPS, class WPAR>
+__device__ __forceinline__ void gather_tile(const typename Chain::Params& p, const Q& q, const OPS& ops, const WPAR& wpar,
+                                            int aw, int ah, int z, int tx0, u32 tile_row) {
     using Root = ResizeRoot<typename Chain::Read>;
     using RZ = typename Root::Resize;
     using Back = typename RZ::BackOp;
     using Raw = typename Back::Raw;
     using W = typename Chain::Write;
-    constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
-
-    // The plane is the grid's z index, known at wave start, so the plane's parameters are fetched together with the
-    // first kernel arguments instead of after them.  Within a plane workgroups are renumbered: hardware deals
-    // consecutive workgroup ids round-robin to the 8 XCDs (the grid's x extent is a multiple of 8); XCD k gets the
-    // k-th contiguous eighth of the plane's tiles so neighbouring tiles (which share source rows) share an L2.
-    const int z = int(blockIdx.z);
-    // Everything the wave needs from the kernel-argument segment, fetched in one go.
-    const typename RZ::Params* rp;
-    if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
     using WP = typename W::Plane;
-    // A scalar load from the kernel-argument segment takes several hundred cycles, and a wave that lives for a few
-    // thousand cannot afford one round trip per first use: geometry, the plane's read parameters, the operations'
-    // parameters and the write's are requested back to back and waited for once.
-    TileGeom gg = g;
-    typename RZ::Params q = *rp;
-    typename Chain::OpParams ops = p.ops;
-    typename WP::Params wpar = W::plane_params(p.write, z);
-    detail::pin_scalars(gg);
-    detail::pin_scalars(q);
-    detail::pin_scalars(ops);
-    detail::pin_scalars(wpar);
-    u32 dims[2] = {p.active_w, p.active_h};
-    asm volatile("" : "+s"(dims[0]), "+s"(dims[1]));
-    const int aw = int(dims[0]), ah = int(dims[1]);
-
-    const u32 per_plane = gg.tiles_x * gg.tiles_y;
-    const u32 chunk = (per_plane + 7u) / 8u;
-    const u32 tin = (blockIdx.x % 8u) * chunk + blockIdx.x / 8u;
-    if (tin >= per_plane) return;
-    const u32 tile_row = gg.tiles_x_magic ? u32(((unsigned long long)tin * gg.tiles_x_magic) >> 32) : tin / gg.tiles_x;
-    const int tx0 = int(tin - tile_row * gg.tiles_x) * TW;
+    constexpr int TH = kGatherBY * YI;
     const int wy = __builtin_amdgcn_readfirstlane(int(threadIdx.y));
     const int y0 = int(tile_row) * TH + wy * YI;
     if (y0 >= ah) return;
@@ -541,6 +514,251 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
 }
 
 template <class Chain, int XI, int YI>
+__device__ __forceinline__ void gather_body(const typename Chain::Params& p, const TileGeom& g) {
+    using Root = ResizeRoot<typename Chain::Read>;
+    using RZ = typename Root::Resize;
+    using W = typename Chain::Write;
+    using WP = typename W::Plane;
+    constexpr int TW = kGatherBX * XI;
+    // The plane is the grid's z index, known at wave start, so the plane's parameters are fetched together with the
+    // first kernel arguments instead of after them.  Within a plane workgroups are renumbered: hardware deals
+    // consecutive workgroup ids round-robin to the 8 XCDs (the grid's x extent is a multiple of 8); XCD k gets the
+    // k-th contiguous eighth of the plane's tiles so neighbouring tiles (which share source rows) share an L2.
+    const int z = int(blockIdx.z);
+    const typename RZ::Params* rp;
+    if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
+    // A scalar load from the kernel-argument segment takes several hundred cycles, and a wave that lives for a few
+    // thousand cannot afford one round trip per first use: geometry, the plane's read parameters, the operations'
+    // parameters and the write's are requested back to back and waited for once.
+    TileGeom gg = g;
+    typename RZ::Params q = *rp;
+    typename Chain::OpParams ops = p.ops;
+    typename WP::Params wpar = W::plane_params(p.write, z);
+    detail::pin_scalars(gg);
+    detail::pin_scalars(q);
+    detail::pin_scalars(ops);
+    detail::pin_scalars(wpar);
+    u32 dims[2] = {p.active_w, p.active_h};
+    asm volatile("" : "+s"(dims[0]), "+s"(dims[1]));
+    const int aw = int(dims[0]), ah = int(dims[1]);
+
+    const u32 per_plane = gg.tiles_x * gg.tiles_y;
+    const u32 chunk = (per_plane + 7u) / 8u;
+    const u32 tin = (blockIdx.x % 8u) * chunk + blockIdx.x / 8u;
+    if (tin >= per_plane) return;
+    const u32 tile_row = gg.tiles_x_magic ? u32(((unsigned long long)tin * gg.tiles_x_magic) >> 32) : tin / gg.tiles_x;
+    const int tx0 = int(tin - tile_row * gg.tiles_x) * TW;
+    gather_tile<Chain, XI, YI>(p, q, ops, wpar, aw, ah, z, tx0, tile_row);
+}
+
+// ---- strip form of the bilinear kernel: narrow outputs (batches of small planes) -------------------------------------
+//
+// A workgroup of four waves owns 8 whole output rows of one plane, up to 256 pixels wide.  A HALF wave (32 lanes) owns
+// one row and each lane the columns lane, lane + 32, lane + 64, ...: a 224-pixel row is seven such steps with no idle
+// lane, where 128-pixel tiles leave one lane in eight without work.  What depends on the column (horizontal weights,
+// the byte offset of the tap window and the bytes to drop from it) is worked out ONCE per workgroup, one column per
+// thread, and handed round through 4 KB of LDS; what depends on the row is worked out once per lane and serves all its
+// pixels.  So the fixed work of a wave is spread over seven pixels per lane instead of four, nearly all of it on the
+// vector unit (the scalar unit is shared by the four SIMDs of a compute unit and was as busy as they were).
+// What the form asks of every plane -- source rows that share their alignment (pitch a multiple of 4), source smaller
+// than 4 GB and at least two columns wide, output plane smaller than 2 GB -- is checked on the host when the parameter
+// block is made (Chain::finalize_write, bit 0 of Params::reserved); launchers take the tile form when the bit is clear.
+// Taps come through a buffer resource whose extent ends with the image, so windows that reach past the last row read
+// zeros in bytes nobody uses and no lane needs a narrower access; the row is part of the lane's offset.
+#ifndef FKD_STRIP_DEPTH
+#define FKD_STRIP_DEPTH 1
+#endif
+constexpr int kStripRows = kGatherBY * FKD_GATHER_YI, kStripStep = 32, kStripMaxWidth = 256, kStripDepth = FKD_STRIP_DEPTH;
+constexpr int kStripThreads = kStripRows * kStripStep;
+static_assert(kStripThreads == kGatherBX * kGatherBY, "the two forms of the bilinear kernel share their workgroup shape");
+
+template <class Chain> constexpr bool strip_capable() {
+    using Root = ResizeRoot<typename Chain::Read>;
+    if constexpr (!Root::value) return false;
+    else if constexpr (HasDefaultPlanes<typename Chain::Read>::value) return false;
+    else {
+        using Back = typename Root::Resize::BackOp;
+        using WP = typename Chain::Write::Plane;
+        if constexpr (!detail::tap_prepared<Back>()) return false;
+        else if constexpr (!Back::kTapPair) return false;
+        else if constexpr (requires { WP::kLaneMasked; }) return WP::kLaneMasked;
+        else return false;
+    }
+}
+
+template <class Chain>
+__device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
+    using Root = ResizeRoot<typename Chain::Read>;
+    using RZ = typename Root::Resize;
+    using Back = typename RZ::BackOp;
+    using Raw = typename Back::Raw;
+    using W = typename Chain::Write;
+    using WP = typename W::Plane;
+    constexpr int D = kStripDepth;
+    constexpr int kEntries = kStripMaxWidth + (D + 1) * kStripStep;
+    // per column: ax, bx, window offset, bytes to drop from the window (bits 0-1) | flags
+    __shared__ detail::u32x4_t column[kEntries];
+    __shared__ u32 any_clamped;
+    constexpr u32 kClamped = 0x80000000u, kOutsideX = 0x40000000u;
+
+    const int z = int(blockIdx.z);
+    const typename RZ::Params* rp;
+    if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
+    typename RZ::Params q = *rp;
+    typename Chain::OpParams ops = p.ops;
+    typename WP::Params wpar = W::plane_params(p.write, z);
+    detail::pin_scalars(q);
+    detail::pin_scalars(ops);
+    detail::pin_scalars(wpar);
+    u32 dims[2] = {p.active_w, p.active_h};
+    asm volatile("" : "+s"(dims[0]), "+s"(dims[1]));
+    const int aw = int(dims[0]), ah = int(dims[1]);
+    int ox = 0, oy = 0;
+    if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; }
+    const int sw = Back::width(q.back), sh = Back::height(q.back);
+    const detail::TapImage image = Back::tap_image_bounded(z, q.back);
+    const int steps = (aw + kStripStep - 1) / kStripStep;
+
+    const int t = int(threadIdx.y) * 64 + int(threadIdx.x);
+    // ---- the column table: one column per thread and pass; the D + 1 steps after the last one hold a window offset
+    // beyond the image's extent, so requesting them touches no memory ----
+    if (t == 0) any_clamped = 0u;
+    __syncthreads();
+    for (int col = t; col < (steps + D + 1) * kStripStep; col += kStripThreads) {
+        detail::u32x4_t e;
+        bool clamped = false;
+        if (col < steps * kStripStep) {
+            const int x = col < aw ? col : aw - 1;
+            const f32 sx = f32(x - ox) * q.fx;
+            const f32 f1 = __builtin_floorf(sx);
+            const f32 ax = (f1 + 1.0f) - sx, bx = sx - f1;
+            const int xi = int(f1);
+            const int x1 = xi < 0 ? 0 : (xi < sw - 1 ? xi : sw - 1);
+            clamped = x1 + 1 > sw - 1;                                  // right tap is the last column again
+            const detail::PairPrep pp = Back::pair_prepare(image, x1 - int(clamped), q.back);
+            u32 flags = pp.shift | (clamped ? kClamped : 0u);
+            if constexpr (RZ::kAR != IGNORE_AR) flags |= (x >= q.x1 && x <= q.x2) ? 0u : kOutsideX;
+            e.x = __builtin_bit_cast(u32, ax); e.y = __builtin_bit_cast(u32, bx); e.z = pp.off; e.w = flags;
+        } else {
+            e.x = 0u; e.y = 0u; e.z = 0xfffffff0u; e.w = 0u;
+        }
+        column[col] = e;
+        if (__builtin_amdgcn_ballot_w64(clamped) != 0ull && threadIdx.x == 0) any_clamped = 1u;
+    }
+    __syncthreads();
+    const bool some_clamped = __builtin_amdgcn_readfirstlane(any_clamped) != 0u;
+
+    // ---- the lane's row ----
+    const int g = t & (kStripStep - 1), r = t >> 5;
+    const int y = int(blockIdx.x) * kStripRows + r;
+    const bool yvalid = y < ah;
+    const int yc = yvalid ? y : ah - 1;
+    const f32 sy = f32(yc - oy) * q.fy;
+    const f32 fy1 = __builtin_floorf(sy);
+    const f32 ay = (fy1 + 1.0f) - sy, by = sy - fy1;
+    const int yi = int(fy1);
+    const int ya = yi < 0 ? 0 : (yi < sh - 1 ? yi : sh - 1);
+    const int yb = ya + 1 < sh - 1 ? ya + 1 : sh - 1;
+    const u32 row_a = Back::tap_row_offset(ya, q.back), row_b = Back::tap_row_offset(yb, q.back);
+    bool yin = true;
+    if constexpr (RZ::kAR != IGNORE_AR) yin = yc >= q.y1 && yc <= q.y2;
+    const auto oplane = WP::plane_ref(z, wpar);
+    // the lane's store offset in step 0; a lane without a row carries an offset beyond the resource's extent
+    const u32 out0 = yvalid ? WP::row_offset(y, oplane) + WP::lane_offset(g, true) : WP::kMaskedOut;
+    const bool partial = (aw & (kStripStep - 1)) != 0;             // the last step has columns beyond the output
+
+    struct StepTaps { detail::u32x4_t e; typename Back::PairBits ab, cd; };
+    auto request = [&](int k, StepTaps& s) {
+        s.e = column[g + kStripStep * k];
+        // (v_alignbyte_b32 takes the bytes to drop from bits 0-1 of its operand, so the flags may ride along)
+        detail::PairPrep pa, pb;
+        pa.off = s.e.z + row_a; pa.shift = s.e.w;
+        pb.off = s.e.z + row_b; pb.shift = s.e.w;
+        s.ab = Back::pair_load_prepared(image, 0u, pa, q.back);
+        s.cd = Back::pair_load_prepared(image, 0u, pb, q.back);
+    };
+    auto run = [&](auto static_tag, auto clamp_tag) {
+        constexpr bool STATIC = decltype(static_tag)::value != 0;
+        constexpr bool CLAMP = decltype(clamp_tag)::value != 0;
+        auto produce = [&](int k, const StepTaps& s, bool beyond) {
+            // (the words are copied out first: a bit cast applied directly to an element of the vector reads element 0)
+            const u32 ax_bits = s.e.x, bx_bits = s.e.y;
+            const f32 ax = __builtin_bit_cast(f32, ax_bits), bx = __builtin_bit_cast(f32, bx_bits);
+            typename RZ::Taps tp;
+            tp.w00 = ax * ay; tp.w10 = bx * ay; tp.w01 = ax * by; tp.w11 = bx * by;
+            Raw a, b, c, d;
+            Back::pair_values(s.ab, typename Back::TapRow{}, 0, a, b);
+            Back::pair_values(s.cd, typename Back::TapRow{}, 0, c, d);
+            if constexpr (CLAMP) { if (s.e.w & kClamped) { a = b; c = d; } }
+            typename RZ::Out v = RZ::blend(Back::finish(a, q.back), Back::finish(b, q.back),
+                                           Back::finish(c, q.back), Back::finish(d, q.back), tp);
+            if constexpr (RZ::kAR != IGNORE_AR) { if (!yin || (s.e.w & kOutsideX)) v = q.bg; }
+            typename Chain::Value res;
+            if constexpr (STATIC) res = Chain::compute_static_ops(v, ops);
+            else res = Chain::compute_checked_ops(v, ops);
+            u32 off = out0 + u32(k) * WP::lane_offset(kStripStep, true);
+            if (beyond) off = WP::kMaskedOut;                         // a step of the prologue that does not exist
+            if (partial && k == steps - 1) {                          // wave uniform, kept a branch
+                asm volatile("" : "+v"(off));
+                if (g + kStripStep * k >= aw) off = WP::kMaskedOut;
+            }
+            WP::put_masked(oplane, 0u, off, res);
+        };
+        // D steps of taps are in flight behind the step being blended.  Every pass through the loop issues the same
+        // accesses in the same order as the prologue did, and the only branches leave the loop: the compiler's wait for
+        // a step's taps can then leave all later accesses in flight.  (Written out per depth with named tap sets: with
+        // an array of sets the compiler rotates registers instead, and a copy of a register waits for its load.)
+        if constexpr (D == 1) {
+            StepTaps s0, s1;
+            request(0, s0);
+            request(1, s1);
+            produce(0, s0, false);
+#pragma unroll 1
+            for (int k = 1; k < steps; k += 2) {
+                request(k + 1, s0);
+                produce(k, s1, false);
+                if (k + 1 >= steps) break;
+                request(k + 2, s1);
+                produce(k + 1, s0, false);
+            }
+        } else {
+            static_assert(D == 2, "depths 1 and 2 are written out");
+            StepTaps s0, s1, s2;
+            request(0, s0);
+            request(1, s1);
+            request(2, s2);
+            produce(0, s0, false);
+            request(3, s0);
+            produce(1, s1, steps < 2);
+#pragma unroll 1
+            for (int k = 2; k < steps; k += 3) {
+                request(k + 2, s1);
+                produce(k, s2, false);
+                if (k + 1 >= steps) break;
+                request(k + 3, s2);
+                produce(k + 1, s0, false);
+                if (k + 2 >= steps) break;
+                request(k + 4, s0);
+                produce(k + 2, s1, false);
+            }
+        }
+    };
+    auto run_static = [&](auto static_tag) {
+        if (some_clamped) run(static_tag, IntTag<1>{});
+        else run(static_tag, IntTag<0>{});
+    };
+    if constexpr (Chain::kQuick) {
+        if (Chain::ops_static(ops)) { run_static(IntTag<1>{}); return; }
+    }
+    run_static(IntTag<0>{});
+}
+
+template <class Chain>
+__global__ __launch_bounds__(kStripThreads) void k_strip(const typename Chain::Params p) {
+    if constexpr (strip_capable<Chain>()) strip_body<Chain>(p);
+}
+
+template <class Chain, int XI, int YI>
 __global__ __launch_bounds__(kGatherBX * kGatherBY) void k_gather(const typename Chain::Params p, const TileGeom g) {
     gather_body<Chain, XI, YI>(p, g);
 }
@@ -551,14 +769,20 @@ template <class Chain> struct RowsConfig {
     // Four elements per thread wherever the chain reads rows; a bilinear read without a tap cursor keeps one
     // element per thread (its taps are gathers, wider threads would only spread them further apart).
     static constexpr bool kScattered = ResizeRoot<typename Chain::Read>::value || is_scattered_read<typename Chain::Read>();
-    static constexpr int V = kScattered ? 1 : 4;
 #ifndef FKD_ROWS
 #define FKD_ROWS 2
 #endif
+#ifndef FKD_SCATTER_V
+#define FKD_SCATTER_V 1
+#endif
+#ifndef FKD_SCATTER_ROWS
+#define FKD_SCATTER_ROWS 1
+#endif
+    static constexpr int V = kScattered ? FKD_SCATTER_V : 4;
     // Two rows per thread; chains long enough to be bound by instruction issue rather than by memory (more than 128
     // bytes of operation parameters) take four, for the independent work per thread.
     static constexpr bool kManyOps = sizeof(typename Chain::Params) - sizeof(typename Chain::Read::Params) - sizeof(typename Chain::Write::Params) > 128 + 16;
-    static constexpr int ROWS = kScattered ? 1 : (kManyOps ? 2 * FKD_ROWS : FKD_ROWS);
+    static constexpr int ROWS = kScattered ? FKD_SCATTER_ROWS : (kManyOps ? 2 * FKD_ROWS : FKD_ROWS);
 };
 
 // ---- divergent batch kernel -------------------------------------------------------------------------------
@@ -608,17 +832,24 @@ struct JitMeta {
     u32 v, rows;         // rows kernel: elements per thread along x, rows per thread
     u32 xi, yi, by;      // gather kernel: pixels per lane along x, rows per wave, waves per workgroup
     u32 max_planes;      // most planes (grid z) a launch may have, 0: no limit of the kernel's own
+    u32 strip_width;     // gather kernel: outputs up to this width are launched in strip form (TileGeom all zero), 0: never
 };
 template <class Chain> constexpr JitMeta jit_meta() {
     if constexpr (IsDivergent<Chain>::value)
-        return JitMeta{0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V), u32(RowsConfig<Chain>::ROWS), 0u, 0u, 0u, u32(Chain::kMaxPlanes)};
+        return JitMeta{0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V), u32(RowsConfig<Chain>::ROWS), 0u, 0u, 0u, u32(Chain::kMaxPlanes), 0u};
     else
         return JitMeta{is_gather_chain<Chain>() ? 1u : 0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V),
-                       u32(RowsConfig<Chain>::ROWS), u32(FKD_GATHER_XI), u32(FKD_GATHER_YI), u32(kGatherBY), 0u};
+                       u32(RowsConfig<Chain>::ROWS), u32(FKD_GATHER_XI), u32(FKD_GATHER_YI), u32(kGatherBY), 0u,
+                       is_gather_chain<Chain>() && strip_capable<Chain>() ? u32(kStripMaxWidth) : 0u};
 }
 template <class Chain> __device__ __forceinline__ void jit_body(const typename Chain::Params& p, const TileGeom& g) {
     if constexpr (IsDivergent<Chain>::value) DivergentBody<Chain>::run(p);
-    else if constexpr (is_gather_chain<Chain>()) gather_body<Chain, FKD_GATHER_XI, FKD_GATHER_YI>(p, g);
+    else if constexpr (is_gather_chain<Chain>()) {
+        if constexpr (strip_capable<Chain>()) {
+            if (g.tiles_x == 0u) { strip_body<Chain>(p); return; }      // wave uniform: the launcher chose the strip form
+        }
+        gather_body<Chain, FKD_GATHER_XI, FKD_GATHER_YI>(p, g);
+    }
     else rows_auto_body<Chain, RowsConfig<Chain>::V, RowsConfig<Chain>::ROWS>(p);
 }
 

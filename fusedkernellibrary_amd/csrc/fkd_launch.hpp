@@ -3,6 +3,7 @@
 #pragma once
 
 #include "fkd_kernels.hpp"
+#include "registry.hpp"
 
 namespace fkd {
 
@@ -30,6 +31,17 @@ template <class Chain>
 hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info) {
     constexpr int XI = FKD_GATHER_XI, YI = FKD_GATHER_YI;
     constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
+    if constexpr (strip_capable<Chain>()) {
+        // Narrow outputs (batches of small planes): the strip form, whose workgroups own 8 whole rows of a plane.
+        if (p.active_w <= unsigned(kStripMaxWidth) && (p.reserved & 1u) != 0 && fklhip::strip_enabled()) {
+            const dim3 grid((p.active_h + kStripRows - 1) / kStripRows, 1, p.active_z), block(kGatherBX, kStripThreads / kGatherBX, 1);
+            if (info) *info = LaunchInfo{"strip", {grid.x, 1, grid.z}, {block.x, block.y, 1}, unsigned((kStripMaxWidth + (kStripDepth + 1) * kStripStep) * 16 + 4)};
+            if (grid.x == 0 || grid.z == 0) return hipSuccess;
+            if (grid.z > 65535u) return hipErrorInvalidConfiguration;
+            hipLaunchKernelGGL((k_strip<Chain>), grid, block, 0, stream, p);
+            return hipGetLastError();
+        }
+    }
     TileGeom g;
     g.tiles_x = (p.active_w + TW - 1) / TW;
     g.tiles_y = (p.active_h + TH - 1) / TH;

@@ -35,9 +35,9 @@
 namespace fklhip {
 namespace {
 
-// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): eight and four 32-bit words.
+// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): nine and four 32-bit words.
 struct JitMeta {
-    unsigned gather, params_bytes, v, rows, xi, yi, by, max_planes;
+    unsigned gather, params_bytes, v, rows, xi, yi, by, max_planes, strip_width;
 };
 struct TileGeom {
     unsigned tiles_x, tiles_y, n_tiles, tiles_x_magic;
@@ -89,6 +89,28 @@ bool signature_is_clean(const char* s) {
     return true;
 }
 
+// Extra preprocessor definitions for kernels compiled at run time, for tuning the kernels' compile-time constants
+// (FKD_ROWS and the like) without rebuilding the library: FKLHIP_JIT_DEFINES="-DNAME=VALUE -DOTHER=VALUE".  Only tokens of
+// that form pass (letters, digits, '_' and '='); anything else in the variable is ignored.
+std::vector<std::string> extra_defines() {
+    std::vector<std::string> out;
+    const char* v = getenv("FKLHIP_JIT_DEFINES");
+    if (!v) return out;
+    std::string token;
+    auto flush = [&] {
+        bool ok = token.size() > 2 && token[0] == '-' && token[1] == 'D';
+        for (size_t i = 2; ok && i < token.size(); ++i) {
+            const char c = token[i];
+            ok = (c >= 'a' && c <= 'z') || (c >= 'A' && c <= 'Z') || (c >= '0' && c <= '9') || c == '_' || c == '=';
+        }
+        if (ok) out.push_back(token);
+        token.clear();
+    };
+    for (; *v; ++v) { if (*v == ' ') flush(); else token.push_back(*v); }
+    flush();
+    return out;
+}
+
 // ---- on-disk cache of code objects (opt in: FKLHIP_JIT_CACHE=<directory>) -----------------------------------------
 
 unsigned long long fnv1a(unsigned long long h, const char* data, size_t n) {
@@ -104,6 +126,7 @@ std::string cache_path(const char* signature, const std::string& arch) {
     unsigned long long a = fnv1a(14695981039346656037ull, std::string(signature));
     unsigned long long b = fnv1a(0x9e3779b97f4a7c15ull, arch);
     for (int i = 0; i < kJitFlagCount; ++i) b = fnv1a(b, std::string(kJitFlags[i]));
+    for (const std::string& d : extra_defines()) b = fnv1a(b, d);
     for (int i = 0; i < kJitHeaderCount; ++i) { b = fnv1a(b, std::string(kJitHeaderNames[i])); b = fnv1a(b, std::string(kJitHeaderTexts[i])); }
     a = fnv1a(a, std::string(reinterpret_cast<const char*>(&b), sizeof(b)));
     char name[64];
@@ -184,12 +207,20 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
     JitKernel* k = const_cast<JitKernel*>(static_cast<const JitKernel*>(ctx));
     if (!blob) return FKLHIP_EINVAL;
     if (bytes != k->meta.params_bytes) return FKLHIP_EBLOB_SIZE;
-    unsigned active[3];
-    memcpy(active, blob, sizeof(active));   // Chain::Params starts with active_w, active_h, active_z
+    unsigned active[4];
+    memcpy(active, blob, sizeof(active));   // Chain::Params starts with active_w, active_h, active_z, reserved (bit 0: strip form allowed)
     const JitMeta& m = k->meta;
     TileGeom g{0, 0, 0, 0};
     unsigned grid[3], block[3] = {64, 4, 1};
-    if (m.gather) {
+    const char* kind = m.gather ? "gather_jit" : "rows_jit";
+    if (m.gather && m.strip_width != 0 && active[0] <= m.strip_width && (active[3] & 1u) != 0 && strip_enabled()) {
+        // strip form: one workgroup per m.by * m.yi output rows of a plane; the all-zero TileGeom tells the kernel
+        kind = "strip_jit";
+        grid[0] = (active[1] + m.by * m.yi - 1) / (m.by * m.yi);
+        grid[1] = 1;
+        grid[2] = active[2];
+        block[1] = m.by;
+    } else if (m.gather) {
         const unsigned tw = 64 * m.xi, th = m.by * m.yi;
         g.tiles_x = (active[0] + tw - 1) / tw;
         g.tiles_y = (active[1] + th - 1) / th;
@@ -204,7 +235,7 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
         grid[1] = (active[1] + 4 * m.rows - 1) / (4 * m.rows);
         grid[2] = active[2];
     }
-    if (info) *info = fkd::LaunchInfo{m.gather ? "gather_jit" : "rows_jit", {grid[0], grid[1], grid[2]}, {block[0], block[1], 1}, 0};
+    if (info) *info = fkd::LaunchInfo{kind, {grid[0], grid[1], grid[2]}, {block[0], block[1], 1}, 0};
     if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return FKLHIP_OK;
     if (grid[1] > 65535u || grid[2] > 65535u) return int(hipErrorInvalidConfiguration);
     if (m.max_planes != 0 && grid[2] > m.max_planes) return int(hipErrorInvalidConfiguration);   // as launch_divergent
@@ -251,6 +282,8 @@ static int build_and_register(const char* signature, bool may_read_cache) {
         std::vector<const char*> opts;
         opts.push_back(arch.c_str());
         for (int i = 0; i < kJitFlagCount; ++i) opts.push_back(kJitFlags[i]);
+        const std::vector<std::string> defines = extra_defines();
+        for (const std::string& d : defines) opts.push_back(d.c_str());
         r = hiprtcCompileProgram(prog, int(opts.size()), opts.data());
         size_t log_size = 0;
         if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {

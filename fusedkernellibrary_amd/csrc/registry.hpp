@@ -2,6 +2,7 @@
 #pragma once
 
 #include <stddef.h>
+#include <stdlib.h>
 
 namespace fkd { struct LaunchInfo; }
 
@@ -17,6 +18,13 @@ struct Entry {
     LaunchFn launch;
     const void* ctx;
 };
+
+// Narrow outputs of bilinear chains are launched in strip form unless FKLHIP_STRIP=0 (read at every launch, so one process
+// can run both forms on the same input; the two give identical results).
+inline bool strip_enabled() {
+    const char* e = getenv("FKLHIP_STRIP");
+    return !(e && e[0] == '0' && e[1] == 0);
+}
 
 // Called from static initialisers of the generated instance files, and by the run-time compiler.
 void register_chain(const char* signature, size_t blob_bytes, LaunchFn fn, const void* ctx = nullptr);

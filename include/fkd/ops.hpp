@@ -487,6 +487,15 @@ FKD_DEV TapImage make_tap_image(const void* data) {
     im.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(data)) - im.lo, 0, 0xffffffffu, 0x00020000);
     return im;
 }
+// `bytes` of image behind `data` (less than 4 GB): the extent ends with the dword that holds the last of them.  That dword
+// starts inside the image, so it lies in a mapped page whatever follows the allocation.
+FKD_DEV TapImage make_tap_image(const void* data, size_t bytes) {
+    TapImage im;
+    im.lo = u32(reinterpret_cast<uintptr_t>(data)) & 3u;
+    const u32 extent = (u32(bytes) + im.lo + 3u) & ~3u;
+    im.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(data)) - im.lo, 0, extent, 0x00020000);
+    return im;
+}
 template <class T> FKD_DEV PairPrep prepare_pair_window(const TapImage& im, u32 off) {
     PairPrep pp;
     if constexpr (PairWindow<T>::kShift) {
@@ -520,8 +529,15 @@ template <class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& fi
         else v[i] = p.w[i];
         if constexpr (sizeof(base_t<T>) < 4) asm("" : "+v"(v[i]));   // keep dwords whole: v_cvt_f32_ubyteN / v_bfe
     }
-    first = unpack_one<0, T>(v);
-    second = unpack_one<1, T>(v);
+    // channel by channel: copying whole 3-byte elements makes the compiler gather each into one register first
+    // (v_perm_b32), although every channel leaves its dword through v_cvt_f32_ubyteN anyway
+    constexpr int N = cn_v<T>;
+    using B = base_t<T>;
+    chan<0>(first) = unpack_elem<0, B>(v);
+    chan<0>(second) = unpack_elem<N, B>(v);
+    if constexpr (N > 1) { chan<1>(first) = unpack_elem<1, B>(v); chan<1>(second) = unpack_elem<N + 1, B>(v); }
+    if constexpr (N > 2) { chan<2>(first) = unpack_elem<2, B>(v); chan<2>(second) = unpack_elem<N + 2, B>(v); }
+    if constexpr (N > 3) { chan<3>(first) = unpack_elem<3, B>(v); chan<3>(second) = unpack_elem<N + 3, B>(v); }
 }
 
 // Store counterpart of load_bits_at: element sizes 2 and multiples of 4 (up to 16) leave as one access.
@@ -1278,6 +1294,11 @@ template <class T> struct Read2D {
     static constexpr bool kFiniteTaps = !(__is_same(base_t<T>, f32) || __is_same(base_t<T>, f64));
     static constexpr bool kBoundedOut = small_integer_base<T>();
     FKD_NAME("Read2D<" + type_name<T>() + ">")
+    // What the strip form of the bilinear kernel asks of a source image (checked on the host, see Chain::finalize): rows
+    // that share their alignment, 32-bit offsets, two columns.
+    FKD_HD static bool strip_ok(const Params& p) {
+        return p.pitch % 4 == 0 && size_t(p.pitch) * p.height < 0xfffffff0ull && p.width >= 2 && p.height >= 1;
+    }
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }
     FKD_DEV static int height(const Params& p) { return int(p.height); }
@@ -1330,6 +1351,12 @@ template <class T> struct Read2D {
     using TapImage = detail::TapImage;
     using PairPrep = detail::PairPrep;
     FKD_DEV static TapImage tap_image(int, const Params& p) { return detail::make_tap_image(p.data); }
+    // The same image with the resource's extent closed at the dword that holds the image's last byte: a window that
+    // reaches past it reads zeros instead of memory (the address check works dword by dword), so lanes on the last
+    // rows need no other form of access.
+    FKD_DEV static TapImage tap_image_bounded(int, const Params& p) {
+        return detail::make_tap_image(p.data, size_t(p.pitch) * (p.height - 1) + size_t(p.width) * sizeof(T));
+    }
     FKD_DEV static u32 tap_row_offset(int y, const Params& p) { return u32(y) * p.pitch; }
     FKD_DEV static PairPrep pair_prepare(const TapImage& im, int x, const Params&) {
         return detail::prepare_pair_window<T>(im, u32(x) * u32(sizeof(T)));
@@ -1675,6 +1702,9 @@ template <class Back> struct Crop {
     static constexpr bool kTapCursor = Back::kTapCursor;
     static constexpr bool kBoundedOut = bounded_out<Back>();
     FKD_NAME("Crop<" + Back::name() + ">")
+    FKD_HD static bool strip_ok(const Params& p) {
+        if constexpr (requires { Back::strip_ok(p.back); }) return p.w >= 2 && p.h >= 1 && Back::strip_ok(p.back); else return false;
+    }
 #if defined(FKD_EXEC_CODE)
     static constexpr bool kFiniteTaps = finite_taps<Back>();
     FKD_DEV static int width(const Params& p) { return p.w; }
@@ -1709,6 +1739,9 @@ template <class Back> struct Crop {
     using PairPrep = detail::PairPrep;
     FKD_DEV static TapImage tap_image(int z, const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_image(z, p.back); else return TapImage{};
+    }
+    FKD_DEV static TapImage tap_image_bounded(int z, const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_image_bounded(z, p.back); else return TapImage{};
     }
     FKD_DEV static u32 tap_row_offset(int y, const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_row_offset(y + p.y, p.back); else return 0u;
@@ -1798,6 +1831,9 @@ template <class Back, class... Ops> struct FusedRead {
     static constexpr bool kTapCursor = Back::kTapCursor;
     static constexpr bool kBoundedOut = bounded_out<Back>() && (finite_map<Ops>() && ...);
     FKD_NAME("FusedRead<" + Back::name() + OpList<Ops...>::names() + ">")
+    FKD_HD static bool strip_ok(const Params& p) {
+        if constexpr (requires { Back::strip_ok(p.back); }) return Back::strip_ok(p.back); else return false;
+    }
 #if defined(FKD_EXEC_CODE)
     static constexpr bool kFiniteTaps = finite_taps<Back>() && (finite_map<Ops>() && ...);
     FKD_DEV static int width(const Params& p) { return Back::width(p.back); }
@@ -1838,6 +1874,9 @@ template <class Back, class... Ops> struct FusedRead {
     FKD_DEV static TapImage tap_image(int z, const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_image(z, p.back); else return TapImage{};
     }
+    FKD_DEV static TapImage tap_image_bounded(int z, const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_image_bounded(z, p.back); else return TapImage{};
+    }
     FKD_DEV static u32 tap_row_offset(int y, const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_row_offset(y, p.back); else return 0u;
     }
@@ -1877,6 +1916,9 @@ template <int AR, class Back> struct ResizeLinear {
     static constexpr bool kBoundedOut = AR == IGNORE_AR && bounded_out<Back>();   // a letterbox colour is a run-time value
     using BackOp = Back;
     FKD_NAME("ResizeLinear<" + istr(AR) + "," + Back::name() + ">")
+    FKD_HD static bool strip_ok(const Params& p, u32 = 1u) {
+        if constexpr (requires { Back::strip_ok(p.back); }) return Back::strip_ok(p.back); else return false;
+    }
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return p.dst_w; }
     FKD_DEV static int height(const Params& p) { return p.dst_h; }
@@ -2123,6 +2165,14 @@ template <int N, class PlaneOp> struct BatchRead {
     static constexpr bool kTapCursor = false;
     static constexpr bool kBoundedOut = bounded_out<PlaneOp>();
     FKD_NAME("BatchRead<" + istr(N) + "," + PlaneOp::name() + ">")
+    FKD_HD static bool strip_ok(const Params& p, u32 planes) {
+        if constexpr (requires { PlaneOp::strip_ok(p.plane[0]); }) {
+            for (u32 z = 0; z < planes && z < u32(N); ++z) if (!PlaneOp::strip_ok(p.plane[z])) return false;
+            return planes <= u32(N);
+        } else {
+            return false;
+        }
+    }
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return PlaneOp::exec(x, y, z, p.plane[z]); }
 #endif
@@ -2270,6 +2320,11 @@ template <class T, bool TRANSPOSED = false> struct TensorSplit {
     using G = detail::PlanarGeometry<B, TRANSPOSED>;
     using Params = typename G::template View<B>;
     FKD_NAME((TRANSPOSED ? "TensorTSplit<" : "TensorSplit<") + type_name<T>() + ">")
+    // An image plane with all its channel planes fits 31-bit byte offsets (stores through a buffer resource, see put_masked).
+    FKD_HD static bool strip_ok(const Params& p) {
+        return G::channel_elements(p) * sizeof(B) * cn_v<T> < size_t(0x7fffffffu) &&
+               G::channel_elements(p) * sizeof(B) * (cn_v<T> - 1) + size_t(p.pitch) * p.height < size_t(0x7fffffffu);
+    }
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static B* at(const Params& p, int x, int y, int z) {
         return reinterpret_cast<B*>(reinterpret_cast<char*>(p.data) + G::image_bytes(p) * z + size_t(y) * p.pitch) + x;
@@ -2320,10 +2375,7 @@ template <class T, bool TRANSPOSED = false> struct TensorSplit {
     static constexpr bool kLaneMasked = sizeof(B) == 4;
     static constexpr u32 kMaskedExtent = 0x7fffffffu, kMaskedOut = 0x80000000u;
     struct PlaneRef { __amdgpu_buffer_rsrc_t rsrc; u32 chan_bytes, pitch; };
-    FKD_DEV static bool plane_maskable(const Params& p) {
-        return G::channel_elements(p) * sizeof(B) * cn_v<T> < size_t(kMaskedExtent) &&
-               G::channel_elements(p) * sizeof(B) * (cn_v<T> - 1) + size_t(p.pitch) * p.height < size_t(kMaskedExtent);
-    }
+    FKD_DEV static bool plane_maskable(const Params& p) { return strip_ok(p); }
     FKD_DEV static PlaneRef plane_ref(int z, const Params& p) {
         char* base = reinterpret_cast<char*>(p.data) + G::image_bytes(p) * z;
         PlaneRef r;
@@ -2335,7 +2387,10 @@ template <class T, bool TRANSPOSED = false> struct TensorSplit {
     FKD_DEV static u32 lane_offset(int x, bool valid) { return valid ? u32(x) * u32(sizeof(B)) : kMaskedOut; }
     FKD_DEV static u32 row_offset(int y, const PlaneRef& r) { return u32(y) * r.pitch; }
     FKD_DEV static void put_masked(const PlaneRef& r, u32 row_off, u32 lane_off, const T& v) {
-        constexpr int kThrough = 1 | 16;     // sc0 sc1: written through the L2, as gstore_through
+#ifndef FKD_STORE_AUX
+#define FKD_STORE_AUX (1 | 16)
+#endif
+        constexpr int kThrough = FKD_STORE_AUX;     // sc0 sc1: written through the L2, as gstore_through
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<0>(v)), r.rsrc, lane_off, row_off, kThrough);
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<1>(v)), r.rsrc, lane_off, row_off + r.chan_bytes, kThrough);
         if constexpr (cn_v<T> > 2) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, chan<2>(v)), r.rsrc, lane_off, row_off + 2u * r.chan_bytes, kThrough);
@@ -2583,6 +2638,15 @@ template <class R, class... Ops, class W> struct Chain<R, OpList<Ops...>, W> {
         else return finite_map<typename TypeAt<K - 1, Ops...>::type>() && prefix_finite<K - 1>();
     }
     static void finalize(Params& p) { finalize_from<0>(p); }
+    // Host, once read AND write are filled in: bit 0 of `reserved` tells the launcher that every active plane meets what
+    // the strip form of the bilinear kernel asks of its source and destination (that form has no other way to decline a
+    // plane).  A parameter block that never came through here keeps the bit clear and gets the tile form.
+    static constexpr u32 kStripChecked = 1u;
+    static void finalize_write(Params& p) {
+        if constexpr (requires { R::strip_ok(p.read, p.active_z); W::strip_ok(p.write); }) {
+            if (R::strip_ok(p.read, p.active_z) && W::strip_ok(p.write)) p.reserved |= kStripChecked;
+        }
+    }
 #endif
 #if defined(FKD_EXEC_CODE)
     static_assert(__is_same(Value, typename W::In), "the write operation does not take the type the chain produces");

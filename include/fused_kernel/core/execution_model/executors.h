@@ -83,6 +83,7 @@ template <typename... IOps> struct FusedChain {
             } else {
                 p.write = lower_iop(std::get<N - 1>(all));
             }
+            Chain::finalize_write(p);
             return p;
         }
     };

@@ -358,6 +358,23 @@ int fklcase_uncompiled_gray_resize(void* stream_, const uint8_t* in, int w, int 
                                           PerThreadWrite<ND::_2D, float>::build(o.ptr()));
     });
 }
+// three crops of a uchar3 image -> letterboxed bilinear resize -> Mul -> planar float tensor (a bilinear chain with narrow
+// planar output that is not compiled ahead of time: the strip form of the kernel, through the run-time compiler)
+int fklcase_uncompiled_letterbox_split_b3(void* stream_, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw, int dh,
+                                          const float* bg, const float* mul, float* out) {
+    return guarded([&] {
+        Stream stream(stream_);
+        const auto in = dev2d<uchar3>(src, w, h, pitch);
+        Tensor<float> o(out, uint(dw), uint(dh), 3u, 3, MemType::Device, 0);
+        const auto crops = rects_from<3>(rects);
+        for (int rep = 0; rep < g_reps; ++rep) executeOperations<TransformDPP<>>(stream,
+            PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
+            Crop<>::build(crops),
+            Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(dw, dh), float3{bg[0], bg[1], bg[2]}),
+            Mul<float3>::build(make_<float3>(mul[0], mul[1], mul[2])),
+            TensorSplit<float3>::build(o.ptr()));
+    });
+}
 // float4 image -> bilinear resize -> float4 image (16-byte elements: one access per tap)
 int fklcase_uncompiled_float4_resize(void* stream_, const float* in, int w, int h, int pitch, int dw, int dh, float* out, int out_pitch) {
     return guarded([&] {

@@ -194,6 +194,14 @@ def uncompiled_gray_resize(src, rect, dst, mul, out):
                                                int(dst[0]), int(dst[1]), C.c_float(float(mul)), _p(out), out.stride(0) * 4))
 
 
+def uncompiled_letterbox_split_b3(src, rects, dst, bg, mul, out):
+    """(H,W,3) u8 cuda, 3 crops -> letterboxed bilinear (dst = (w,h)) -> * mul -> out (3,3,dh,dw) f32 cuda."""
+    r, b, m = _host(rects, np.int32), _host(bg, np.float32), _host(mul, np.float32)
+    _ok(cases().fklcase_uncompiled_letterbox_split_b3(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0),
+                                                      r.ctypes.data_as(C.c_void_p), int(dst[0]), int(dst[1]),
+                                                      b.ctypes.data_as(C.c_void_p), m.ctypes.data_as(C.c_void_p), _p(out)))
+
+
 def uncompiled_float4_resize(src, dst, out):
     """(H,W,4) f32 cuda -> bilinear -> out (dh,dw,4) f32 cuda."""
     _ok(cases().fklcase_uncompiled_float4_resize(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, int(dst[0]), int(dst[1]),

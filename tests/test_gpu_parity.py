@@ -145,7 +145,7 @@ def test_config2_reduced_odd_width(device, n):
 def test_config3_full_size(device):
     c = wl.config3()
     got = run_c3(c, device)
-    assert last_launch()["kernel"] == "gather"
+    assert last_launch()["kernel"] == "strip"
     want = ol.oracle_crop_resize_norm_split(c["src"], c["rects"], c["dst"], c["sub"], c["div"])
     exact = check_float(got, want, "config 3 vs oracle")
     assert exact and sha(got) == DIG["c3_full"], "config 3 is expected to be bit-identical to the reference CPU backend"
