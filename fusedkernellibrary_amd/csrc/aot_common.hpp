@@ -7,6 +7,7 @@
 #include "registry.hpp"
 #include <fklhip.h>
 
+#include <stdint.h>
 #include <string.h>
 #include <string>
 
@@ -16,7 +17,11 @@ template <class Chain> int aot_launch(const void*, const void* blob, size_t byte
     using Params = typename Chain::Params;
     if (!blob) return FKLHIP_EINVAL;
     if (bytes != sizeof(Params)) return FKLHIP_EBLOB_SIZE;
-    Params p;   // by-value copy: the caller's block may go away as soon as we return
+    // The runtime copies the block into its kernel-argument buffer during the launch call, so the caller's block may go
+    // away as soon as we return; a block that is not aligned for its type is copied to one that is first.
+    if (reinterpret_cast<uintptr_t>(blob) % alignof(Params) == 0)
+        return int(fkd::launch_chain<Chain>(*static_cast<const Params*>(blob), static_cast<hipStream_t>(stream), info));
+    Params p;
     memcpy(&p, blob, sizeof(Params));
     return int(fkd::launch_chain<Chain>(p, static_cast<hipStream_t>(stream), info));
 }

@@ -571,6 +571,7 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
 constexpr int kStripRows = kGatherBY * FKD_GATHER_YI, kStripStep = 32, kStripMaxWidth = 256, kStripDepth = FKD_STRIP_DEPTH;
 constexpr int kStripThreads = kStripRows * kStripStep;
 static_assert(kStripThreads == kGatherBX * kGatherBY, "the two forms of the bilinear kernel share their workgroup shape");
+static_assert(kStripThreads == kStripMaxWidth && (kStripDepth + 1) * kStripStep <= kStripThreads, "one table column per thread");
 
 template <class Chain> constexpr bool strip_capable() {
     using Root = ResizeRoot<typename Chain::Read>;
@@ -598,7 +599,7 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     constexpr int kEntries = kStripMaxWidth + (D + 1) * kStripStep;
     // per column: ax, bx, window offset, bytes to drop from the window (bits 0-1) | flags
     __shared__ detail::u32x4_t column[kEntries];
-    __shared__ u32 any_clamped;
+    __shared__ u32 wave_clamped[kStripThreads / 64];
     constexpr u32 kClamped = 0x80000000u, kOutsideX = 0x40000000u;
 
     const int z = int(blockIdx.z);
@@ -620,33 +621,22 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     const int steps = (aw + kStripStep - 1) / kStripStep;
 
     const int t = int(threadIdx.y) * 64 + int(threadIdx.x);
-    // ---- the column table: one column per thread and pass; the D + 1 steps after the last one hold a window offset
-    // beyond the image's extent, so requesting them touches no memory ----
-    if (t == 0) any_clamped = 0u;
-    __syncthreads();
-    for (int col = t; col < (steps + D + 1) * kStripStep; col += kStripThreads) {
+    // What depends on the column: the horizontal weights, the window's byte offset in a row, and flags beside the bytes to drop.
+    auto column_entry = [&](int col, bool& clamped) {
+        const int x = col < aw ? col : aw - 1;                          // columns beyond the output shadow the last one
+        const f32 sx = f32(x - ox) * q.fx;
+        const f32 f1 = __builtin_floorf(sx);
+        const f32 ax = (f1 + 1.0f) - sx, bx = sx - f1;
+        const int xi = int(f1);
+        const int x1 = xi < 0 ? 0 : (xi < sw - 1 ? xi : sw - 1);
+        clamped = x1 + 1 > sw - 1;                                      // right tap is the last column again
+        const detail::PairPrep pp = Back::pair_prepare(image, x1 - int(clamped), q.back);
+        u32 flags = pp.shift | (clamped ? kClamped : 0u);
+        if constexpr (RZ::kAR != IGNORE_AR) flags |= (x >= q.x1 && x <= q.x2) ? 0u : kOutsideX;
         detail::u32x4_t e;
-        bool clamped = false;
-        if (col < steps * kStripStep) {
-            const int x = col < aw ? col : aw - 1;
-            const f32 sx = f32(x - ox) * q.fx;
-            const f32 f1 = __builtin_floorf(sx);
-            const f32 ax = (f1 + 1.0f) - sx, bx = sx - f1;
-            const int xi = int(f1);
-            const int x1 = xi < 0 ? 0 : (xi < sw - 1 ? xi : sw - 1);
-            clamped = x1 + 1 > sw - 1;                                  // right tap is the last column again
-            const detail::PairPrep pp = Back::pair_prepare(image, x1 - int(clamped), q.back);
-            u32 flags = pp.shift | (clamped ? kClamped : 0u);
-            if constexpr (RZ::kAR != IGNORE_AR) flags |= (x >= q.x1 && x <= q.x2) ? 0u : kOutsideX;
-            e.x = __builtin_bit_cast(u32, ax); e.y = __builtin_bit_cast(u32, bx); e.z = pp.off; e.w = flags;
-        } else {
-            e.x = 0u; e.y = 0u; e.z = 0xfffffff0u; e.w = 0u;
-        }
-        column[col] = e;
-        if (__builtin_amdgcn_ballot_w64(clamped) != 0ull && threadIdx.x == 0) any_clamped = 1u;
-    }
-    __syncthreads();
-    const bool some_clamped = __builtin_amdgcn_readfirstlane(any_clamped) != 0u;
+        e.x = __builtin_bit_cast(u32, ax); e.y = __builtin_bit_cast(u32, bx); e.z = pp.off; e.w = flags;
+        return e;
+    };
 
     // ---- the lane's row ----
     const int g = t & (kStripStep - 1), r = t >> 5;
@@ -662,14 +652,9 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     const u32 row_a = Back::tap_row_offset(ya, q.back), row_b = Back::tap_row_offset(yb, q.back);
     bool yin = true;
     if constexpr (RZ::kAR != IGNORE_AR) yin = yc >= q.y1 && yc <= q.y2;
-    const auto oplane = WP::plane_ref(z, wpar);
-    // the lane's store offset in step 0; a lane without a row carries an offset beyond the resource's extent
-    const u32 out0 = yvalid ? WP::row_offset(y, oplane) + WP::lane_offset(g, true) : WP::kMaskedOut;
-    const bool partial = (aw & (kStripStep - 1)) != 0;             // the last step has columns beyond the output
 
     struct StepTaps { detail::u32x4_t e; typename Back::PairBits ab, cd; };
-    auto request = [&](int k, StepTaps& s) {
-        s.e = column[g + kStripStep * k];
+    auto fetch = [&](StepTaps& s) {
         // (v_alignbyte_b32 takes the bytes to drop from bits 0-1 of its operand, so the flags may ride along)
         detail::PairPrep pa, pb;
         pa.off = s.e.z + row_a; pa.shift = s.e.w;
@@ -677,6 +662,47 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
         s.ab = Back::pair_load_prepared(image, 0u, pa, q.back);
         s.cd = Back::pair_load_prepared(image, 0u, pb, q.back);
     };
+    auto request = [&](int k, StepTaps& s) {
+        s.e = column[g + kStripStep * k];
+        fetch(s);
+        __builtin_amdgcn_sched_barrier(0);      // the next step's taps leave before anything waits for this step's
+    };
+    // The taps of step 0 are requested before the table exists, from the lane's own working out of its first column:
+    // they are then on their way while the table is made and the workgroup meets at the barrier.
+    StepTaps first;
+    {
+        bool unused;
+        first.e = column_entry(g, unused);
+        fetch(first);
+    }
+
+    // ---- the column table: one column per thread (the workgroup has as many threads as the form has columns); the
+    // D + 1 steps after the last one hold a window offset beyond the image's extent, so requesting them touches no
+    // memory.  Each wave notes whether it met a clamped column. ----
+    {
+        bool clamped = false;
+        detail::u32x4_t e = column_entry(t, clamped);
+        if (t >= steps * kStripStep) { e.z = 0xfffffff0u; clamped = false; }
+        column[t] = e;
+        if (t < (D + 1) * kStripStep) {
+            detail::u32x4_t none;
+            none.x = 0u; none.y = 0u; none.z = 0xfffffff0u; none.w = 0u;
+            column[kStripMaxWidth + t] = none;
+        }
+        const bool any = __builtin_amdgcn_ballot_w64(clamped) != 0ull;
+        if (threadIdx.x == 0) wave_clamped[threadIdx.y] = any ? 1u : 0u;
+    }
+    __syncthreads();
+    u32 met = 0;
+#pragma unroll
+    for (int w = 0; w < kStripThreads / 64; ++w) met |= wave_clamped[w];
+    const bool some_clamped = __builtin_amdgcn_readfirstlane(met) != 0u;
+
+    const auto oplane = WP::plane_ref(z, wpar);
+    // the lane's store offset in step 0; a lane without a row carries an offset beyond the resource's extent
+    const u32 out0 = yvalid ? WP::row_offset(y, oplane) + WP::lane_offset(g, true) : WP::kMaskedOut;
+    const bool partial = (aw & (kStripStep - 1)) != 0;             // the last step has columns beyond the output
+
     auto run = [&](auto static_tag, auto clamp_tag) {
         constexpr bool STATIC = decltype(static_tag)::value != 0;
         constexpr bool CLAMP = decltype(clamp_tag)::value != 0;
@@ -709,8 +735,7 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
         // a step's taps can then leave all later accesses in flight.  (Written out per depth with named tap sets: with
         // an array of sets the compiler rotates registers instead, and a copy of a register waits for its load.)
         if constexpr (D == 1) {
-            StepTaps s0, s1;
-            request(0, s0);
+            StepTaps s0 = first, s1;
             request(1, s1);
             produce(0, s0, false);
 #pragma unroll 1
@@ -723,8 +748,7 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
             }
         } else {
             static_assert(D == 2, "depths 1 and 2 are written out");
-            StepTaps s0, s1, s2;
-            request(0, s0);
+            StepTaps s0 = first, s1, s2;
             request(1, s1);
             request(2, s2);
             produce(0, s0, false);

@@ -1,5 +1,5 @@
 // fkd_launch.hpp -- host-side launchers of the ahead-of-time compiled kernels (grid geometry, host-side alignment
-// check, hipLaunchKernelGGL).  Launch geometry being replaced: FK/core/execution_model/executors.h:242-351.
+// check, hipLaunchKernel).  Launch geometry being replaced: FK/core/execution_model/executors.h:242-351.
 #pragma once
 
 #include "fkd_kernels.hpp"
@@ -8,6 +8,14 @@
 namespace fkd {
 
 // ---- host-side launchers -------------------------------------------------------------------------------
+
+// Launch with pointers to the arguments: the runtime then makes the only copy of the (up to 8 KB) parameter block,
+// straight into its kernel-argument buffer; the <<< >>> form would first copy it by value onto this thread's stack.
+template <class Kernel, class... Args>
+inline hipError_t launch_by_pointer(Kernel kernel, dim3 grid, dim3 block, hipStream_t stream, const Args&... args) {
+    void* ptrs[] = {const_cast<void*>(static_cast<const void*>(&args))...};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, 0, stream);
+}
 
 inline const char* aligned_name(bool aligned) { return aligned ? "rows" : "rows_unaligned"; }
 
@@ -22,9 +30,8 @@ hipError_t launch_rows(const typename Chain::Params& p, hipStream_t stream, Laun
     if (info) *info = LaunchInfo{aligned_name(aligned), {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
     if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
     if (grid.y > 65535u || grid.z > 65535u) return hipErrorInvalidConfiguration;
-    if (aligned) hipLaunchKernelGGL((k_rows<Chain, V, ROWS, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((k_rows<Chain, V, ROWS, false>), grid, block, 0, stream, p);
-    return hipGetLastError();
+    if (aligned) return launch_by_pointer(&k_rows<Chain, V, ROWS, true>, grid, block, stream, p);
+    return launch_by_pointer(&k_rows<Chain, V, ROWS, false>, grid, block, stream, p);
 }
 
 template <class Chain>
@@ -38,8 +45,7 @@ hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, La
             if (info) *info = LaunchInfo{"strip", {grid.x, 1, grid.z}, {block.x, block.y, 1}, unsigned((kStripMaxWidth + (kStripDepth + 1) * kStripStep) * 16 + 4)};
             if (grid.x == 0 || grid.z == 0) return hipSuccess;
             if (grid.z > 65535u) return hipErrorInvalidConfiguration;
-            hipLaunchKernelGGL((k_strip<Chain>), grid, block, 0, stream, p);
-            return hipGetLastError();
+            return launch_by_pointer(&k_strip<Chain>, grid, block, stream, p);
         }
     }
     TileGeom g;
@@ -52,8 +58,7 @@ hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, La
     if (info) *info = LaunchInfo{"gather", {grid.x, 1, grid.z}, {block.x, block.y, 1}, 0};
     if (g.n_tiles == 0) return hipSuccess;
     if (grid.z > 65535u) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((k_gather<Chain, XI, YI>), grid, block, 0, stream, p, g);
-    return hipGetLastError();
+    return launch_by_pointer(&k_gather<Chain, XI, YI>, grid, block, stream, p, g);
 }
 
 // Several chains in one launch: the grid of the rows kernel over the largest extent, alignment decided per plane on
@@ -67,8 +72,7 @@ hipError_t launch_divergent(const typename D::Params& p, hipStream_t stream, Lau
     if (info) *info = LaunchInfo{"divergent", {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
     if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
     if (grid.y > 65535u || grid.z > unsigned(D::kMaxPlanes)) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((k_divergent<D>), grid, block, 0, stream, p);
-    return hipGetLastError();
+    return launch_by_pointer(&k_divergent<D>, grid, block, stream, p);
 }
 
 template <class Chain>

@@ -746,30 +746,45 @@ template <class I, class P, class O> struct Div {
         }
         return true;
     }
+    // What the host works out for one divisor: the reciprocal in two floats, and which sequence it licenses
+    // (0 none: outside the accepted range; 1 five instructions; 2 two instructions).  A pure function of d that costs
+    // about half a microsecond, and applications divide by the same constants launch after launch (a normalisation's
+    // standard deviations), so each thread remembers the last divisors it analysed.
+    struct Analysis { f32 d, r, l; i32 mode; };
+    static Analysis analyse(f32 d) {
+        Analysis a{d, 0.0f, 0.0f, 0};
+        const f32 m = __builtin_fabsf(d);
+        if (!(m >= 0x1p-40f && m <= 0x1p40f)) return a;
+        a.r = exact_reciprocal(d);
+        a.l = reciprocal_low(d, a.r);
+        a.mode = (m >= 0x1p-30f && m <= 0x1p30f && two_step_proven(d, a.r, a.l)) ? 2 : 1;
+        return a;
+    }
+    static Analysis analyse_cached(f32 d) {
+        constexpr u32 kSlots = 16;
+        thread_local Analysis slot[kSlots] = {};        // d = 0 in an unused slot: zero is never analysed (mode 0)
+        const u32 bits = __builtin_bit_cast(u32, d);
+        Analysis& s = slot[(bits ^ (bits >> 9) ^ (bits >> 18)) % kSlots];
+        if (__builtin_bit_cast(u32, s.d) != bits || bits == 0u) s = analyse(d);
+        return s;
+    }
     static Params make(const P& v) {
         Params p{};
         p.v = v;
         p.fast = 0;
         if constexpr (kReciprocal) {
-            bool ok = true, two = true;
-            auto one = [&](f32 d) {
-                const f32 a = __builtin_fabsf(d);
-                if (!(a >= 0x1p-40f && a <= 0x1p40f)) { ok = false; return 0.0f; }
-                return exact_reciprocal(d);
+            i32 mode = 2;
+            auto one = [&](f32 d, f32& r, f32& l) {
+                const Analysis a = analyse_cached(d);
+                r = a.r; l = a.l;
+                mode = a.mode < mode ? a.mode : mode;
             };
-            p.rcp = map1<P>(v, one);
-            if (ok) {
-                p.rcp_lo = map2<P>(v, p.rcp, [](f32 d, f32 r) { return reciprocal_low(d, r); });
-                auto proven = [&](f32 d, f32 r, f32 l) {
-                    const f32 a = __builtin_fabsf(d);
-                    if (!(a >= 0x1p-30f && a <= 0x1p30f) || !two_step_proven(d, r, l)) two = false;
-                };
-                proven(chan_or_scalar<0>(v), chan_or_scalar<0>(p.rcp), chan_or_scalar<0>(p.rcp_lo));
-                if constexpr (cn_v<P> > 1) proven(chan<1>(v), chan<1>(p.rcp), chan<1>(p.rcp_lo));
-                if constexpr (cn_v<P> > 2) proven(chan<2>(v), chan<2>(p.rcp), chan<2>(p.rcp_lo));
-                if constexpr (cn_v<P> > 3) proven(chan<3>(v), chan<3>(p.rcp), chan<3>(p.rcp_lo));
-            }
-            p.fast = ok ? (two ? 2 : 1) : 0;
+            one(chan<0>(v), chan<0>(p.rcp), chan<0>(p.rcp_lo));
+            if constexpr (cn_v<P> > 1) one(chan<1>(v), chan<1>(p.rcp), chan<1>(p.rcp_lo));
+            if constexpr (cn_v<P> > 2) one(chan<2>(v), chan<2>(p.rcp), chan<2>(p.rcp_lo));
+            if constexpr (cn_v<P> > 3) one(chan<3>(v), chan<3>(p.rcp), chan<3>(p.rcp_lo));
+            if (mode == 0) { p.rcp = P{}; p.rcp_lo = P{}; }       // as before: no reciprocal is published for a refused divisor
+            p.fast = mode;
         }
         return p;
     }
@@ -1908,7 +1923,8 @@ template <int AR, class Back> struct ResizeLinear {
     // Both scale factors are whole numbers and every source coordinate index * factor is an exact float: every source
     // point is then a pixel and the bilinear weights are exactly 1, 0, 0, 0.
     FKD_HD static i32 whole_factors(i32 dst_w, i32 dst_h, f32 fx, f32 fy) {
-        return fx >= 1.0f && fy >= 1.0f && fx == __builtin_floorf(fx) && fy == __builtin_floorf(fy) &&
+        // (whole numbers up to 2^24 survive the trip through an integer; no library call on the host)
+        return fx >= 1.0f && fy >= 1.0f && fx <= 16777216.0f && fy <= 16777216.0f && fx == f32(i32(fx)) && fy == f32(i32(fy)) &&
                f32(dst_w) * fx <= 16777216.0f && f32(dst_h) * fy <= 16777216.0f;
     }
     static constexpr bool kTapCursor = false;

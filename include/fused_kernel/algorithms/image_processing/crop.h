@@ -47,10 +47,7 @@ template <typename BackIOp> struct Lower<Crop<BackIOp>, std::enable_if_t<!std::i
     static constexpr bool available = true;
     using type = fkd::Crop<device_op_t<BackIOp>>;
     static typename type::Params params(const OperationData<Crop<BackIOp>>& d) {
-        typename type::Params p{};
-        p.x = int(d.params.x); p.y = int(d.params.y); p.w = d.params.width; p.h = d.params.height;
-        p.back = lower_iop(d.backIOp);
-        return p;
+        return typename type::Params{int(d.params.x), int(d.params.y), int(d.params.width), int(d.params.height), lower_iop(d.backIOp)};
     }
 };
 } // namespace amd

@@ -195,20 +195,16 @@ struct Lower<ResizeComplete<AR, Ternary<InterpolateComplete<IT, BackIOp>>>> {
     using Self = ResizeComplete<AR, Ternary<InterpolateComplete<IT, BackIOp>>>;
     using type = fkd::ResizeLinear<(AR == AspectRatio::IGNORE_AR ? fkd::IGNORE_AR : fkd::PRESERVE_AR), device_op_t<BackIOp>>;
     static typename type::Params params(const OperationData<Self>& d) {
-        typename type::Params p{};
-        p.dst_w = d.params.dstSize.width;
-        p.dst_h = d.params.dstSize.height;
-        p.fx = d.params.src_conv_factors.x;
-        p.fy = d.params.src_conv_factors.y;
-        p.whole = type::whole_factors(p.dst_w, p.dst_h, p.fx, p.fy);
+        // (one aggregate initialisation, the back operation's parameters built in place: this runs once per plane of a batch)
+        const int dw = d.params.dstSize.width, dh = d.params.dstSize.height;
+        const float fx = d.params.src_conv_factors.x, fy = d.params.src_conv_factors.y;
         if constexpr (AR == AspectRatio::IGNORE_AR) {
-            p.x1 = 0; p.y1 = 0; p.x2 = p.dst_w - 1; p.y2 = p.dst_h - 1;
+            return typename type::Params{dw, dh, fx, fy, 0, 0, dw - 1, dh - 1, typename type::Out{}, type::whole_factors(dw, dh, fx, fy),
+                                         lower_iop(d.backIOp.backIOp)};
         } else {
-            p.x1 = d.params.x1; p.y1 = d.params.y1; p.x2 = d.params.x2; p.y2 = d.params.y2;
-            p.bg = to_dev(d.params.defaultValue);
+            return typename type::Params{dw, dh, fx, fy, d.params.x1, d.params.y1, d.params.x2, d.params.y2, to_dev(d.params.defaultValue),
+                                         type::whole_factors(dw, dh, fx, fy), lower_iop(d.backIOp.backIOp)};
         }
-        p.back = lower_iop(d.backIOp.backIOp);
-        return p;
     }
 };
 } // namespace amd

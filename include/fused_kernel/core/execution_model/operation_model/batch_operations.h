@@ -5,6 +5,9 @@
 #ifndef FK_AMD_BATCH_OPERATIONS_H
 #define FK_AMD_BATCH_OPERATIONS_H
 
+#include <new>
+#include <type_traits>
+
 #ifndef FK_AMD_OPERATION_MODEL_H
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
 #else
@@ -30,6 +33,16 @@ struct BatchReadParams<BATCH, PlanePolicy::PROCESS_ALL, Operation, NullType> {
 template <PlanePolicy PP = PlanePolicy::PROCESS_ALL, size_t BATCH = 1, typename Operation = TypeList<void>> struct BatchRead;
 
 namespace batch_detail {
+// slot = make(), with the value built where it lives: at run time the result of make() initialises the slot directly
+// (an assignment builds it on the stack field by field and copies it over whole, which stalls once per plane of a batch).
+template <typename T, typename F> constexpr void build_in(T& slot, F&& make) {
+    if (std::is_constant_evaluated()) {
+        slot = make();
+    } else {
+        static_assert(std::is_trivially_destructible_v<T>);
+        ::new (static_cast<void*>(&slot)) T(make());
+    }
+}
 // Members every concrete BatchRead flavour shares.
 template <typename Self, typename Op, size_t B, PlanePolicy POLICY, typename Params, typename Out, bool COMPLETE>
 struct ReadCommon {
@@ -101,7 +114,7 @@ template <> struct BatchRead<PlanePolicy::PROCESS_ALL, 1, TypeList<void>> {
                                                  BatchRead<PlanePolicy::PROCESS_ALL, BATCH, NewOperation>,
                                                  BatchRead<PlanePolicy::PROCESS_ALL, BATCH, TypeList<NewOperation>>>;
         typename BatchReadType::ParamsType store{{}, ActiveThreads{max_width, max_height, uint(BATCH)}};
-        for (size_t i = 0; i < BATCH; ++i) store.opData[i] = iOps[i];
+        for (size_t i = 0; i < BATCH; ++i) batch_detail::build_in(store.opData[i], [&]() -> std::remove_reference_t<decltype(store.opData[i])> { return iOps[i]; });
         return BatchReadType::build(store);
     }
 };
@@ -126,7 +139,7 @@ template <> struct BatchRead<PlanePolicy::CONDITIONAL_WITH_DEFAULT, 1, TypeList<
         if constexpr (std::is_same_v<NewOutputType, DefaultType>) def = defaultValue;
         else def = amd_cast_default<NewOutputType>(defaultValue);
         typename BatchReadType::ParamsType store{{}, usedPlanes, def, ActiveThreads{max_width, max_height, uint(BATCH)}};
-        for (size_t i = 0; i < BATCH; ++i) store.opData[i] = iOps[i];
+        for (size_t i = 0; i < BATCH; ++i) batch_detail::build_in(store.opData[i], [&]() -> std::remove_reference_t<decltype(store.opData[i])> { return iOps[i]; });
         return BatchReadType::build(store);
     }
 private:
@@ -149,8 +162,8 @@ struct BatchUtils {
         constexpr size_t B = IOpType::Operation::BATCH;
         std::array<Instantiable<Operation>, B> result{};
         for (size_t i = 0; i < B; ++i) {
-            if constexpr (IOpType::template is<ReadType>) result[i] = Operation::build(batchIOp.params.opData[i]);
-            else result[i] = Operation::build(OperationData<Operation>{batchIOp.params[i]});
+            if constexpr (IOpType::template is<ReadType>) batch_detail::build_in(result[i], [&] { return Operation::build(batchIOp.params.opData[i]); });
+            else batch_detail::build_in(result[i], [&] { return Operation::build(OperationData<Operation>{batchIOp.params[i]}); });
         }
         return result;
     }
@@ -160,7 +173,7 @@ struct BatchUtils {
     static constexpr auto build_batch(const std::array<ArrayType, BATCH>& firstArray, const Arrays&... arrays) {
         using Built = decltype(Operation::build(std::declval<ArrayType>(), std::declval<Arrays>()[0]...));
         std::array<Built, BATCH> result{};
-        for (size_t i = 0; i < BATCH; ++i) result[i] = Operation::build(firstArray[i], arrays[i]...);
+        for (size_t i = 0; i < BATCH; ++i) batch_detail::build_in(result[i], [&] { return Operation::build(firstArray[i], arrays[i]...); });
         return result;
     }
 };
@@ -223,8 +236,12 @@ struct Lower<BatchRead<PlanePolicy::PROCESS_ALL, B, Op>, std::enable_if_t<isComp
     using Self = BatchRead<PlanePolicy::PROCESS_ALL, B, Op>;
     using type = fkd::BatchRead<int(B), typename Lower<Op>::type>;
     static typename type::Params params(const OperationData<Self>& d) {
-        typename type::Params p{};
-        for (size_t i = 0; i < B; ++i) p.plane[i] = Lower<Op>::params(d.params.opData[i]);
+        // each plane's parameters are built where they live (an assignment would build them on the stack in small
+        // pieces and read them back whole, which stalls on every plane)
+        typename type::Params p;
+        using PlaneParams = std::remove_reference_t<decltype(p.plane[0])>;
+        static_assert(std::is_trivially_destructible_v<PlaneParams>);
+        for (size_t i = 0; i < B; ++i) ::new (static_cast<void*>(&p.plane[i])) PlaneParams(Lower<Op>::params(d.params.opData[i]));
         return p;
     }
 };

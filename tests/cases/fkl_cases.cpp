@@ -31,6 +31,8 @@
 #include "border_chains.h"  // padding chains, shared the same way
 #include "circular_chains.h"  // divergent launches and the CircularTensor window, shared the same way
 
+#include <time.h>
+
 using namespace fk;
 
 namespace {
@@ -38,9 +40,23 @@ namespace {
 thread_local char g_error[2048] = "";
 thread_local int g_reps = 1;   // how many times the next chain is enqueued (benchmarks time the whole run)
 
+// Timing of the next driver call (benchmarks): one event recorded on `stream` right before the call's first launch and one
+// right after its last, so the bracket holds the `reps` launches and nothing of the caller's own preparations.
+struct Timing { void* stream = nullptr; void* first = nullptr; void* last = nullptr; bool armed = false; long long start_ns = 0; };
+thread_local Timing g_timing;
+long long monotonic_ns() {
+    timespec ts{};
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (long long)ts.tv_sec * 1000000000ll + ts.tv_nsec;
+}
+
 template <typename F> int guarded(F body) {
+    const bool timed = g_timing.armed;
+    g_timing.armed = false;
     try {
+        if (timed) { g_timing.start_ns = monotonic_ns(); gpuErrchk(fklhip_event_record(g_timing.first, g_timing.stream)); }
         body();
+        if (timed) gpuErrchk(fklhip_event_record(g_timing.last, g_timing.stream));
         g_reps = 1;
         return 0;
     } catch (const std::exception& e) {
@@ -207,6 +223,10 @@ const char* fklcase_last_error(void) { return g_error; }
 // The next driver call on this thread enqueues its chain `reps` times back to back (through the full host API
 // each time); resets to 1 afterwards.
 void fklcase_set_reps(int reps) { g_reps = reps > 0 ? reps : 1; }
+// The next driver call on this thread records `first` on `stream` before its first launch and `last` after its last one.
+void fklcase_time_next(void* stream, void* first, void* last) { g_timing = Timing{stream, first, last, true, 0}; }
+// CLOCK_MONOTONIC at the start of the last timed driver call, in nanoseconds.
+long long fklcase_timed_start_ns(void) { return g_timing.start_ns; }
 
 int fklcase_crop_resize_par_u8_b5(void* stream, const uint8_t* src, int w, int h, int pitch, const int32_t* rects, int dw,
                                   int dh, const float* bg, const float* mul, const float* sub, uint8_t* out) {

@@ -24,6 +24,8 @@ def cases() -> C.CDLL:
             raise RuntimeError(f"{CASES_SO} is missing: run __graft_entry__.build()")
         c = C.CDLL(CASES_SO)
         c.fklcase_last_error.restype = C.c_char_p
+        c.fklcase_timed_start_ns.restype = C.c_longlong
+        c.fklcase_time_next.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         _cases = c
     return _cases
 
@@ -38,6 +40,16 @@ def _ok(rc: int) -> None:
 def set_reps(reps: int) -> None:
     """The next chain call enqueues its kernel `reps` times back to back through the C++ host API."""
     cases().fklcase_set_reps(int(reps))
+
+
+def time_next(stream, first_event, last_event) -> None:
+    """The next chain call records `first_event` on `stream` before its first launch and `last_event` after its last."""
+    cases().fklcase_time_next(stream, first_event, last_event)
+
+
+def timed_start_ns() -> int:
+    """CLOCK_MONOTONIC (nanoseconds) at the start of the last chain call that was timed with time_next."""
+    return int(cases().fklcase_timed_start_ns())
 
 
 def _stream():
