@@ -7,9 +7,10 @@ BGR->RGB -> (x - mean) / std -> planar float32 64x3x224x224), issued through the
 (executeOperations<TransformDPP<>>) -> C ABI -> one gfx950 kernel.
 
 Every measurement is W warm-up steps, a synchronisation, and then exactly K timed steps back to back on one stream.  The
-first launches after a synchronisation reach the GPU slowly (the runtime's first submissions after an idle queue take
-about 15 us each on the host), so a short run (K = 20) reads about 10 % above a long one (K = 200); `kernel_us_5_runs_*`
-of the headline shows four more runs of K steps without idle time in between.
+events (and the host clock) that bracket the K steps are taken by the case driver itself, right before its first launch
+and right after its last: this script needs about 100 us of Python to marshal a call's arguments, and with the bracket
+around the Python call a short run (K = 20) would charge that idle time to the kernel.  `kernel_us_5_runs_min_mean_max`
+of the headline shows the K steps repeated four more times.
 
 Prints ONE JSON line.  `value` is output Mpix/s of the whole job; `roofline` prices the kernel's algorithmic bytes
 against the 8 TB/s HBM peak using the launch duration measured with HIP events on the launch stream;
@@ -270,16 +271,18 @@ def main():
                    "sum_of_crop_areas_bytes": int(sum(int(r[2]) * int(r[3]) for r in c3["rects"])) * 3},
         "roofline": {"bound": "hbm", "achieved": r3["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": r3["frac_of_hbm_peak"], "traffic": TRAFFIC_C3_BYTES,
-                     "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"]},
+                     "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"],
+                     "kernel_us_5_runs_min_mean_max": r3["kernel_us_5_runs_min_mean_max"]},
         "cpu_baseline": cpu,
         "others": {k: v for k, v in results.items() if k != "c3"},
     }
     print(json.dumps(line))
 
 
-# HBM bytes one launch of configuration 3 moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE scaled by what the
-# same counters read for the plain copy chain of known size (profiles/k_gather_config3_traffic.txt); None until measured.
-TRAFFIC_C3_BYTES = 51193000
+# HBM bytes one launch of configuration 3 moves: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this script, scaled by what the
+# same counters read for its plain copy chain of known size.  Measured once, not in this run (the counters need the
+# profiler attached): profiles/k_strip_config3.txt holds the commands and the readings (run of 2026-11-25, fkd::k_strip).
+TRAFFIC_C3_BYTES = 52599000
 
 if __name__ == "__main__":
     main()
