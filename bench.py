@@ -44,6 +44,8 @@ def parse():
                     help="print to stderr the kernel symbol and signature of every chain compiled at run time")
     ap.add_argument("--issue-rate", action="store_true",
                     help="run the stand-alone instruction-issue measurement (fusedkernellibrary_amd/probe_issue_rate) and exit")
+    ap.add_argument("--uchar3-access", action="store_true",
+                    help="run the stand-alone comparison of access forms for uchar3 rows (fusedkernellibrary_amd/probe_uchar3_rows) and exit")
     ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
@@ -80,9 +82,9 @@ class Timer:
 
 def main():
     args = parse()
-    if args.issue_rate:
+    if args.issue_rate or args.uchar3_access:
         import subprocess
-        probe = os.path.join(ROOT, "fusedkernellibrary_amd", "probe_issue_rate")
+        probe = os.path.join(ROOT, "fusedkernellibrary_amd", "probe_issue_rate" if args.issue_rate else "probe_uchar3_rows")
         if not os.path.exists(probe):
             print(f"bench.py: {probe} is missing: build it with `python -m fusedkernellibrary_amd.build`", file=sys.stderr)
             sys.exit(1)
