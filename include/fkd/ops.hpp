@@ -1363,6 +1363,8 @@ template <class T> struct Read2D {
     // once per wave, a prepared column once per lane, a scalar offset per row.
     static constexpr bool kTapPrepared = true;
     FKD_DEV static bool tap_rows_share_alignment(const Params& p) { return p.pitch % 4 == 0 && size_t(p.pitch) * p.height < 0xfffffff0ull; }
+    // Every byte offset inside the image fits 32 bits (the buffer-resource forms of the tap accesses).
+    FKD_DEV static bool tap_offsets_fit(const Params& p) { return size_t(p.pitch) * p.height < 0xfffffff0ull; }
     using TapImage = detail::TapImage;
     using PairPrep = detail::PairPrep;
     FKD_DEV static TapImage tap_image(int, const Params& p) { return detail::make_tap_image(p.data); }
@@ -1750,6 +1752,9 @@ template <class Back> struct Crop {
     FKD_DEV static bool tap_rows_share_alignment(const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_rows_share_alignment(p.back); else return false;
     }
+    FKD_DEV static bool tap_offsets_fit(const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_offsets_fit(p.back); else return false;
+    }
     using TapImage = detail::TapImage;
     using PairPrep = detail::PairPrep;
     FKD_DEV static TapImage tap_image(int z, const Params& p) {
@@ -1883,6 +1888,9 @@ template <class Back, class... Ops> struct FusedRead {
     static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
     FKD_DEV static bool tap_rows_share_alignment(const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_rows_share_alignment(p.back); else return false;
+    }
+    FKD_DEV static bool tap_offsets_fit(const Params& p) {
+        if constexpr (kTapPrepared) return Back::tap_offsets_fit(p.back); else return false;
     }
     using TapImage = detail::TapImage;
     using PairPrep = detail::PairPrep;
@@ -2104,6 +2112,45 @@ template <int WT, class Back> struct Warp {
         }
         const int sw = Back::width(p.back), sh = Back::height(p.back);
         Out o;
+#if defined(FKD_DEVICE_CODE)
+        if constexpr (kPairTaps && detail::tap_prepared<Back>()) {
+            // Images below 4 GB (wave uniform): the two line-pair taps through a buffer resource that ends with the image.
+            // Row and column are one 32-bit byte offset per lane (no 64-bit address arithmetic on the vector unit), the
+            // window starts at the dword at or below it, and a window that reaches past the image's last row reads zeros
+            // in bytes nobody uses, so no wave needs the element-wise path.  Lanes whose source point lies outside take
+            // the taps of pixel (0, 0) and drop them, so that no load waits behind a branch.
+            if (sw >= 2 && Back::tap_offsets_fit(p.back)) {
+                const bool inside = sx >= 0.f && sx < f32(sw) && sy >= 0.f && sy < f32(sh);
+                const f32 cx = inside ? sx : 0.f, cy = inside ? sy : 0.f;
+                const int x1 = int(__builtin_floorf(cx)), y1 = int(__builtin_floorf(cy));
+                const int y2r = y1 + 1 < sh - 1 ? y1 + 1 : sh - 1;
+                const bool edge = x1 >= sw - 1;           // x1 + 1 is past the line: both taps are the last pixel
+                const int xp = edge ? sw - 2 : x1;
+                const detail::TapImage image = Back::tap_image_bounded(z, p.back);
+                const detail::PairPrep col = Back::pair_prepare(image, xp, p.back);
+                const u32 column_bytes = col.off + col.shift;             // from the resource's base
+                const u32 ta = column_bytes + Back::tap_row_offset(y1, p.back), tb = column_bytes + Back::tap_row_offset(y2r, p.back);
+                const auto wa = Back::pair_load_prepared(image, 0u, detail::PairPrep{ta & ~3u, ta & 3u}, p.back);
+                const auto wb = Back::pair_load_prepared(image, 0u, detail::PairPrep{tb & ~3u, tb & 3u}, p.back);
+                const f32 ax = f32(x1 + 1) - cx, bx = cx - f32(x1), ay = f32(y1 + 1) - cy, by = cy - f32(y1);
+                const f32 w00 = ax * ay, w10 = bx * ay, w01 = ax * by, w11 = bx * by;
+                typename Back::Raw a0, a1, b0, b1;
+                Back::pair_values(wa, typename Back::TapRow{}, xp, a0, a1);
+                Back::pair_values(wb, typename Back::TapRow{}, xp, b0, b1);
+                const Src a = Back::finish(edge ? a1 : a0, p.back), b = Back::finish(a1, p.back);
+                const Src c = Back::finish(edge ? b1 : b0, p.back), d = Back::finish(b1, p.back);
+                auto one = [&](auto pa, auto pb, auto pc, auto pd) {
+                    const f32 v = ((f32(pa) * w00 + f32(pb) * w10) + f32(pc) * w01) + f32(pd) * w11;
+                    return inside ? v : 0.f;
+                };
+                chan<0>(o) = one(chan<0>(a), chan<0>(b), chan<0>(c), chan<0>(d));
+                if constexpr (cn_v<Src> > 1) chan<1>(o) = one(chan<1>(a), chan<1>(b), chan<1>(c), chan<1>(d));
+                if constexpr (cn_v<Src> > 2) chan<2>(o) = one(chan<2>(a), chan<2>(b), chan<2>(c), chan<2>(d));
+                if constexpr (cn_v<Src> > 3) chan<3>(o) = one(chan<3>(a), chan<3>(b), chan<3>(c), chan<3>(d));
+                return o;
+            }
+        }
+#endif
         if constexpr (kPairTaps) {
             // Taps x1 and x1 + 1 of a source line in one access each, issued by every lane (lanes whose source point
             // lies outside take the taps of pixel (0, 0) and drop them), so that no load waits behind a branch.  A wave
