@@ -713,9 +713,14 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
             typename RZ::Taps tp;
             tp.w00 = ax * ay; tp.w10 = bx * ay; tp.w01 = ax * by; tp.w11 = bx * by;
             Raw a, b, c, d;
-            Back::pair_values(s.ab, typename Back::TapRow{}, 0, a, b);
-            Back::pair_values(s.cd, typename Back::TapRow{}, 0, c, d);
-            if constexpr (CLAMP) { if (s.e.w & kClamped) { a = b; c = d; } }
+            if constexpr (CLAMP) {
+                const bool clamped = (s.e.w & kClamped) != 0u;
+                Back::pair_values_dup(s.ab, clamped, a, b);
+                Back::pair_values_dup(s.cd, clamped, c, d);
+            } else {
+                Back::pair_values(s.ab, typename Back::TapRow{}, 0, a, b);
+                Back::pair_values(s.cd, typename Back::TapRow{}, 0, c, d);
+            }
             typename RZ::Out v = RZ::blend(Back::finish(a, q.back), Back::finish(b, q.back),
                                            Back::finish(c, q.back), Back::finish(d, q.back), tp);
             if constexpr (RZ::kAR != IGNORE_AR) { if (!yin || (s.e.w & kOutsideX)) v = q.bg; }

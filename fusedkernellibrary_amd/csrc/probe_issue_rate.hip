@@ -98,8 +98,8 @@ __global__ __launch_bounds__(256) void k_pixel(u32* out, int iters, u32 seed, f3
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             Px a, b, c, d;
-            fkd::detail::pair_window_values<Px>(top[i], a, b);
-            fkd::detail::pair_window_values<Px>(bot[i], c, d);
+            fkd::detail::pair_window_values(top[i], a, b);
+            fkd::detail::pair_window_values(bot[i], c, d);
             RZ::Taps tp;
             tp.w00 = axs[i] * ay; tp.w10 = bxs[i] * ay; tp.w01 = axs[i] * by; tp.w11 = bxs[i] * by;
             Out3 v = RZ::blend(a, b, c, d, tp);

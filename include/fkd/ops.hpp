@@ -520,7 +520,11 @@ template <class T> FKD_DEV PairWindow<T> load_prepared_pair_window(const TapImag
     return p;
 }
 #endif
-template <class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& first, T& second) {
+// DUP: lanes with `dup` set take the window's SECOND element for both values (a tap pair that ends at the image's last
+// column).  For 3-byte elements that is one byte permutation and one select on the aligned dwords (bytes 3,4,5,3 of the
+// first two dwords replace the first one; the second dword, which holds the second element's last two channels, stays);
+// for elements that are whole dwords it is a select per dword; other sizes select the unpacked values.
+template <bool DUP = false, class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& first, T& second, bool dup = false) {
     using PW = PairWindow<T>;
     u32 v[PW::kOut];
 #pragma unroll
@@ -528,6 +532,16 @@ template <class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& fi
         if constexpr (PW::kShift) v[i] = __builtin_amdgcn_alignbyte(p.w[i + 1 < PW::kWords ? i + 1 : i], p.w[i], p.shift);
         else v[i] = p.w[i];
         if constexpr (sizeof(base_t<T>) < 4) asm("" : "+v"(v[i]));   // keep dwords whole: v_cvt_f32_ubyteN / v_bfe
+    }
+    constexpr bool kDupBytes = DUP && sizeof(T) == 3, kDupWords = DUP && sizeof(T) % 4 == 0;
+    if constexpr (kDupBytes) {
+        const u32 twice = __builtin_amdgcn_perm(v[1], v[0], 0x03050403u);
+        v[0] = dup ? twice : v[0];
+        asm("" : "+v"(v[0]));
+    } else if constexpr (kDupWords) {
+        constexpr int E = int(sizeof(T)) / 4;
+#pragma unroll
+        for (int i = 0; i < E; ++i) v[i] = dup ? v[E + i] : v[i];
     }
     // channel by channel: copying whole 3-byte elements makes the compiler gather each into one register first
     // (v_perm_b32), although every channel leaves its dword through v_cvt_f32_ubyteN anyway
@@ -538,6 +552,7 @@ template <class T> FKD_DEV void pair_window_values(const PairWindow<T>& p, T& fi
     if constexpr (N > 1) { chan<1>(first) = unpack_elem<1, B>(v); chan<1>(second) = unpack_elem<N + 1, B>(v); }
     if constexpr (N > 2) { chan<2>(first) = unpack_elem<2, B>(v); chan<2>(second) = unpack_elem<N + 2, B>(v); }
     if constexpr (N > 3) { chan<3>(first) = unpack_elem<3, B>(v); chan<3>(second) = unpack_elem<N + 3, B>(v); }
+    if constexpr (DUP && !kDupBytes && !kDupWords) { if (dup) first = second; }
 }
 
 // Store counterpart of load_bits_at: element sizes 2 and multiples of 4 (up to 16) leave as one access.
@@ -1357,7 +1372,11 @@ template <class T> struct Read2D {
         return detail::load_pair_window<T>(r.p, u32(x) * u32(sizeof(T)));
     }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow&, int, Raw& first, Raw& second) {
-        detail::pair_window_values<T>(b, first, second);
+        detail::pair_window_values<false, T>(b, first, second);
+    }
+    // The same with lanes (`dup`) that take the second element for both values.
+    FKD_DEV static void pair_values_dup(const PairBits& b, bool dup, Raw& first, Raw& second) {
+        detail::pair_window_values<true, T>(b, first, second, dup);
     }
     // Buffer-resource form of pair_load for images whose rows share their alignment (see detail::TapImage): the image
     // once per wave, a prepared column once per lane, a scalar offset per row.
@@ -1574,12 +1593,28 @@ template <bool VU> struct ReadNV {
 #endif
 #if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        if constexpr (V == 4 && (A & 3) != 0) {
+            // four pixels: their luma is one dword, their two chroma pairs another (x is a multiple of four here)
+            const u32 luma = *detail::gconst<u32>(p.data + size_t(y) * p.pitch + x);
+            u32 uv = *detail::gconst<u32>(p.data + size_t(p.pitch) * p.height + size_t(y >> 1) * p.pitch + x);
+            u32 l = luma;
+            asm("" : "+v"(l), "+v"(uv));     // keep the dwords whole: bytes leave through v_cvt_f32_ubyteN / v_bfe
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+            for (int i = 0; i < 4; ++i) {
+                const u32 pair = uv >> (16 * (i >> 1));
+                out[i].v.x = u8((l >> (8 * i)) & 0xffu);
+                out[i].v.y = u8((pair >> (VU ? 8 : 0)) & 0xffu);
+                out[i].v.z = u8((pair >> (VU ? 0 : 8)) & 0xffu);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+        }
     }
     using Raw = Out;
     FKD_DEV static Out finish(const Raw& r, const Params&) { return r; }
-    FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // gathers element-wise either way
+    // Whole-dword row reads need luma and chroma rows that start on dword boundaries and a run that starts on a group of four.
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && xoff % 4 == 0; }
     static constexpr bool kTapOverread = true;    // pair_load only; tap_load reads exact bytes
     struct TapRow { const char* luma; const char* chroma; int x0; bool last; };
     FKD_DEV static TapRow tap_row(int x0, int y, int, const Params& p) {
@@ -1680,10 +1715,52 @@ template <int PF> struct ReadYUV {
 #endif
 #if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        if constexpr (V == 4 && (A & 3) != 0) {
+            // Four pixels as whole dwords (x is a multiple of four here): packed 4:2:2 holds them in two groups of four
+            // samples, semi-planar formats in four luma samples and two chroma pairs.
+            constexpr int S = int(sizeof(B));                 // bytes per sample
+            constexpr int kBits = 8 * S;
+            constexpr u32 kMask = S == 1 ? 0xffu : 0xffffu;
+            auto sample = [&](const u32* w, int k) { return B((w[k * S / 4] >> ((k * kBits) & 31)) & kMask); };
+            if constexpr (L::kSemiPlanar) {
+                u32 l[S], c[S];
+                const u8* lp = p.data + size_t(y) * p.pitch + size_t(x) * S;
+                const u8* cp = p.data + size_t(p.pitch) * p.height + size_t(L::k420 ? y >> 1 : y) * p.pitch + size_t(x) * S;
+                if constexpr (S == 1) { l[0] = *detail::gconst<u32>(lp); c[0] = *detail::gconst<u32>(cp); }
+                else {
+                    const detail::u32x2_t a = *detail::gconst<detail::u32x2_a4>(lp), b = *detail::gconst<detail::u32x2_a4>(cp);
+                    l[0] = a.x; l[1] = a.y; c[0] = b.x; c[1] = b.y;
+                }
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+                for (int i = 0; i < S; ++i) asm("" : "+v"(l[i]), "+v"(c[i]));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    out[i].v.x = sample(l, i);
+                    out[i].v.y = sample(c, 2 * (i >> 1) + (L::kSwapUV ? 1 : 0));
+                    out[i].v.z = sample(c, 2 * (i >> 1) + (L::kSwapUV ? 0 : 1));
+                }
+            } else {
+                u32 g[2 * S];
+                const u8* gp = p.data + size_t(y) * p.pitch + size_t(x) * 2 * S;
+                if constexpr (S == 1) { const detail::u32x2_t a = *detail::gconst<detail::u32x2_a4>(gp); g[0] = a.x; g[1] = a.y; }
+                else { const detail::u32x4_t a = *detail::gconst<detail::u32x4_a4>(gp); g[0] = a.x; g[1] = a.y; g[2] = a.z; g[3] = a.w; }
+#pragma unroll
+                for (int i = 0; i < 2 * S; ++i) asm("" : "+v"(g[i]));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int base = 4 * (i >> 1);            // first sample of the pixel's group: U Y0 V Y1 (UYVY) or Y0 U Y1 V (Y210)
+                    const bool even = (i & 1) == 0;
+                    if constexpr (PF == PF_UYVY) { out[i].v.x = sample(g, base + (even ? 1 : 3)); out[i].v.y = sample(g, base); out[i].v.z = sample(g, base + 2); }
+                    else { out[i].v.x = sample(g, base + (even ? 0 : 2)); out[i].v.y = sample(g, base + 1); out[i].v.z = sample(g, base + 3); }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
+        }
     }
-    FKD_HD static bool rows_aligned(const Params&, int) { return true; }   // element-wise either way
+    // Whole-dword row reads need rows that start on dword boundaries and a run that starts on a group of four pixels.
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return detail::dword_aligned(p.data) && p.pitch % 4 == 0 && xoff % 4 == 0; }
     // No tap cursor: a bilinear resize over this read takes its taps through exec().  The names below only let the
     // wrappers that forward a cursor (Crop, FusedRead) be formed around this read.
     using Raw = Out;
@@ -1748,6 +1825,10 @@ template <class Back> struct Crop {
     using PairBits = typename detail::TapTypesOf<Back>::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
+    FKD_DEV static void pair_values_dup(const PairBits& b, bool dup, Raw& first, Raw& second) {
+        if constexpr (requires { Back::pair_values_dup(b, dup, first, second); }) Back::pair_values_dup(b, dup, first, second);
+        else { Back::pair_values(b, TapRow{}, 0, first, second); if (dup) first = second; }
+    }
     static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
     FKD_DEV static bool tap_rows_share_alignment(const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_rows_share_alignment(p.back); else return false;
@@ -1885,6 +1966,10 @@ template <class Back, class... Ops> struct FusedRead {
     using PairBits = typename detail::TapTypesOf<Back>::PairBits;
     FKD_DEV static PairBits pair_load(const TapRow& r, int x, const Params& p) { return Back::pair_load(r, x, p.back); }
     FKD_DEV static void pair_values(const PairBits& b, const TapRow& r, int x, Raw& first, Raw& second) { Back::pair_values(b, r, x, first, second); }
+    FKD_DEV static void pair_values_dup(const PairBits& b, bool dup, Raw& first, Raw& second) {
+        if constexpr (requires { Back::pair_values_dup(b, dup, first, second); }) Back::pair_values_dup(b, dup, first, second);
+        else { Back::pair_values(b, TapRow{}, 0, first, second); if (dup) first = second; }
+    }
     static constexpr bool kTapPrepared = detail::tap_prepared<Back>();
     FKD_DEV static bool tap_rows_share_alignment(const Params& p) {
         if constexpr (kTapPrepared) return Back::tap_rows_share_alignment(p.back); else return false;
