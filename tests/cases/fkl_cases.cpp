@@ -395,6 +395,31 @@ int fklcase_uncompiled_letterbox_split_b3(void* stream_, const uint8_t* src, int
             TensorSplit<float3>::build(o.ptr()));
     });
 }
+// crop of an image of 2-, 4- or 6-byte pixels (uchar2, uchar4, ushort3) -> bilinear resize -> Mul by a scalar -> planar float
+// tensor: narrow planar outputs of pixel types other than uchar3 (the strip form's other ways of handling a clamped tap pair)
+extern "C++" {
+template <typename Px, typename Fx>
+void resize_split_of(void* stream_, const void* src, int w, int h, int pitch, const int32_t* rect, int dw, int dh, float mul, float* out) {
+    Stream stream(stream_);
+    const auto in = dev2d<Px>(src, w, h, pitch);
+    Tensor<float> o(out, uint(dw), uint(dh), 1u, cn<Px>, MemType::Device, 0);
+    executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, Px>::build(in.ptr()),
+                                      Crop<>::build(Rect(rect[0], rect[1], rect[2], rect[3])),
+                                      Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)), Mul<Fx, float, Fx>::build(mul),
+                                      TensorSplit<Fx>::build(o.ptr()));
+}
+}   // extern "C++"
+int fklcase_uncompiled_resize_split(void* stream_, int kind, const void* src, int w, int h, int pitch, const int32_t* rect, int dw, int dh,
+                                    float mul, float* out) {
+    return guarded([&] {
+        switch (kind) {
+        case 0: resize_split_of<uchar2, float2>(stream_, src, w, h, pitch, rect, dw, dh, mul, out); break;
+        case 1: resize_split_of<uchar4, float4>(stream_, src, w, h, pitch, rect, dw, dh, mul, out); break;
+        case 2: resize_split_of<ushort3, float3>(stream_, src, w, h, pitch, rect, dw, dh, mul, out); break;
+        default: throw std::runtime_error("fklcase_uncompiled_resize_split: kind must be 0 (uchar2), 1 (uchar4) or 2 (ushort3)");
+        }
+    });
+}
 // float4 image -> bilinear resize -> float4 image (16-byte elements: one access per tap)
 int fklcase_uncompiled_float4_resize(void* stream_, const float* in, int w, int h, int pitch, int dw, int dh, float* out, int out_pitch) {
     return guarded([&] {

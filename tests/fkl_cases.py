@@ -214,6 +214,13 @@ def uncompiled_letterbox_split_b3(src, rects, dst, bg, mul, out):
                                                       b.ctypes.data_as(C.c_void_p), m.ctypes.data_as(C.c_void_p), _p(out)))
 
 
+def uncompiled_resize_split(kind, src, rect, dst, mul, out):
+    """kind 0: (H,W,2) u8, 1: (H,W,4) u8, 2: (H,W,3) u16 cuda -> crop -> bilinear (dst = (w,h)) -> * mul -> out (cn,dh,dw) f32 cuda."""
+    r = _host(rect, np.int32)
+    _ok(cases().fklcase_uncompiled_resize_split(_stream(), int(kind), _p(src), src.shape[1], src.shape[0], src.stride(0) * src.element_size(),
+                                                r.ctypes.data_as(C.c_void_p), int(dst[0]), int(dst[1]), C.c_float(float(mul)), _p(out)))
+
+
 def uncompiled_float4_resize(src, dst, out):
     """(H,W,4) f32 cuda -> bilinear -> out (dh,dw,4) f32 cuda."""
     _ok(cases().fklcase_uncompiled_float4_resize(_stream(), _p(src), src.shape[1], src.shape[0], src.stride(0) * 4, int(dst[0]), int(dst[1]),

@@ -145,6 +145,30 @@ def test_letterboxed_chain_compiled_on_first_use(device, dst):
     assert results[False].tobytes() == want.tobytes()
 
 
+@pytest.mark.parametrize("kind,cn,dtype", [(0, 2, np.uint8), (1, 4, np.uint8), (2, 3, np.uint16)])
+@pytest.mark.parametrize("dst,rect", [((200, 40), (10, 5, 60, 90)),       # enlarging: the last columns repeat the crop's last pixel
+                                      ((64, 64), (0, 0, 160, 120)),       # reducing, the whole image
+                                      ((33, 9), (158, 117, 2, 3))])        # the image's last rows and columns
+def test_other_pixel_types_compiled_on_first_use(device, kind, cn, dtype, dst, rect):
+    """2-, 4- and 6-byte pixels: the tap pair of a clamped column is handled per element size (dword select for 4 bytes, on
+    the unpacked values otherwise)."""
+    import torch
+    rng = np.random.RandomState(90 + kind)
+    w, h = 160, 120
+    img = rng.randint(0, 1024 if dtype == np.uint16 else 256, (h, w, cn)).astype(dtype)
+    src = torch.from_numpy(img.view(np.int16) if dtype == np.uint16 else img).to(device)
+    want = np.zeros((cn, dst[1], dst[0]), np.float32)
+    ol.execute([ol.read_2d(img, cn, crop=rect, resize=dst, ar=ol.IGNORE_AR)], [ol.op(ol.MUL, (0.5, 0.5, 0.5, 0.5))],
+               [ol.write(ol.TENSOR_SPLIT, want, cn, dst[0], dst[1], 1, cn)])
+    for on in (True, False):
+        with strip_switched(on):
+            out = torch.full((cn, dst[1], dst[0]), -7.0, dtype=torch.float32, device=device)
+            cases.uncompiled_resize_split(kind, src, rect, dst, 0.5, out)
+            torch.cuda.synchronize()
+            assert last_launch()["kernel"] == ("strip_jit" if on else "gather_jit")
+            assert out.cpu().numpy().tobytes() == want.tobytes(), (kind, dst, rect, on)
+
+
 def test_configuration_3_takes_the_strip_form(device):
     import torch
     c = wl.config3()
