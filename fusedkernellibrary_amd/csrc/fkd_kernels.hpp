@@ -811,7 +811,10 @@ template <class Chain> struct RowsConfig {
     // Two rows per thread; chains long enough to be bound by instruction issue rather than by memory (more than 128
     // bytes of operation parameters) take four, for the independent work per thread.
     static constexpr bool kManyOps = sizeof(typename Chain::Params) - sizeof(typename Chain::Read::Params) - sizeof(typename Chain::Write::Params) > 128 + 16;
-    static constexpr int ROWS = kScattered ? FKD_SCATTER_ROWS : (kManyOps ? 2 * FKD_ROWS : FKD_ROWS);
+#ifndef FKD_ROWS_MANY
+#define FKD_ROWS_MANY (2 * FKD_ROWS)
+#endif
+    static constexpr int ROWS = kScattered ? FKD_SCATTER_ROWS : (kManyOps ? FKD_ROWS_MANY : FKD_ROWS);
 };
 
 // ---- divergent batch kernel -------------------------------------------------------------------------------
