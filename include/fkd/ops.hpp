@@ -879,6 +879,17 @@ template <class I, class O> struct Cast {
     }
 };
 
+// IsEven<I>: per channel, whether an integer is even; the answer is a byte holding 0 or 1 (the layout of a host bool).
+// FK/algorithms/basic_ops/logical.h:23-35.
+template <class I> struct IsEven {
+    static_assert(base_t<I>(1) / base_t<I>(2) == base_t<I>(0), "integer channels only");
+    using In = I; using Out = vec_t<u8, cn_v<I>>; using Params = Empty;
+    FKD_NAME("IsEven<" + type_name<I>() + ">")
+    FKD_DEV static Out exec(const I& a, const Params&) {
+        return map1<Out>(a, [](auto x) { return u8((x & 1) == 0 ? 1 : 0); });
+    }
+};
+
 // VectorReorder<T,i0,i1,i2,i3>: out[c] = in[idx[c]] (BGR<->RGB is 2,1,0).  FK/algorithms/basic_ops/vector_ops.h:43-56,
 // reached through ColorConversion<COLOR_BGR2RGB,...>, FK/algorithms/image_processing/color_conversion.h:472-476.
 template <class T, int I0, int I1, int I2 = 2, int I3 = 3> struct Reorder {
@@ -981,10 +992,11 @@ template <> struct DepthConsts<CD_FN12> {
 // weights Kr, Kb of the primaries (itu_color.h:150-158), then the limited-range scaling of the luma and chroma
 // columns (to RGB) or rows (to YCbCr).  All binary32, in the reference's expression order, evaluated at compile time.
 struct ColorMatrix { f32 m[9]; };
+constexpr f32 luma_weight_red(int cp) { return cp == CP_BT601 ? 0.299f : (cp == CP_BT709 ? 0.2126f : 0.2627f); }
+constexpr f32 luma_weight_blue(int cp) { return cp == CP_BT601 ? 0.114f : (cp == CP_BT709 ? 0.0722f : 0.0593f); }
 template <int CD, int CR, int CP, bool TO_RGB> constexpr ColorMatrix color_matrix() {
     static_assert(CP >= 0 && CP <= 2 && (CR == CR_LIMITED || CR == CR_FULL), "unknown colour primaries or range");
-    constexpr f32 Kr = CP == CP_BT601 ? 0.299f : (CP == CP_BT709 ? 0.2126f : 0.2627f);
-    constexpr f32 Kb = CP == CP_BT601 ? 0.114f : (CP == CP_BT709 ? 0.0722f : 0.0593f);
+    constexpr f32 Kr = luma_weight_red(CP), Kb = luma_weight_blue(CP);
     constexpr f32 Kg = 1.0f - Kr - Kb;
     using D = DepthConsts<CD>;
     ColorMatrix c{};

@@ -1,6 +1,7 @@
 // Equal<T>: host-side comparison of two values (all channels equal), the helper the reference's benchmarks and tests
-// use to compare results they have downloaded.  Interface counterpart: FK/algorithms/basic_ops/logical.h:92-120.
-// IsEven, Max and Min of that header have no MI355X kernel and are not provided.
+// use to compare results they have downloaded; IsEven<I>: whether an integer (each channel of an integer vector) is
+// even.  Interface counterpart: FK/algorithms/basic_ops/logical.h:23-35, 92-120.
+// Max and Min of that header have no MI355X kernel and are not provided.
 #ifndef FK_AMD_LOGICAL_H
 #define FK_AMD_LOGICAL_H
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
@@ -11,5 +12,18 @@ template <typename I1, typename I2 = I1> struct Equal : UnaryOperation<Tuple<I1,
     FK_STATIC_STRUCT(Equal, Equal)
     static constexpr bool exec(const Tuple<I1, I2>& input) { return static_cast<bool>(get<0>(input) == get<1>(input)); }
 };
+
+template <typename I> struct IsEven : UnaryOperation<I, VectorType_t<bool, cn<I>>, IsEven<I>> {
+    static_assert(std::is_integral_v<VBase<I>>, "IsEven works on integers and vectors of integers");
+    using Parent = UnaryOperation<I, VectorType_t<bool, cn<I>>, IsEven<I>>;
+    FK_STATIC_STRUCT(IsEven, IsEven)
+};
+namespace amd {
+template <typename I> struct Lower<IsEven<I>> {
+    static constexpr bool available = true;
+    using type = fkd::IsEven<dev_t<I>>;
+    static typename type::Params params(const OperationData<IsEven<I>>&) { return {}; }
+};
+} // namespace amd
 } // namespace fk
 #endif

@@ -92,6 +92,9 @@ template <typename T> struct operation_of<T, true> { using type = typename T::Op
 // Works on Operations and on IOps alike.
 template <typename Tag, typename T> constexpr bool opIs = op_detail::op_is<Tag, std::decay_t<T>>::value;
 template <typename T> constexpr bool isOperation = op_detail::has_instance<std::decay_t<T>>::value;
+// The class-template spellings of the same tests (FK/core/execution_model/operation_model/operation_types.h:79-91).
+template <typename Tag, typename T, typename = void> struct OpIs : std::bool_constant<opIs<Tag, T>> {};
+template <typename T, typename = void> struct HasInstanceType : std::bool_constant<isOperation<T>> {};
 template <typename T> constexpr bool isAnyReadType = opIs<ReadType, T> || opIs<ReadBackType, T> || opIs<IncompleteReadBackType, T>;
 template <typename T> constexpr bool isCompleteOperation =
     isOperation<T> && !opIs<IncompleteReadBackType, T> &&
@@ -194,6 +197,7 @@ namespace amd {
 
 // fk element type -> fkd element type
 template <typename T> struct DevType { using type = T; };
+template <> struct DevType<bool> { using type = fkd::u8; };   // one byte holding 0 or 1
 template <> struct DevType<unsigned char> { using type = fkd::u8; };
 template <> struct DevType<signed char> { using type = fkd::i8; };
 template <> struct DevType<char> { using type = fkd::i8; };
@@ -220,6 +224,20 @@ template <typename V> dev_t<V> to_dev(const V& v) {
         if constexpr (cn<V> > 3) fkd::chan<3>(d) = v.w;
     }
     return d;
+}
+
+// ... and back: a device value as the host type V.
+template <typename V> V from_dev(const dev_t<V>& d) {
+    if constexpr (!isVector<V>) {
+        return static_cast<V>(d);
+    } else {
+        V v{};
+        v.x = static_cast<VBase<V>>(fkd::chan<0>(d));
+        if constexpr (cn<V> > 1) v.y = static_cast<VBase<V>>(fkd::chan<1>(d));
+        if constexpr (cn<V> > 2) v.z = static_cast<VBase<V>>(fkd::chan<2>(d));
+        if constexpr (cn<V> > 3) v.w = static_cast<VBase<V>>(fkd::chan<3>(d));
+        return v;
+    }
 }
 
 template <typename T, typename Q = T> fkd::RawPtr2D<Q> to_dev(const RawPtr<ND::_2D, T>& p) {
@@ -275,6 +293,12 @@ template <typename I, typename O, typename Child_, bool IS_FUSED = false> struct
     using InstantiableType = Unary<Child_>;
     static constexpr bool IS_FUSED_OP = IS_FUSED;
     static constexpr InstantiableType build() { return {}; }
+    // The Operation applied to one value on the calling thread (the reference's Operations are host functions too): the
+    // body is the device operation's own, compiled for the host.  An Operation that defines its own exec hides this one.
+    template <typename C = Child_> static OutputType exec(const InputType& input) {
+        using L = amd::Lower<C>;
+        return amd::from_dev<OutputType>(L::type::exec(amd::to_dev(input), L::params(OperationData<C>{})));
+    }
 };
 
 template <typename I, typename P, typename O, typename Child_, bool IS_FUSED = false> struct BinaryOperation {
@@ -288,6 +312,14 @@ template <typename I, typename P, typename O, typename Child_, bool IS_FUSED = f
     static constexpr bool IS_FUSED_OP = IS_FUSED;
     static constexpr InstantiableType build(const OperationDataType& opData) { return {opData}; }
     static constexpr InstantiableType build(const ParamsType& params) { return {{params}}; }
+    // (see UnaryOperation::exec)
+    template <typename C = Child_> static OutputType exec(const InputType& input, const ParamsType& params) {
+        using L = amd::Lower<C>;
+        return amd::from_dev<OutputType>(L::type::exec(amd::to_dev(input), L::params(OperationData<C>{params})));
+    }
+    template <typename C = Child_> static OutputType exec(const InputType& input, const OperationData<C>& opData) {
+        return exec<C>(input, opData.params);
+    }
 };
 
 template <typename I, typename P, typename BIOp, typename O, typename Child_, bool IS_FUSED = false> struct TernaryOperation {

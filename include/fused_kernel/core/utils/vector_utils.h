@@ -4,6 +4,8 @@
 #ifndef FK_AMD_VECTOR_UTILS_H
 #define FK_AMD_VECTOR_UTILS_H
 
+#include <cmath>
+#include <utility>
 #include <type_traits>
 
 #include <fused_kernel/core/data/vector_types.h>

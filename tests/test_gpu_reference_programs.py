@@ -16,11 +16,27 @@ TESTS = ["tests_algorithm_test_crop", "tests_algorithm_test_batchresize_build", 
          "tests_algorithm_test_warp", "tests_algorithm_test_border_reader", "tests_data_test_ptr_nd", "tests_data_test_rect",
          "tests_data_test_circular_tensor", "tests_data_parallel_patterns_test_divergent_batch",
          "tests_examples_compiler_explorer_example", "tests_buildAPI_batch_build_compilation_time",
-         "tests_operation_test_cricular_batch", "tests_examples_readme_test_code", "utests_core_execution_model_utest_executors"]
+         "tests_operation_test_cricular_batch", "tests_examples_readme_test_code", "utests_core_execution_model_utest_executors",
+         "tests_string_test_IOps_to_string",
+         # the reference's unit tests of the colour operations (every case goes through Executor<TransformDPP<>>, that is
+         # through a kernel compiled at run time; its literal conversion matrices are compared at compile time with the
+         # ones this library computes) and of Deinterlace
+         "utests_algorithm_image_processing_utest_color_conversion", "utests_algorithm_image_processing_utest_deinterlace"]
 # host-only logic (no device call): also run where there is no GPU
-HOST_TESTS = ["tests_thread_fusion_test_thread_fusion"]
+HOST_TESTS = ["tests_thread_fusion_test_thread_fusion", "tests_string_test_struct_to_string", "tests_string_test_literal_to_string"]
 BENCHMARKS = ["benchmarks_fusion_benchmark_horizontal_fusion", "benchmarks_fusion_benchmark_thread_fusion",
               "benchmarks_latencyhiding_benchmark_latency_hiding", "benchmarks_numinstructions_benchmark_numinstructions_x_operation"]
+
+
+# One expectation in the reference's colour unit test contradicts the reference's own code: SaturateDenormalizePixel
+# <float3, uchar3, p8bit> of 0.5 is static_cast<uchar>(0.5f * 255) = 127 (color_conversion.h:108-120, 137-150; the test's
+# other expectations, 63.75 -> 63 and 229.5 -> 229, truncate too), the test's table says 128
+# (utest_color_conversion.h:282-296).  The reference's CPU backend returns 127 as well (tests/test_oracle_depth_and_
+# transposed.py).  That case, and only that case, may fail; every other case of the program has to succeed.
+KNOWN_REFERENCE_DEFECTS = {
+    "utests_algorithm_image_processing_utest_color_conversion":
+        ("fk::SaturateDenormalizePixel<fk::Float3, fk::Uchar3, (fk::ColorDepth)0>", "index 0 for vector index 1: Expected value 128, got 127"),
+}
 
 
 def run_program(name, tmp_path):
@@ -28,6 +44,13 @@ def run_program(name, tmp_path):
     if not os.path.exists(exe):
         pytest.skip("oracle/_ref/programs was not built (needs the reference tree at build time)")
     r = subprocess.run([exe], cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    if name in KNOWN_REFERENCE_DEFECTS:
+        case, message = KNOWN_REFERENCE_DEFECTS[name]
+        cases = [c for c in r.stdout.split("Running test for ")[1:]]
+        failed = [c for c in cases if "Success!!" not in c]
+        assert len(cases) >= 10 and len(failed) == 1 and case in failed[0] and message in failed[0] \
+            and failed[0].count("Mismatch") == 1, f"{name}\n{r.stdout[-3000:]}\n{r.stderr[-2000:]}"
+        return r.stdout.replace(failed[0], "")
     assert r.returncode == 0, f"{name} exited with {r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
     return r.stdout
 
