@@ -879,6 +879,80 @@ template <class I, class O> struct Cast {
     }
 };
 
+// ---- the per-channel functions of the reference's basic_ops headers that a chain may hold between read and write ----
+// math.h:26-170 (Abs, Sqr, Sqrt, Ln, Exp, AbsDiff), logical.h:37-88 (Max, Min), bitwise.h:23-157 (BwAnd, BwOr, BwXor,
+// BwNot, ShiftLeft, ShiftRight).  Each is a C++ expression on one channel (and on the matching channel of a launch
+// constant, a scalar constant being broadcast), evaluated in the types the expression promotes to and converted to the
+// output's channel type: FK/core/constexpr_libs/constexpr_vector_exec.h:24-108 (cxp::Exec) and the channel-wise operators
+// of FK/core/utils/vector_utils.h:508-600.  Map1 / Map2 carry the function as a type.
+namespace fn {
+#define FKD_FN(text) FKD_NAME(text)
+struct Abs {      // s < 0 ? -s : s for signed channel types, s for unsigned ones (so -0.f and NaN come back unchanged)
+    FKD_FN("fn::Abs")
+    template <class T> FKD_HD static auto apply(T s) {
+        if constexpr (T(-1) < T(0)) return s < T(0) ? static_cast<T>(-s) : s;
+        else return s;
+    }
+};
+struct Sqr { FKD_FN("fn::Sqr") template <class T> FKD_HD static auto apply(T s) { return s * s; } };
+// sqrtf / logf / expf of the channel converted to float.  The square root is correctly rounded on both sides; the
+// logarithm and the exponential are the platform's, so device and host agree to a few units in the last place.
+struct Sqrt { FKD_FN("fn::Sqrt") template <class T> FKD_HD static f32 apply(T s) { return __builtin_sqrtf(static_cast<f32>(s)); } };
+struct Ln { FKD_FN("fn::Ln") template <class T> FKD_HD static f32 apply(T s) { return __builtin_logf(static_cast<f32>(s)); } };
+struct Exp { FKD_FN("fn::Exp") template <class T> FKD_HD static f32 apply(T s) { return __builtin_expf(static_cast<f32>(s)); } };
+struct BwNot { FKD_FN("fn::BwNot") template <class T> FKD_HD static auto apply(T s) { return ~s; } };
+// std::max / std::min of two values of ONE type: (a < b) ? b : a and (b < a) ? b : a, so a NaN input comes back and a NaN
+// constant never does.
+struct Max { FKD_FN("fn::Max") template <class T> FKD_HD static T apply(T a, T b) { return (a < b) ? b : a; } };
+struct Min { FKD_FN("fn::Min") template <class T> FKD_HD static T apply(T a, T b) { return (b < a) ? b : a; } };
+struct AbsDiff {
+    FKD_FN("fn::AbsDiff")
+    template <class A, class B> FKD_HD static auto apply(A a, B b) {
+        const auto d = a - b;
+        return d < decltype(d)(0) ? -d : d;
+    }
+};
+struct BwAnd { FKD_FN("fn::BwAnd") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a & b; } };
+struct BwOr { FKD_FN("fn::BwOr") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a | b; } };
+struct BwXor { FKD_FN("fn::BwXor") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a ^ b; } };
+struct ShiftLeft { FKD_FN("fn::ShiftLeft") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a << b; } };
+struct ShiftRight { FKD_FN("fn::ShiftRight") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a >> b; } };
+#undef FKD_FN
+} // namespace fn
+template <class F, class I, class O> struct Map1 {
+    static_assert(cn_v<I> == cn_v<O>, "one output channel per input channel");
+    using In = I; using Out = O; using Params = Empty;
+    FKD_NAME("Map1<" + F::name() + "," + type_name<I>() + "," + type_name<O>() + ">")
+    FKD_DEV static O exec(const I& a, const Params&) {
+        return map1<O>(a, [](auto x) { return static_cast<base_t<O>>(F::apply(x)); });
+    }
+};
+template <class F, class I, class P, class O> struct Map2 {
+    static_assert(cn_v<I> == cn_v<O> && (cn_v<P> == cn_v<I> || cn_v<P> == 1), "a constant per channel, or one for all");
+    using In = I; using Out = O;
+    struct Params { P v; };
+    static constexpr bool kValueParams = true;
+    FKD_NAME("Map2<" + F::name() + "," + type_name<I>() + "," + type_name<P>() + "," + type_name<O>() + ">")
+    FKD_DEV static O exec(const I& a, const Params& p) {
+        return map2<O>(a, p.v, [](auto x, auto y) { return static_cast<base_t<O>>(F::apply(x, y)); });
+    }
+};
+
+// MxVFloat3<BinaryType>: a float3 times a 3x3 matrix held row by row, per row three products summed as (a + b) + c.
+// FK/algorithms/basic_ops/algebraic.h:25-40.
+struct MxV3 {
+    using In = Vec<f32, 3>; using Out = Vec<f32, 3>;
+    struct Params { f32 m[9]; };
+    FKD_NAME("MxV3")
+    FKD_DEV static Out exec(const In& a, const Params& p) {
+        Out o;
+        o.x = (a.x * p.m[0] + a.y * p.m[1]) + a.z * p.m[2];
+        o.y = (a.x * p.m[3] + a.y * p.m[4]) + a.z * p.m[5];
+        o.z = (a.x * p.m[6] + a.y * p.m[7]) + a.z * p.m[8];
+        return o;
+    }
+};
+
 // IsEven<I>: per channel, whether an integer is even; the answer is a byte holding 0 or 1 (the layout of a host bool).
 // FK/algorithms/basic_ops/logical.h:23-35.
 template <class I> struct IsEven {

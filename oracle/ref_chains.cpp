@@ -15,6 +15,10 @@
 #include <fused_kernel/algorithms/basic_ops/memory_operations.h>
 #include <fused_kernel/algorithms/basic_ops/arithmetic.h>
 #include <fused_kernel/algorithms/basic_ops/cast.h>
+#include <fused_kernel/algorithms/basic_ops/math.h>
+#include <fused_kernel/algorithms/basic_ops/logical.h>
+#include <fused_kernel/algorithms/basic_ops/bitwise.h>
+#include <fused_kernel/algorithms/basic_ops/algebraic.h>
 #include <fused_kernel/algorithms/image_processing/crop.h>
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
@@ -36,6 +40,7 @@
 #include "../tests/cases/color_chains.h"
 #include "../tests/cases/border_chains.h"
 #include "../tests/cases/circular_chains.h"
+#include "../tests/cases/pointwise_chains.h"
 
 using namespace fk;
 using CpuDPP = TransformDPP<ParArch::CPU>;
@@ -401,6 +406,13 @@ int fklref_normalize(int which, const void* src, int w, int h, int pitch, float*
 int fklref_depth_ops(int which, const void* src, int w, int h, int pitch, void* out, int out_pitch, float lo, float hi) {
     CpuStream s;
     const int rc = RefColor::depth_ops(s, MemType::Host, which, src, w, h, pitch, out, out_pitch, lo, hi);
+    s.sync();
+    return rc;
+}
+// Operation number `which` of tests/cases/pointwise_chains.h on the CPU backend.
+int fklref_pointwise(int which, const void* src, int w, int h, int pitch, void* out, int out_pitch, const float* c, const float* m) {
+    CpuStream s;
+    const int rc = pointwise_chains::Chains<CpuDPP, CpuStream>::run(s, MemType::Host, which, src, w, h, pitch, out, out_pitch, c, m);
     s.sync();
     return rc;
 }

@@ -8,6 +8,10 @@
 #include <fused_kernel/algorithms/basic_ops/arithmetic.h>
 #include <fused_kernel/algorithms/basic_ops/cast.h>
 #include <fused_kernel/algorithms/basic_ops/static_loop.h>
+#include <fused_kernel/algorithms/basic_ops/math.h>
+#include <fused_kernel/algorithms/basic_ops/logical.h>
+#include <fused_kernel/algorithms/basic_ops/bitwise.h>
+#include <fused_kernel/algorithms/basic_ops/algebraic.h>
 #include <fused_kernel/core/data/ptr_utils.h>
 #include <fused_kernel/algorithms/image_processing/crop.h>
 #include <fused_kernel/algorithms/image_processing/color_conversion.h>
@@ -30,6 +34,7 @@
 #include "color_chains.h"   // pixel-format and colour-conversion chains, shared with the reference-backend harness
 #include "border_chains.h"  // padding chains, shared the same way
 #include "circular_chains.h"  // divergent launches and the CircularTensor window, shared the same way
+#include "pointwise_chains.h" // one per-channel Operation of math.h / logical.h / bitwise.h / algebraic.h, shared the same way
 
 #include <time.h>
 
@@ -569,6 +574,15 @@ int fklcase_depth_ops(void* stream_, int which, const void* src, int w, int h, i
 }
 
 } // extern "C"
+
+// ---- per-channel Operations (pointwise_chains.h on the GPU) --------------------------------------------------------
+extern "C" int fklcase_pointwise(void* stream_, int which, const void* src, int w, int h, int pitch, void* out, int out_pitch,
+                                 const float* c, const float* m) {
+    return guarded_rc([&] {
+        Stream s(stream_);
+        return pointwise_chains::Chains<TransformDPP<>, Stream>::run(s, MemType::Device, which, src, w, h, pitch, out, out_pitch, c, m);
+    });
+}
 
 // ---- padding through BorderReader (border_chains.h on the GPU) ----------------------------------------------------
 extern "C" int fklcase_pad(void* stream_, int elem, int border_type, const void* src, int w, int h, int pitch, int left, int top,

@@ -290,6 +290,15 @@ def depth_ops(which, src, out, lo=0.0, hi=1.0):
                                   C.c_float(float(lo)), C.c_float(float(hi))))
 
 
+def pointwise(which, src_bytes, width, height, out_bytes, c=(0, 0, 0, 0), m=(1, 0, 0, 0, 1, 0, 0, 0, 1)):
+    """Chain number `which` of tests/cases/pointwise_chains.h.  src_bytes / out_bytes: 2-D u8 cuda tensors holding `height`
+    rows of `width` elements of the chain's input / output type (a row may be longer than its elements: the pitch)."""
+    cv = np.ascontiguousarray(c, dtype=np.float32)
+    mv = np.ascontiguousarray(m, dtype=np.float32)
+    _ok(cases().fklcase_pointwise(_stream(), int(which), _p(src_bytes), int(width), int(height), _pitch(src_bytes), _p(out_bytes),
+                                  _pitch(out_bytes), cv.ctypes.data_as(C.c_void_p), mv.ctypes.data_as(C.c_void_p)))
+
+
 def pad(src, border_type, left, top, out, value=(0, 0, 0)):
     """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out."""
     v = np.zeros(4, np.float32)

@@ -684,6 +684,28 @@ def ref_depth_ops(which, src, lo=0.0, hi=1.0):
     return out
 
 
+# ---- per-channel Operations (tests/cases/pointwise_chains.h; numpy restatement: oracle/pointwise_oracle.py) ----------
+
+def pointwise_oracle():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("pointwise_oracle", os.path.join(ROOT, "oracle", "pointwise_oracle.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def ref_pointwise(which, src, c=(0, 0, 0, 0), m=(1, 0, 0, 0, 1, 0, 0, 0, 1)):
+    """Chain `which` of tests/cases/pointwise_chains.h on the reference's CPU backend (or, under host_executor, on this
+    repository's own CPU executor)."""
+    in_dtype, cn, out_dtype = pointwise_oracle().CASES[which]
+    src = np.ascontiguousarray(src, dtype=in_dtype)
+    out = np.zeros(src.shape, out_dtype)
+    rc = ref().fklref_pointwise(int(which), C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], C.c_void_p(_ptr(out)),
+                                out.strides[0], _f32p(np.asarray(c, np.float32)), _f32p(np.asarray(m, np.float32)))
+    assert rc == 0, rc
+    return out
+
+
 # ---- transposed tensors: TensorTSplit / TensorTPack --------------------------------------------------------------------
 
 def oracle_transposed_round_trip(images, mul, mul2):

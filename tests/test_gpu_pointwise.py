@@ -1,0 +1,61 @@
+"""GPU parity of the per-channel Operations of math.h / logical.h / bitwise.h / algebraic.h (Abs, Sqr, Sqrt, Ln, Exp, AbsDiff,
+Max, Min, BwAnd, BwOr, BwXor, BwNot, ShiftLeft, ShiftRight, MxVFloat3) in a chain Read -> Operation -> Write: the chain
+texts of tests/cases/pointwise_chains.h through the C++ host API and the C ABI, compiled at run time, against the numpy
+restatement (oracle/pointwise_oracle.py, itself pinned by the reference's CPU backend).  Bit-exact, except Ln and Exp:
+the platform's logf / expf, 1e-5 relative."""
+import numpy as np
+import pytest
+
+import fkl_cases as cases
+import oracle_lib as ol
+import pointwise_cases as pc
+
+po = ol.pointwise_oracle()
+ALL = sorted(po.CASES)
+
+
+def run_on_gpu(device, which, src, pad_in=0, pad_out=0):
+    import torch
+    in_dtype, cn, out_dtype = po.CASES[which]
+    h, w = src.shape[:2]
+    in_row = w * cn * np.dtype(in_dtype).itemsize
+    out_row = w * cn * np.dtype(out_dtype).itemsize
+    host_in = np.zeros((h, in_row + pad_in), np.uint8)
+    host_in[:, :in_row] = np.ascontiguousarray(src).view(np.uint8).reshape(h, in_row)
+    dev_in = torch.from_numpy(host_in).to(device)
+    dev_out = torch.full((h, out_row + pad_out), 0xA5, dtype=torch.uint8, device=device)
+    cases.pointwise(which, dev_in, w, h, dev_out, pc.constants(which), pc.MATRIX)
+    torch.cuda.synchronize()
+    got = dev_out.cpu().numpy()
+    assert np.all(got[:, out_row:] == 0xA5), "bytes beyond the rows were written"
+    return np.ascontiguousarray(got[:, :out_row]).view(out_dtype).reshape(src.shape)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", ALL)
+def test_operation_matches_the_oracle(device, which):
+    # a size with partial runs at the row ends, rows that start on odd addresses for the narrow types, and special values
+    for seed, (h, w, pad_in, pad_out) in enumerate(((7, 45, 0, 0), (33, 130, 3, 5))):
+        if np.dtype(po.CASES[which][0]).itemsize > 1 or np.dtype(po.CASES[which][2]).itemsize > 1:
+            pad_in, pad_out = pad_in * 4, pad_out * 4          # rows of wider elements stay aligned to their element
+        src = pc.inputs(which, po.CASES, h, w, seed)
+        want = po.run(which, src, pc.constants(which), pc.MATRIX)
+        got = run_on_gpu(device, which, src, pad_in, pad_out)
+        assert pc.same(which, got, want, po.INEXACT), (which, seed)
+
+
+@pytest.mark.gpu
+def test_full_size_properties(device):
+    # 4K: Abs is idempotent, Max then Min with the same constants clamps, x ^ c ^ c = x, (x << 5) >> 5 keeps the low bits
+    h, w = 2160, 3840
+    x = pc.inputs(0, po.CASES, h, w // 3, 7)
+    a1 = run_on_gpu(device, 0, x)
+    assert run_on_gpu(device, 0, a1).tobytes() == a1.tobytes() and not np.any(a1[np.isfinite(a1)] < 0)
+    u = pc.inputs(17, po.CASES, h, w, 8)
+    assert run_on_gpu(device, 17, run_on_gpu(device, 17, u)).tobytes() == u.tobytes()
+    sh = run_on_gpu(device, 19, u)
+    assert np.array_equal(sh, (u << np.uint32(5)))
+    f = pc.inputs(11, po.CASES, h, w // 3, 9)
+    lo = run_on_gpu(device, 11, f)
+    fin = ~np.isnan(f)
+    assert np.all(lo[fin] >= np.broadcast_to(np.array(pc.constants(11)[:3], np.float32), f.shape)[fin])

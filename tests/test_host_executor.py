@@ -15,6 +15,7 @@ import test_oracle_border as t_border
 import test_oracle_color as t_color
 import test_oracle_depth_and_transposed as t_depth
 import test_oracle_window as t_window
+import test_oracle_pointwise as t_pointwise
 
 pytestmark = pytest.mark.skipif(not ol.have_hostexec(), reason="oracle/libfkl_hostexec.so not built (make -C oracle hostexec)")
 
@@ -114,3 +115,9 @@ def test_transposed_tensor():
 @pytest.mark.parametrize("oldest_first", [False, True])
 def test_transposed_window(batch, oldest_first):
     on_host_executor(t_depth.test_transposed_window_matches_reference_backend, batch, oldest_first)
+
+
+@pytest.mark.parametrize("which", t_pointwise.ALL)
+def test_per_channel_operations(which):
+    # Abs ... MxVFloat3 (tests/cases/pointwise_chains.h): this repository's CPU executor against the numpy restatement
+    on_host_executor(t_pointwise.test_oracle_equals_the_reference_backend, which)
