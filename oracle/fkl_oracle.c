@@ -162,8 +162,10 @@ float fklo_bilinear(float p00, float p10, float p01, float p11, float sx, float 
 }
 
 /* Resize<...>::build(backIOp, dstSize, bg) and compute_target_size,
- * FK/algorithms/image_processing/resize.h:164-233 (PRESERVE_AR) and :266-278 (IGNORE_AR).
- * Factors are computed in double on the host and narrowed once. */
+ * FK/algorithms/image_processing/resize.h:164-233 (the three PRESERVE_AR modes) and :266-278 (IGNORE_AR).
+ * Factors are computed in double on the host and narrowed once.  PRESERVE_AR_RN_EVEN (:212-221) makes the width the
+ * even number at or below the rounded one (or, when that exceeds the destination, the height likewise);
+ * PRESERVE_AR_LEFT (:177-191) puts the picture at the left edge instead of centring it. */
 void fklo_compute_resize_params(int32_t src_w, int32_t src_h, int32_t dst_w, int32_t dst_h,
                                 int32_t ar, fklo_resize_params *out) {
     out->dst_w = dst_w;
@@ -179,16 +181,18 @@ void fklo_compute_resize_params(int32_t src_w, int32_t src_h, int32_t dst_w, int
     const float scale = (float)dst_h / (float)src_h;
     int tw = (int)fklo_round_half_away(scale * (float)src_w);
     int th = dst_h;
+    if (ar == FKLO_PRESERVE_AR_RN_EVEN) tw -= tw % 2;
     if (tw > dst_w) {
         const float scale2 = (float)dst_w / (float)src_w;
         tw = dst_w;
         th = (int)fklo_round_half_away(scale2 * (float)src_h);
+        if (ar == FKLO_PRESERVE_AR_RN_EVEN) th -= th % 2;
     }
     const double cfx = (double)tw / (double)src_w;
     const double cfy = (double)th / (double)src_h;
     out->fx = (float)(1.0 / cfx);
     out->fy = (float)(1.0 / cfy);
-    out->x1 = (dst_w - tw) / 2;
+    out->x1 = ar == FKLO_PRESERVE_AR_LEFT ? 0 : (dst_w - tw) / 2;
     out->y1 = (dst_h - th) / 2;
     out->x2 = out->x1 + tw - 1;
     out->y2 = out->y1 + th - 1;

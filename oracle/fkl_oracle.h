@@ -49,7 +49,7 @@ enum fklo_read_kind {
                             data = channel 0 of this image plane                        */
 };
 
-enum fklo_aspect { FKLO_PRESERVE_AR = 0, FKLO_IGNORE_AR = 1 };
+enum fklo_aspect { FKLO_PRESERVE_AR = 0, FKLO_IGNORE_AR = 1, FKLO_PRESERVE_AR_RN_EVEN = 2, FKLO_PRESERVE_AR_LEFT = 3 };
 
 enum fklo_opcode {
     FKLO_MUL = 1,              /* out = in * p   (per channel, result float)           */

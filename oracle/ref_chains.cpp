@@ -334,6 +334,23 @@ int fklref_yuv2rgb_709_full_matrix(float* m9) {
 
 #endif
 
+// The same for any aspect-ratio mode (0 PRESERVE_AR, 2 PRESERVE_AR_RN_EVEN, 3 PRESERVE_AR_LEFT).
+extern "C++" template <AspectRatio AR> void resize_params_of(int sw, int sh, int dw, int dh, int32_t* out4, float* f2) {
+    constexpr RawPtr<ND::_2D, uchar3> dummy{nullptr, {1u << 14, 1u << 14, 3u << 14}};
+    const auto back = PerThreadRead<ND::_2D, uchar3>::build(dummy).then(Crop<>::build(Rect(0, 0, sw, sh)));
+    const auto r = back.then(Resize<InterpolationType::INTER_LINEAR, AR>::build(Size(dw, dh), float3{0.f, 0.f, 0.f}));
+    out4[0] = r.params.x1; out4[1] = r.params.y1; out4[2] = r.params.x2; out4[3] = r.params.y2;
+    f2[0] = r.params.src_conv_factors.x; f2[1] = r.params.src_conv_factors.y;
+}
+int fklref_resize_params_ar(int ar, int sw, int sh, int dw, int dh, int32_t* out4, float* f2) {
+    switch (ar) {
+    case 0: resize_params_of<AspectRatio::PRESERVE_AR>(sw, sh, dw, dh, out4, f2); return 0;
+    case 2: resize_params_of<AspectRatio::PRESERVE_AR_RN_EVEN>(sw, sh, dw, dh, out4, f2); return 0;
+    case 3: resize_params_of<AspectRatio::PRESERVE_AR_LEFT>(sw, sh, dw, dh, out4, f2); return 0;
+    default: return 2;
+    }
+}
+
 // Letterbox geometry and factors the reference computes for one crop size (PRESERVE_AR), read back from the
 // built IOp: out = {x1, y1, x2, y2}, f = {fx, fy}.
 int fklref_resize_params_par(int sw, int sh, int dw, int dh, int32_t* out4, float* f2) {

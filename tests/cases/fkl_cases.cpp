@@ -425,6 +425,28 @@ int fklcase_uncompiled_resize_split(void* stream_, int kind, const void* src, in
         }
     });
 }
+// uchar3 image -> crop -> letterboxed bilinear resize in one of the aspect-ratio modes -> float3 image
+// (0 PRESERVE_AR, 2 PRESERVE_AR_RN_EVEN, 3 PRESERVE_AR_LEFT: one kernel, the geometry is made on the host)
+extern "C++" template <AspectRatio AR>
+void letterbox_of(void* stream_, const uint8_t* src, int w, int h, int pitch, const int32_t* rect, int dw, int dh, const float* bg, float* out, int out_pitch) {
+    Stream stream(stream_);
+    const auto i = dev2d<uchar3>(src, w, h, pitch);
+    const auto o = dev2d<float3>(out, dw, dh, out_pitch);
+    executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, uchar3>::build(i.ptr()), Crop<>::build(Rect(rect[0], rect[1], rect[2], rect[3])),
+                                      Resize<InterpolationType::INTER_LINEAR, AR>::build(Size(dw, dh), make_<float3>(bg[0], bg[1], bg[2])),
+                                      PerThreadWrite<ND::_2D, float3>::build(o.ptr()));
+}
+int fklcase_letterbox_ar(void* stream_, int ar, const uint8_t* src, int w, int h, int pitch, const int32_t* rect, int dw, int dh,
+                         const float* bg, float* out, int out_pitch) {
+    return guarded([&] {
+        switch (ar) {
+        case 0: letterbox_of<AspectRatio::PRESERVE_AR>(stream_, src, w, h, pitch, rect, dw, dh, bg, out, out_pitch); break;
+        case 2: letterbox_of<AspectRatio::PRESERVE_AR_RN_EVEN>(stream_, src, w, h, pitch, rect, dw, dh, bg, out, out_pitch); break;
+        case 3: letterbox_of<AspectRatio::PRESERVE_AR_LEFT>(stream_, src, w, h, pitch, rect, dw, dh, bg, out, out_pitch); break;
+        default: throw std::runtime_error("fklcase_letterbox_ar: ar must be 0, 2 or 3");
+        }
+    });
+}
 // float4 image -> bilinear resize -> float4 image (16-byte elements: one access per tap)
 int fklcase_uncompiled_float4_resize(void* stream_, const float* in, int w, int h, int pitch, int dw, int dh, float* out, int out_pitch) {
     return guarded([&] {

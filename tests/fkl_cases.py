@@ -290,6 +290,15 @@ def depth_ops(which, src, out, lo=0.0, hi=1.0):
                                   C.c_float(float(lo)), C.c_float(float(hi))))
 
 
+def letterbox_ar(ar, src, rect, bg, out):
+    """src (H,W,3) u8 cuda -> Crop(rect = x, y, w, h) -> Resize<INTER_LINEAR, ar>(out's size, bg) -> out (dh,dw,3) f32 cuda;
+    ar: 0 PRESERVE_AR, 2 PRESERVE_AR_RN_EVEN, 3 PRESERVE_AR_LEFT."""
+    r = _host(rect, np.int32)
+    b = _host(bg, np.float32)
+    _ok(cases().fklcase_letterbox_ar(_stream(), int(ar), _p(src), src.shape[1], src.shape[0], _pitch(src), r.ctypes.data_as(C.c_void_p),
+                                     out.shape[1], out.shape[0], b.ctypes.data_as(C.c_void_p), _p(out), _pitch(out)))
+
+
 def pointwise(which, src_bytes, width, height, out_bytes, c=(0, 0, 0, 0), m=(1, 0, 0, 0, 1, 0, 0, 0, 1)):
     """Chain number `which` of tests/cases/pointwise_chains.h.  src_bytes / out_bytes: 2-D u8 cuda tensors holding `height`
     rows of `width` elements of the chain's input / output type (a row may be longer than its elements: the pitch)."""

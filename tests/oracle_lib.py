@@ -290,6 +290,17 @@ def oracle_crop_resize_par_u8(src, rects, dst, bg, mul, sub):
     return out
 
 
+PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT = 2, 3
+
+
+def oracle_letterbox_ar(ar, src, rect, dst, bg):
+    """src (H,W,3) u8 -> crop -> letterboxed bilinear resize in aspect-ratio mode `ar` -> (dh,dw,3) f32."""
+    dw, dh = dst
+    out = np.zeros((dh, dw, 3), np.float32)
+    execute([read_2d(src, 3, crop=rect, resize=dst, ar=ar, bg=bg)], [], [write(WRITE_2D, out, 3, dw, dh)])
+    return out
+
+
 def oracle_crop_resize_norm_split(src, rects, dst, sub, div):
     dw, dh = dst
     b = len(rects)

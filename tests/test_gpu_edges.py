@@ -67,6 +67,26 @@ def test_letterbox_both_orientations(device):
         assert np.array_equal(out.cpu().numpy(), want), dst
 
 
+def test_letterbox_in_the_even_and_left_aligned_modes(device):
+    # PRESERVE_AR_RN_EVEN and PRESERVE_AR_LEFT (and PRESERVE_AR through the same driver): the geometry is made on the host,
+    # the kernel is the letterboxing one; band pixels are the background exactly, the picture is the oracle's bit for bit
+    import torch
+    rng = np.random.RandomState(143)
+    src_np = rng.randint(0, 256, (300, 400, 3)).astype(np.uint8)
+    src = torch.from_numpy(src_np).to(device)
+    bg = np.array([3, 200, 77], np.float32)
+    for rect in ([0, 0, 400, 300], [10, 10, 31, 200], [10, 10, 301, 21], [50, 60, 7, 230], [5, 5, 111, 67]):
+        for dst in ((128, 64), (64, 128), (33, 33), (97, 35)):
+            for ar in (ol.PRESERVE_AR, ol.PRESERVE_AR_RN_EVEN, ol.PRESERVE_AR_LEFT):
+                out = torch.zeros((dst[1], dst[0], 3), dtype=torch.float32, device=device)
+                cases.letterbox_ar(ar, src, rect, bg, out)
+                torch.cuda.synchronize()
+                want = ol.oracle_letterbox_ar(ar, src_np, np.array(rect, np.int32), dst, bg)
+                assert out.cpu().numpy().tobytes() == want.tobytes(), (rect, dst, ar)
+                if ar == ol.PRESERVE_AR_LEFT and rect[2] * dst[1] < rect[3] * dst[0]:      # narrower than the frame: band on the right only
+                    assert not np.array_equal(want[dst[1] // 2, 0], bg) and np.array_equal(want[dst[1] // 2, -1], bg)
+
+
 def test_unaligned_pitch_and_odd_width_rows(device):
     import torch
     rng = np.random.RandomState(44)

@@ -121,3 +121,8 @@ def test_transposed_window(batch, oldest_first):
 def test_per_channel_operations(which):
     # Abs ... MxVFloat3 (tests/cases/pointwise_chains.h): this repository's CPU executor against the numpy restatement
     on_host_executor(t_pointwise.test_oracle_equals_the_reference_backend, which)
+
+
+def test_resize_geometry_of_every_aspect_ratio_mode():
+    # Resize<INTER_LINEAR, AR>::build of this repository's headers (PRESERVE_AR, PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT)
+    on_host_executor(t_core.test_aspect_ratio_modes_match_the_live_reference_on_random_sizes)

@@ -130,6 +130,42 @@ def test_letterbox_geometry_matches_reference():
         assert float(np.float32(rp.fx)) == want["fx"] and float(np.float32(rp.fy)) == want["fy"], key
 
 
+def _geometry_of_the_oracle(ar, sw, sh, dw, dh):
+    rp = ol.ResizeParams()
+    ol.oracle().fklo_compute_resize_params(sw, sh, dw, dh, ar, C.byref(rp))
+    return [rp.x1, rp.y1, rp.x2, rp.y2], float(np.float32(rp.fx)), float(np.float32(rp.fy))
+
+
+def test_aspect_ratio_modes_match_the_committed_reference_vectors():
+    # PRESERVE_AR (0), PRESERVE_AR_RN_EVEN (2), PRESERVE_AR_LEFT (3): tests/golden/resize_geometry_reference_vectors.json
+    with open(os.path.join(HERE, "golden", "resize_geometry_reference_vectors.json")) as f:
+        vectors = json.load(f)
+    assert len(vectors) == 45
+    for key, want in vectors.items():
+        ar, rest = key.split(":")
+        src, dst = rest.split("->")
+        (sw, sh), (dw, dh) = (tuple(int(v) for v in t.split("x")) for t in (src, dst))
+        rect, fx, fy = _geometry_of_the_oracle(int(ar), sw, sh, dw, dh)
+        assert rect == want["rect"] and fx == want["fx"] and fy == want["fy"], key
+        if int(ar) == 2:
+            assert (rect[2] - rect[0] + 1) % 2 == 0 or (rect[3] - rect[1] + 1) % 2 == 0       # one side made even
+        if int(ar) == 3:
+            assert rect[0] == 0
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="oracle/_ref not built")
+def test_aspect_ratio_modes_match_the_live_reference_on_random_sizes():
+    rng = np.random.default_rng(77)
+    for _ in range(300):
+        sw, sh, dw, dh = (int(v) for v in rng.integers(2, 700, 4))
+        for ar in (0, 2, 3):
+            o4 = (C.c_int32 * 4)()
+            f2 = (C.c_float * 2)()
+            assert ol.ref().fklref_resize_params_ar(ar, sw, sh, dw, dh, o4, f2) == 0
+            rect, fx, fy = _geometry_of_the_oracle(ar, sw, sh, dw, dh)
+            assert rect == list(o4) and fx == float(np.float32(f2[0])) and fy == float(np.float32(f2[1])), (ar, sw, sh, dw, dh)
+
+
 def test_golden_c1():
     c = wl.config1(**CASES["c1_small"])
     rects = np.array(META["c1_small_rects"], np.int32)
