@@ -2540,6 +2540,65 @@ template <class T> struct Write2D {
 #endif
 };
 
+// SplitWrite<_2D, T>: channel c of every value goes to an image of its own, each with its own pitch.
+// FK/algorithms/basic_ops/memory_operations.h:336-390.
+template <class T> struct SplitWrite2D {
+    static_assert(cn_v<T> >= 2, "two to four channels");
+    using In = T;
+    using B = base_t<T>;
+    static constexpr int N = cn_v<T>;
+    struct Params { RawPtr2D<B> c[N]; };
+    FKD_NAME("SplitWrite2D<" + type_name<T>() + ">")
+    template <int I> FKD_HD static B pick(const T& v) { return chan<I>(v); }
+#if defined(FKD_EXEC_CODE)
+    FKD_DEV static void exec(int x, int y, int, const T& v, const Params& p) {
+        detail::store_elem(detail::row_ptr(p.c[0].data, p.c[0].pitch, x, y), pick<0>(v));
+        detail::store_elem(detail::row_ptr(p.c[1].data, p.c[1].pitch, x, y), pick<1>(v));
+        if constexpr (N > 2) detail::store_elem(detail::row_ptr(p.c[2].data, p.c[2].pitch, x, y), pick<2>(v));
+        if constexpr (N > 3) detail::store_elem(detail::row_ptr(p.c[3].data, p.c[3].pitch, x, y), pick<3>(v));
+    }
+#endif
+#if defined(FKD_DEVICE_CODE)
+    template <int I, int V, int A> FKD_DEV static void channel_run(int x, int y, const Slot<T> (&v)[V], const Params& p) {
+        Slot<B> run[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) run[i].v = pick<I>(v[i].v);
+        detail::store_run<B, V, A>(detail::row_ptr(p.c[I].data, p.c[I].pitch, x, y), run);
+    }
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Slot<T> (&v)[V], const Params& p) {
+        channel_run<0, V, A>(x, y, v, p);
+        channel_run<1, V, A>(x, y, v, p);
+        if constexpr (N > 2) channel_run<2, V, A>(x, y, v, p);
+        if constexpr (N > 3) channel_run<3, V, A>(x, y, v, p);
+    }
+    FKD_HD static bool rows_aligned(const Params& p) {
+        bool ok = true;
+        for (int i = 0; i < N; ++i) ok = ok && detail::dword_aligned(p.c[i].data) && p.c[i].pitch % 4 == 0;
+        return ok;
+    }
+    using Plane = SplitWrite2D;
+    FKD_DEV static const Params& plane_params(const Params& p, int) { return p; }
+    struct RowRef { B* p[N]; };
+    FKD_DEV static RowRef row(int y, int, const Params& p) {
+        RowRef r;
+#pragma unroll
+        for (int i = 0; i < N; ++i) r.p[i] = detail::row_ptr(p.c[i].data, p.c[i].pitch, 0, y);
+        return r;
+    }
+    FKD_DEV static void put(const RowRef& r, int x, const T& v) {
+        const u32 off = u32(x) * u32(sizeof(B));
+        detail::store_elem_at<B>(reinterpret_cast<char*>(r.p[0]), off, pick<0>(v));
+        detail::store_elem_at<B>(reinterpret_cast<char*>(r.p[1]), off, pick<1>(v));
+        if constexpr (N > 2) detail::store_elem_at<B>(reinterpret_cast<char*>(r.p[2]), off, pick<2>(v));
+        if constexpr (N > 3) detail::store_elem_at<B>(reinterpret_cast<char*>(r.p[3]), off, pick<3>(v));
+    }
+    template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<T> (&v)[V]) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) put(r, x + i, v[i].v);
+    }
+#endif
+};
+
 // TensorWrite<T> / PerThreadWrite<_3D,T>: FK/algorithms/basic_ops/memory_operations.h:159-179; plane z at
 // z*plane_pitch*color_planes (FK/core/data/rawptr.h:215-226).
 template <class T> struct TensorWrite {

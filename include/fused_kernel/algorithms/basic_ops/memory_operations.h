@@ -1,9 +1,12 @@
 // Per-element memory operations: PerThreadRead / PerThreadWrite (pitched 1-D/2-D/3-D), TensorRead / TensorWrite,
 // TensorSplit (planar writer) and TensorPack (its reader), and the circular-buffer views CircularTensorRead /
 // CircularTensorWrite.  Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:26-212, 243-290, 413-432,
-// 505-587.  CircularBatchRead / CircularBatchWrite (434-503) and the transposed-plane forms TensorTSplit / TensorTPack (214-241, 292-327) too.
+// 505-587.  CircularBatchRead / CircularBatchWrite (434-503), the transposed-plane forms TensorTSplit / TensorTPack (214-241, 292-327)
+// and SplitWrite (336-390: one image per channel) too.
 #ifndef FK_AMD_MEMORY_OPERATIONS_H
 #define FK_AMD_MEMORY_OPERATIONS_H
+
+#include <vector>
 
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
 
@@ -37,6 +40,36 @@ struct PerThreadWrite : WriteOperation<T, RawPtr<D, T>, T, TF::ENABLED, PerThrea
     static InstantiableType build(const Ptr<D, T>& ptr) { return {{ptr.ptr()}}; }
     static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.dims.width; }
     static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.dims.pitch; }
+};
+
+// SplitWrite<D, T>: channel c of every value goes to an image of its own (x, y, z, w), each with its own pitch.
+// Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:336-390.
+template <ND D, typename T, typename Enabler = void> struct SplitWriteParams {};
+template <ND D, typename T> struct SplitWriteParams<D, T, std::enable_if_t<cn<T> == 2>> {
+    RawPtr<D, VBase<T>> x, y;
+};
+template <ND D, typename T> struct SplitWriteParams<D, T, std::enable_if_t<cn<T> == 3>> {
+    RawPtr<D, VBase<T>> x, y, z;
+};
+template <ND D, typename T> struct SplitWriteParams<D, T, std::enable_if_t<cn<T> == 4>> {
+    RawPtr<D, VBase<T>> x, y, z, w;
+};
+template <ND D, typename T>
+struct SplitWrite : WriteOperation<T, SplitWriteParams<D, T>, VBase<T>, TF::DISABLED, SplitWrite<D, T>> {
+    static_assert(cn<T> >= 2, "Split operations can only be used with types of 2, 3 or 4 channels.");
+    using Parent = WriteOperation<T, SplitWriteParams<D, T>, VBase<T>, TF::DISABLED, SplitWrite<D, T>>;
+    using typename Parent::OperationDataType;
+    using typename Parent::InstantiableType;
+    FK_STATIC_STRUCT(SplitWrite, SplitWrite)
+    using Parent::build;
+    // one image per channel, in channel order (at() throws when there are too few)
+    static InstantiableType build(const std::vector<Ptr2D<VBase<T>>>& output) {
+        if constexpr (cn<T> == 2) return {{{output.at(0).ptr(), output.at(1).ptr()}}};
+        else if constexpr (cn<T> == 3) return {{{output.at(0).ptr(), output.at(1).ptr(), output.at(2).ptr()}}};
+        else return {{{output.at(0).ptr(), output.at(1).ptr(), output.at(2).ptr(), output.at(3).ptr()}}};
+    }
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.x.dims.width; }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.x.dims.pitch; }
 };
 
 // Deduces dimension and element type from the pointer: ReadOp::build(ptr), WriteOp::build(ptr).
@@ -274,6 +307,19 @@ template <typename T> struct Lower<PerThreadWrite<ND::_2D, T>> {
     static constexpr bool available = true;
     using type = fkd::Write2D<dev_t<T>>;
     static typename type::Params params(const OperationData<PerThreadWrite<ND::_2D, T>>& d) { return to_dev<T, dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<SplitWrite<ND::_2D, T>> {
+    static constexpr bool available = true;
+    using B = typename DevType<VBase<T>>::type;
+    using type = fkd::SplitWrite2D<dev_t<T>>;
+    static typename type::Params params(const OperationData<SplitWrite<ND::_2D, T>>& d) {
+        typename type::Params p{};
+        p.c[0] = to_dev<VBase<T>, B>(d.params.x);
+        p.c[1] = to_dev<VBase<T>, B>(d.params.y);
+        if constexpr (cn<T> > 2) p.c[2] = to_dev<VBase<T>, B>(d.params.z);
+        if constexpr (cn<T> > 3) p.c[3] = to_dev<VBase<T>, B>(d.params.w);
+        return p;
+    }
 };
 template <typename T> struct Lower<PerThreadWrite<ND::_1D, T>> {
     static constexpr bool available = true;

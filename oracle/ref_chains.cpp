@@ -433,6 +433,14 @@ int fklref_pointwise(int which, const void* src, int w, int h, int pitch, void* 
     s.sync();
     return rc;
 }
+// SplitWrite chain number `which` of tests/cases/pointwise_chains.h on the CPU backend.
+int fklref_split_write(int which, const void* src, int w, int h, int pitch, int dw, int dh, void* const* outs, const int* out_pitch,
+                       const float* c) {
+    CpuStream s;
+    const int rc = pointwise_chains::Chains<CpuDPP, CpuStream>::split_write(s, MemType::Host, which, src, w, h, pitch, dw, dh, outs, out_pitch, c);
+    s.sync();
+    return rc;
+}
 #ifndef FKL_HARNESS_PUBLIC_API_ONLY
 // ccMatrix<range, primaries, direction, depth> as the reference computes it at compile time, row major.
 // to_rgb = 1 selects YCbCr2RGB.

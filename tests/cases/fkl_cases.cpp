@@ -606,6 +606,14 @@ extern "C" int fklcase_pointwise(void* stream_, int which, const void* src, int 
     });
 }
 
+extern "C" int fklcase_split_write(void* stream_, int which, const void* src, int w, int h, int pitch, int dw, int dh, void* const* outs,
+                                   const int* out_pitch, const float* c) {
+    return guarded_rc([&] {
+        Stream s(stream_);
+        return pointwise_chains::Chains<TransformDPP<>, Stream>::split_write(s, MemType::Device, which, src, w, h, pitch, dw, dh, outs, out_pitch, c);
+    });
+}
+
 // ---- padding through BorderReader (border_chains.h on the GPU) ----------------------------------------------------
 extern "C" int fklcase_pad(void* stream_, int elem, int border_type, const void* src, int w, int h, int pitch, int left, int top,
                            int out_w, int out_h, const float* value, void* out, int out_pitch) {

@@ -1,5 +1,6 @@
 // pointwise_chains.h -- chains of one per-channel Operation of the basic_ops headers (math.h, logical.h, bitwise.h,
-// algebraic.h) between a read and a write, spelled ONCE with the public C++ API of the fused-kernel library.
+// algebraic.h) between a read and a write, and chains that end in SplitWrite, spelled ONCE with the public C++ API of the
+// fused-kernel library.
 //
 // This text is compiled twice: by tests/cases/fkl_cases.cpp against this repository's headers (the chains then run as
 // gfx950 kernels on device memory), and by oracle/ref_chains.cpp against the reference library's own headers (the
@@ -10,6 +11,7 @@
 #pragma once
 
 #include <cstdint>
+#include <vector>
 
 namespace pointwise_chains {
 
@@ -62,6 +64,54 @@ template <class DPP, class StreamT> struct Chains {
         case 21: one<float3, float3>(s, mem, MxVFloat3<BinaryType>::build(mat), src, w, h, pitch, out, out_pitch); return 0;
         case 22: one<uchar, float>(s, mem, Exp<uchar, float>::build(), src, w, h, pitch, out, out_pitch); return 0;
         case 23: one<short2, short2>(s, mem, Abs<short2>::build(), src, w, h, pitch, out, out_pitch); return 0;
+        default: return 2;
+        }
+    }
+
+    // ---- SplitWrite<_2D, T>: one output image per channel, each with its own pitch --------------------------------
+    template <class O> static std::vector<Ptr2D<VBase<O>>> planes_of(void* const* outs, const int* out_pitch, int w, int h, MemType mem) {
+        std::vector<Ptr2D<VBase<O>>> v;
+        for (int c = 0; c < cn<O>; ++c) v.push_back(wrap<VBase<O>>(outs[c], w, h, out_pitch[c], mem));
+        return v;
+    }
+    // 0 uchar3 image -> its three planes              1 uchar3 -> Cast -> Mul{c} -> three float planes
+    // 2 float4 image -> its four planes               3 uchar3 -> Crop(8, 4, w - 16, h - 8) -> Resize(dw x dh) -> three float planes
+    // 4 float2 image -> its two planes
+    static int split_write(StreamT& s, MemType mem, int which, const void* src, int w, int h, int pitch, int dw, int dh,
+                           void* const* outs, const int* out_pitch, const float* c) {
+        switch (which) {
+        case 0: {
+            const auto in = wrap<uchar3>(src, w, h, pitch, mem);
+            executeOperations<DPP>(s, PerThreadRead<ND::_2D, uchar3>::build(in.ptr()),
+                                   SplitWrite<ND::_2D, uchar3>::build(planes_of<uchar3>(outs, out_pitch, w, h, mem)));
+            return 0;
+        }
+        case 1: {
+            const auto in = wrap<uchar3>(src, w, h, pitch, mem);
+            executeOperations<DPP>(s, PerThreadRead<ND::_2D, uchar3>::build(in.ptr()), Cast<uchar3, float3>::build(),
+                                   Mul<float3>::build(make_<float3>(c[0], c[1], c[2])),
+                                   SplitWrite<ND::_2D, float3>::build(planes_of<float3>(outs, out_pitch, w, h, mem)));
+            return 0;
+        }
+        case 2: {
+            const auto in = wrap<float4>(src, w, h, pitch, mem);
+            executeOperations<DPP>(s, PerThreadRead<ND::_2D, float4>::build(in.ptr()),
+                                   SplitWrite<ND::_2D, float4>::build(planes_of<float4>(outs, out_pitch, w, h, mem)));
+            return 0;
+        }
+        case 3: {
+            const auto in = wrap<uchar3>(src, w, h, pitch, mem);
+            executeOperations<DPP>(s, PerThreadRead<ND::_2D, uchar3>::build(in.ptr()), Crop<>::build(Rect(8, 4, w - 16, h - 8)),
+                                   Resize<InterpolationType::INTER_LINEAR>::build(Size(dw, dh)),
+                                   SplitWrite<ND::_2D, float3>::build(planes_of<float3>(outs, out_pitch, dw, dh, mem)));
+            return 0;
+        }
+        case 4: {
+            const auto in = wrap<float2>(src, w, h, pitch, mem);
+            executeOperations<DPP>(s, PerThreadRead<ND::_2D, float2>::build(in.ptr()),
+                                   SplitWrite<ND::_2D, float2>::build(planes_of<float2>(outs, out_pitch, w, h, mem)));
+            return 0;
+        }
         default: return 2;
         }
     }

@@ -308,6 +308,17 @@ def pointwise(which, src_bytes, width, height, out_bytes, c=(0, 0, 0, 0), m=(1, 
                                   _pitch(out_bytes), cv.ctypes.data_as(C.c_void_p), mv.ctypes.data_as(C.c_void_p)))
 
 
+def split_write(which, src_bytes, width, height, outs, dst=None, c=(1, 1, 1, 1)):
+    """SplitWrite chain number `which` of tests/cases/pointwise_chains.h.  src_bytes: 2-D u8 cuda tensor holding the input
+    image's rows; outs: one 2-D cuda tensor per channel (each may have a pitch of its own); dst = (dw, dh) for chain 3."""
+    dw, dh = dst if dst is not None else (width, height)
+    ptrs = (C.c_void_p * 4)(*[C.c_void_p(o.data_ptr()) for o in outs])
+    pitches = (C.c_int * 4)(*[_pitch(o) for o in outs])
+    cv = np.ascontiguousarray(c, dtype=np.float32)
+    _ok(cases().fklcase_split_write(_stream(), int(which), _p(src_bytes), int(width), int(height), _pitch(src_bytes), int(dw), int(dh),
+                                    ptrs, pitches, cv.ctypes.data_as(C.c_void_p)))
+
+
 def pad(src, border_type, left, top, out, value=(0, 0, 0)):
     """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out."""
     v = np.zeros(4, np.float32)

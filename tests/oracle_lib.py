@@ -717,6 +717,43 @@ def ref_pointwise(which, src, c=(0, 0, 0, 0), m=(1, 0, 0, 0, 1, 0, 0, 0, 1)):
     return out
 
 
+# SplitWrite chains of tests/cases/pointwise_chains.h: which -> (input dtype, channels, output dtype)
+SPLIT_WRITE_CASES = {0: (np.uint8, 3, np.uint8), 1: (np.uint8, 3, np.float32), 2: (np.float32, 4, np.float32),
+                     3: (np.uint8, 3, np.float32), 4: (np.float32, 2, np.float32)}
+
+
+def oracle_split_write(which, src, dst=None, c=(1, 1, 1, 1)):
+    """The planes SplitWrite<_2D, T> leaves: channel k of every value in image k (FK/algorithms/basic_ops/
+    memory_operations.h:361-377).  Chain 1 multiplies by c first, chain 3 crops and resizes to dst = (dw, dh) first."""
+    _, cn, out_dtype = SPLIT_WRITE_CASES[which]
+    h, w = src.shape[:2]
+    if which == 1:
+        val = (src.astype(np.float32) * np.asarray(c[:3], np.float32)).astype(np.float32)
+    elif which == 3:
+        dw, dh = dst
+        val = np.zeros((dh, dw, 3), np.float32)
+        execute([read_2d(src, 3, crop=np.array([8, 4, w - 16, h - 8], np.int32), resize=(dw, dh), ar=IGNORE_AR)], [],
+                [write(WRITE_2D, val, 3, dw, dh)])
+    else:
+        val = src
+    return [np.ascontiguousarray(val[..., k]).astype(out_dtype) for k in range(cn)]
+
+
+def ref_split_write(which, src, dst=None, c=(1, 1, 1, 1), pad=(0, 0, 0, 0)):
+    """The same chains on the reference's CPU backend; `pad` = extra elements at the end of each output image's rows."""
+    in_dtype, cn, out_dtype = SPLIT_WRITE_CASES[which]
+    src = np.ascontiguousarray(src, dtype=in_dtype)
+    h, w = src.shape[:2]
+    dw, dh = dst if dst is not None else (w, h)
+    bufs = [np.full((dh, dw + pad[k]), 0, out_dtype) for k in range(cn)]
+    outs = (C.c_void_p * 4)(*[C.c_void_p(_ptr(b)) for b in bufs])
+    pitches = (C.c_int * 4)(*[b.strides[0] for b in bufs])
+    rc = ref().fklref_split_write(int(which), C.c_void_p(_ptr(src)), w, h, src.strides[0], dw, dh, outs, pitches,
+                                  _f32p(np.asarray(c, np.float32)))
+    assert rc == 0, rc
+    return [np.ascontiguousarray(b[:, :dw]) for b in bufs]
+
+
 # ---- transposed tensors: TensorTSplit / TensorTPack --------------------------------------------------------------------
 
 def oracle_transposed_round_trip(images, mul, mul2):

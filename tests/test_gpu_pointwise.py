@@ -59,3 +59,28 @@ def test_full_size_properties(device):
     lo = run_on_gpu(device, 11, f)
     fin = ~np.isnan(f)
     assert np.all(lo[fin] >= np.broadcast_to(np.array(pc.constants(11)[:3], np.float32), f.shape)[fin])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", sorted(ol.SPLIT_WRITE_CASES))
+def test_split_write_matches_the_oracle(device, which):
+    # SplitWrite<_2D, T>: one image per channel, each with a pitch of its own (padding columns must stay untouched)
+    import torch
+    import test_oracle_pointwise as t
+    in_dtype, cn, out_dtype = ol.SPLIT_WRITE_CASES[which]
+    tdt = {np.uint8: torch.uint8, np.float32: torch.float32}[out_dtype]
+    for seed, (h, w) in enumerate(((24, 40), (37, 53), (64, 256))):
+        src = t._split_input(which, h, w, seed)
+        dst = (29, 17) if which == 3 else None
+        dw, dh = dst if dst else (w, h)
+        c = (0.5, -2.0, 3.25, 0)
+        want = ol.oracle_split_write(which, src, dst, c)
+        dev_in = torch.from_numpy(np.ascontiguousarray(src).view(np.uint8).reshape(h, -1)).to(device)
+        pads = (0, 3, 1, 2) if out_dtype == np.float32 else (0, 3, 5, 2)
+        bufs = [torch.full((dh, dw + pads[k]), 77, dtype=tdt, device=device) for k in range(cn)]
+        cases.split_write(which, dev_in, w, h, [b[:, :dw] for b in bufs], dst, c)
+        torch.cuda.synchronize()
+        for k in range(cn):
+            got = bufs[k].cpu().numpy()
+            assert got[:, :dw].tobytes() == want[k].tobytes(), (which, seed, k)
+            assert np.all(got[:, dw:] == 77), "padding columns were written"

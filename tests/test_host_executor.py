@@ -126,3 +126,8 @@ def test_per_channel_operations(which):
 def test_resize_geometry_of_every_aspect_ratio_mode():
     # Resize<INTER_LINEAR, AR>::build of this repository's headers (PRESERVE_AR, PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT)
     on_host_executor(t_core.test_aspect_ratio_modes_match_the_live_reference_on_random_sizes)
+
+
+@pytest.mark.parametrize("which", sorted(ol.SPLIT_WRITE_CASES))
+def test_split_write(which):
+    on_host_executor(t_pointwise.test_split_write_equals_the_reference_backend, which)

@@ -65,3 +65,32 @@ def test_oracle_equals_the_committed_reference_vectors(which):
     src = pc.inputs(which, po.CASES, 5, 9, 0)
     assert src.tobytes() == g[f"in_{which}"].tobytes(), "the seeded inputs changed: regenerate the fixture"
     assert pc.same(which, po.run(which, src, pc.constants(which), pc.MATRIX), g[f"out_{which}"], po.INEXACT)
+
+
+def _split_input(which, h, w, seed):
+    in_dtype, cn, _ = ol.SPLIT_WRITE_CASES[which]
+    rng = np.random.default_rng(500 + 10 * which + seed)
+    if in_dtype == np.uint8:
+        return rng.integers(0, 256, (h, w, cn), dtype=np.uint8)
+    return rng.uniform(-100, 100, (h, w, cn)).astype(np.float32)
+
+
+def test_split_write_closed_form():
+    src = np.arange(2 * 3 * 3, dtype=np.uint8).reshape(2, 3, 3)
+    planes = ol.oracle_split_write(0, src)
+    assert [p.tolist() for p in planes] == [[[0, 3, 6], [9, 12, 15]], [[1, 4, 7], [10, 13, 16]], [[2, 5, 8], [11, 14, 17]]]
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="oracle/_ref not built")
+@pytest.mark.parametrize("which", sorted(ol.SPLIT_WRITE_CASES))
+def test_split_write_equals_the_reference_backend(which):
+    # every output image with a pitch of its own
+    for seed, (h, w) in enumerate(((24, 40), (37, 53))):
+        src = _split_input(which, h, w, seed)
+        dst = (29, 17) if which == 3 else None
+        c = (0.5, -2.0, 3.25, 0)
+        want = ol.ref_split_write(which, src, dst, c, pad=(0, 3, 1, 2))
+        got = ol.oracle_split_write(which, src, dst, c)
+        assert len(got) == len(want)
+        for g, r in zip(got, want):
+            assert g.dtype == r.dtype and g.tobytes() == r.tobytes(), (which, seed)
