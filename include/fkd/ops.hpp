@@ -912,6 +912,10 @@ struct AbsDiff {
         return d < decltype(d)(0) ? -d : d;
     }
 };
+struct Add { FKD_FN("fn::Add") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a + b; } };
+struct Sub { FKD_FN("fn::Sub") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a - b; } };
+struct Mul { FKD_FN("fn::Mul") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a * b; } };
+struct Div { FKD_FN("fn::Div") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a / b; } };
 struct BwAnd { FKD_FN("fn::BwAnd") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a & b; } };
 struct BwOr { FKD_FN("fn::BwOr") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a | b; } };
 struct BwXor { FKD_FN("fn::BwXor") template <class A, class B> FKD_HD static auto apply(A a, B b) { return a ^ b; } };
@@ -935,6 +939,18 @@ template <class F, class I, class P, class O> struct Map2 {
     FKD_NAME("Map2<" + F::name() + "," + type_name<I>() + "," + type_name<P>() + "," + type_name<O>() + ">")
     FKD_DEV static O exec(const I& a, const Params& p) {
         return map2<O>(a, p.v, [](auto x, auto y) { return static_cast<base_t<O>>(F::apply(x, y)); });
+    }
+};
+
+// The two-input forms of the same operations (Add<I1, I2, O, UnaryType> ... in arithmetic.h:26-124, bitwise.h, logical.h,
+// math.h): the value is a pair, as DualRead2D hands it over, and the function is applied to its two halves channel by
+// channel (a scalar half is broadcast).
+template <class F, class A, class B, class O> struct Zip {
+    static_assert(cn_v<A> == cn_v<O> || cn_v<B> == cn_v<O>, "one output channel per input channel");
+    using In = Two<A, B>; using Out = O; using Params = Empty;
+    FKD_NAME("Zip<" + F::name() + "," + type_name<A>() + "," + type_name<B>() + "," + type_name<O>() + ">")
+    FKD_DEV static O exec(const In& v, const Params&) {
+        return map2<O>(v.a, v.b, [](auto x, auto y) { return static_cast<base_t<O>>(F::apply(x, y)); });
     }
 };
 
@@ -2537,6 +2553,28 @@ template <class T> struct Write2D {
     template <int V> FKD_DEV static void put_run(const RowRef& r, int x, const Slot<T> (&v)[V]) {
         detail::store_run_at<T, V>(reinterpret_cast<char*>(r.p), u32(x) * u32(sizeof(T)), v);
     }
+#endif
+};
+
+// DualSourceRead<_2D, T>: the elements of two images at the same position, as a pair.
+// FK/algorithms/basic_ops/memory_operations.h:585-640.  The extent is the first image's.
+template <class T> struct DualRead2D {
+    using Out = Two<T, T>;
+    using One = Read2D<T>;
+    struct Params { typename One::Params a, b; };
+    FKD_NAME("DualRead2D<" + type_name<T>() + ">")
+#if defined(FKD_EXEC_CODE)
+    FKD_DEV static Out exec(int x, int y, int z, const Params& p) { return Out{One::exec(x, y, z, p.a), One::exec(x, y, z, p.b)}; }
+#endif
+#if defined(FKD_DEVICE_CODE)
+    template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Params& p, Slot<Out> (&out)[V]) {
+        Slot<T> ra[V], rb[V];
+        One::template exec_row<V, A>(x, y, z, p.a, ra);
+        One::template exec_row<V, A>(x, y, z, p.b, rb);
+#pragma unroll
+        for (int i = 0; i < V; ++i) { out[i].v.a = ra[i].v; out[i].v.b = rb[i].v; }
+    }
+    FKD_HD static bool rows_aligned(const Params& p, int xoff) { return One::rows_aligned(p.a, xoff) && One::rows_aligned(p.b, xoff); }
 #endif
 };
 

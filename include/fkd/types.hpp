@@ -98,6 +98,9 @@ template <class O, class A, class B, class F> FKD_HD O map2(const A& a, const B&
 
 struct Empty {};
 
+// Two values travelling through a chain side by side (what a read of two sources hands to a two-input operation).
+template <class A, class B> struct Two { A a; B b; };
+
 // Heterogeneous parameter pack with a layout both compilers agree on (plain nested aggregates).
 template <class... Ts> struct Tup;
 template <> struct Tup<> {};
@@ -147,6 +150,9 @@ FKD_TN(f32, "f32") FKD_TN(f64, "f64")
 #undef FKD_TN
 template <class T, int N> struct TypeName<Vec<T, N>> {
     static std::string get() { return "Vec<" + TypeName<T>::get() + "," + std::to_string(N) + ">"; }
+};
+template <class A, class B> struct TypeName<Two<A, B>> {
+    static std::string get() { return "Two<" + TypeName<A>::get() + "," + TypeName<B>::get() + ">"; }
 };
 template <class T> std::string type_name() { return TypeName<T>::get(); }
 #endif

@@ -1,12 +1,29 @@
-// Add / Sub / Mul / Div as Binary operations (value op parameter, channel-wise, a scalar parameter is broadcast).
-// Interface counterpart: FK/algorithms/basic_ops/arithmetic.h:26-124.  The tuple-input Unary forms of the
-// reference are not part of the fused data-parallel path and are not provided.
+// Add / Sub / Mul / Div as Binary operations (value op parameter, channel-wise, a scalar parameter is broadcast) and in
+// their two-input Unary forms (the value is a Tuple<I1, I2>, as DualSourceRead hands it over).
+// Interface counterpart: FK/algorithms/basic_ops/arithmetic.h:26-124.
 #ifndef FK_AMD_ARITHMETIC_H
 #define FK_AMD_ARITHMETIC_H
 
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+#include <fused_kernel/core/data/tuple.h>
 
 namespace fk {
+
+// The two-input form of an Operation Name<I1, I2, O, IT> whose primary template is already declared: the value is a
+// Tuple<I1, I2> and the body is the expression of fkd::fn::Name on its halves.  Shared with logical.h, bitwise.h, math.h.
+#define FK_AMD_TWO_INPUTS(Name)                                                                                 \
+    template <typename I1, typename I2, typename O>                                                             \
+    struct Name<I1, I2, O, UnaryType> : UnaryOperation<Tuple<I1, I2>, O, Name<I1, I2, O, UnaryType>> {          \
+        using Parent = UnaryOperation<Tuple<I1, I2>, O, Name<I1, I2, O, UnaryType>>;                            \
+        FK_STATIC_STRUCT(Name, Name)                                                                            \
+    };                                                                                                          \
+    namespace amd {                                                                                             \
+    template <typename I1, typename I2, typename O> struct Lower<Name<I1, I2, O, UnaryType>> {                  \
+        static constexpr bool available = true;                                                                 \
+        using type = fkd::Zip<fkd::fn::Name, dev_t<I1>, dev_t<I2>, dev_t<O>>;                                   \
+        static typename type::Params params(const OperationData<Name<I1, I2, O, UnaryType>>&) { return {}; }    \
+    };                                                                                                          \
+    }
 
 #define FK_AMD_ARITH(Name)                                                                                      \
     template <typename I1, typename I2 = I1, typename O = I1, typename IT = BinaryType> struct Name;            \
@@ -28,6 +45,9 @@ FK_AMD_ARITH(Add)
 FK_AMD_ARITH(Sub)
 FK_AMD_ARITH(Mul)
 #undef FK_AMD_ARITH
+FK_AMD_TWO_INPUTS(Add)
+FK_AMD_TWO_INPUTS(Sub)
+FK_AMD_TWO_INPUTS(Mul)
 
 // Div: the device parameter block also carries the correctly rounded reciprocal of the divisor (see fkd::Div).
 template <typename I1, typename I2 = I1, typename O = I1, typename IT = BinaryType> struct Div;
@@ -45,6 +65,8 @@ template <typename I, typename P, typename O> struct Lower<Div<I, P, O, BinaryTy
     }
 };
 }
+
+FK_AMD_TWO_INPUTS(Div)
 
 } // namespace fk
 #endif

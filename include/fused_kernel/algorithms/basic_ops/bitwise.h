@@ -1,7 +1,7 @@
 // BwAnd, BwOr, BwXor (value op constant), BwNot, ShiftLeft, ShiftRight (value shifted by a constant), per channel, as
 // Operations of a chain.  Interface counterpart: FK/algorithms/basic_ops/bitwise.h:23-157.  The results have the type
-// the C++ operator yields on the channel types (int for anything narrower), converted to O's channel type; the
-// two-input forms that take a Tuple are not provided.
+// the C++ operator yields on the channel types (int for anything narrower), converted to O's channel type.  BwAnd, BwOr
+// and BwXor also have the two-input forms that take a Tuple<I1, I2>.
 #ifndef FK_AMD_BITWISE_H
 #define FK_AMD_BITWISE_H
 #include <fused_kernel/algorithms/basic_ops/math.h>
@@ -9,6 +9,9 @@ namespace fk {
 FK_AMD_VALUE_AND_CONSTANT(BwAnd)
 FK_AMD_VALUE_AND_CONSTANT(BwOr)
 FK_AMD_VALUE_AND_CONSTANT(BwXor)
+FK_AMD_TWO_INPUTS(BwAnd)
+FK_AMD_TWO_INPUTS(BwOr)
+FK_AMD_TWO_INPUTS(BwXor)
 template <typename I, typename O = I> struct BwNot : UnaryOperation<I, O, BwNot<I, O>> {
     using Parent = UnaryOperation<I, O, BwNot<I, O>>;
     FK_STATIC_STRUCT(BwNot, BwNot)

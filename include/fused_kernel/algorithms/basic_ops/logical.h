@@ -2,7 +2,7 @@
 // use to compare results they have downloaded; IsEven<I>: whether an integer (each channel of an integer vector) is
 // even.  Interface counterpart: FK/algorithms/basic_ops/logical.h:23-35, 92-120.
 // Max<I, P, O> / Min<I, P, O>: the larger / smaller of value and constant per channel, std::max / std::min of two values
-// of one channel type (logical.h:37-88); their two-input forms that take a Tuple are not provided.
+// of one channel type (logical.h:37-88), and their two-input forms on a Tuple<I, P>.
 #ifndef FK_AMD_LOGICAL_H
 #define FK_AMD_LOGICAL_H
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
@@ -11,6 +11,8 @@
 namespace fk {
 FK_AMD_VALUE_AND_CONSTANT(Max)
 FK_AMD_VALUE_AND_CONSTANT(Min)
+FK_AMD_TWO_INPUTS(Max)
+FK_AMD_TWO_INPUTS(Min)
 template <typename I1, typename I2 = I1> struct Equal : UnaryOperation<Tuple<I1, I2>, bool, Equal<I1, I2>> {
     using Parent = UnaryOperation<Tuple<I1, I2>, bool, Equal<I1, I2>>;
     FK_STATIC_STRUCT(Equal, Equal)

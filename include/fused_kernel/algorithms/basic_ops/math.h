@@ -1,10 +1,10 @@
 // Abs, Sqr, Sqrt, Ln, Exp (one value in, per channel) and AbsDiff (|value - constant| per channel) as Operations of a
 // chain.  Interface counterpart: FK/algorithms/basic_ops/math.h:59-170; the expressions themselves are in
 // fkd::fn (include/fkd/ops.hpp).  As in the reference, O is the type the expression yields per channel (Sqr<uchar3>
-// needs O = int3, Sqrt<uchar3> O = float3); the two-input form of AbsDiff that takes a Tuple is not provided.
+// needs O = int3, Sqrt<uchar3> O = float3).  AbsDiff also has the two-input form that takes a Tuple<I1, I2>.
 #ifndef FK_AMD_MATH_H
 #define FK_AMD_MATH_H
-#include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+#include <fused_kernel/algorithms/basic_ops/arithmetic.h>
 namespace fk {
 #define FK_AMD_MATH_UNARY(Name)                                                                                  \
     template <typename I, typename O = I> struct Name : UnaryOperation<I, O, Name<I, O>> {                       \
@@ -43,5 +43,6 @@ FK_AMD_MATH_UNARY(Exp)
     };                                                                                                           \
     }
 FK_AMD_VALUE_AND_CONSTANT(AbsDiff)
+FK_AMD_TWO_INPUTS(AbsDiff)
 } // namespace fk
 #endif

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include <fused_kernel/core/execution_model/operation_model/operation_model.h>
+#include <fused_kernel/core/data/tuple.h>
 
 namespace fk {
 
@@ -70,6 +71,34 @@ struct SplitWrite : WriteOperation<T, SplitWriteParams<D, T>, VBase<T>, TF::DISA
     }
     static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.x.dims.width; }
     static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.x.dims.pitch; }
+};
+
+// DualSourceRead<D, T>: the elements of two images at the same position as a Tuple<T, T>, for the two-input forms of the
+// arithmetic, bitwise and comparison Operations (image-by-image work in one kernel).  The extent is the first image's.
+// Interface counterpart: FK/algorithms/basic_ops/memory_operations.h:585-640.
+template <ND D, typename T> struct DualSourceReadParams {
+    RawPtr<D, T> src1;
+    RawPtr<D, T> src2;
+};
+template <ND D, typename T>
+struct DualSourceRead : ReadOperation<T, DualSourceReadParams<D, T>, Tuple<T, T>, TF::DISABLED, DualSourceRead<D, T>> {
+    using Parent = ReadOperation<T, DualSourceReadParams<D, T>, Tuple<T, T>, TF::DISABLED, DualSourceRead<D, T>>;
+    using typename Parent::OperationDataType;
+    using typename Parent::InstantiableType;
+    FK_STATIC_STRUCT(DualSourceRead, DualSourceRead)
+    using Parent::build;
+    static InstantiableType build(const Ptr<D, T>& src1, const Ptr<D, T>& src2) { return {{DualSourceReadParams<D, T>{src1.ptr(), src2.ptr()}}}; }
+    static constexpr uint num_elems_x(const Point, const OperationDataType& opData) { return opData.params.src1.dims.width; }
+    static constexpr uint num_elems_y(const Point, const OperationDataType& opData) {
+        if constexpr (D == ND::_1D) return 1; else return opData.params.src1.dims.height;
+    }
+    static constexpr uint num_elems_z(const Point, const OperationDataType& opData) {
+        if constexpr (D == ND::_1D || D == ND::_2D) return 1; else return opData.params.src1.dims.planes;
+    }
+    static constexpr uint pitch(const Point, const OperationDataType& opData) { return opData.params.src1.dims.pitch; }
+    static constexpr ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return {num_elems_x(Point{0, 0, 0}, opData), num_elems_y(Point{0, 0, 0}, opData), num_elems_z(Point{0, 0, 0}, opData)};
+    }
 };
 
 // Deduces dimension and element type from the pointer: ReadOp::build(ptr), WriteOp::build(ptr).
@@ -285,6 +314,13 @@ template <typename T> struct Lower<PerThreadRead<ND::_2D, T>> {
     static constexpr bool available = true;
     using type = fkd::Read2D<dev_t<T>>;
     static typename type::Params params(const OperationData<PerThreadRead<ND::_2D, T>>& d) { return to_dev<T, const dev_t<T>>(d.params); }
+};
+template <typename T> struct Lower<DualSourceRead<ND::_2D, T>> {
+    static constexpr bool available = true;
+    using type = fkd::DualRead2D<dev_t<T>>;
+    static typename type::Params params(const OperationData<DualSourceRead<ND::_2D, T>>& d) {
+        return typename type::Params{to_dev<T, const dev_t<T>>(d.params.src1), to_dev<T, const dev_t<T>>(d.params.src2)};
+    }
 };
 template <typename T> struct Lower<PerThreadRead<ND::_1D, T>> {
     static constexpr bool available = true;

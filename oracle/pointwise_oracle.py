@@ -9,6 +9,8 @@ to (numpy integer arithmetic is done in the promoted type explicitly, then cast 
   BwAnd, BwOr, BwXor, BwNot, shifts  FK/algorithms/basic_ops/bitwise.h:23-157 with the operators of
                                      FK/core/utils/vector_utils.h:565-600
   MxVFloat3<BinaryType>              FK/algorithms/basic_ops/algebraic.h:25-40
+  the two-input forms on a pair      FK/algorithms/basic_ops/arithmetic.h:26-124 (Add, Sub, Mul, Div: the channel-wise operators of
+                                     vector_utils.h:508-563 on the two halves), and the UnaryType forms in the headers above
   per-channel application            FK/core/constexpr_libs/constexpr_vector_exec.h:24-108
 
 Pinned by: the reference's CPU backend on the same inputs (oracle/_ref, tests/test_oracle_pointwise.py), closed forms
@@ -146,4 +148,42 @@ def run(which, src, c=(0, 0, 0, 0), m=(1, 0, 0, 0, 1, 0, 0, 0, 1)):
     if which == 19: return op_shift(True, src, as_int(np.uint32), out_dtype)
     if which == 20: return op_shift(False, src, as_int(np.int32), out_dtype)
     if which == 21: return op_mxv3(src, m)
+    raise KeyError(which)
+
+
+# two-image chains of tests/cases/pointwise_chains.h (`dual`): which -> (input dtype, channels, output dtype)
+DUAL_CASES = {
+    0: (np.float32, 3, np.float32), 1: (np.uint8, 3, np.int32), 2: (np.float32, 1, np.float32), 3: (np.float32, 3, np.float32),
+    4: (np.float32, 3, np.float32), 5: (np.uint32, 1, np.uint32), 6: (np.float32, 3, np.float32), 7: (np.int32, 1, np.int32),
+    8: (np.uint8, 3, np.uint8), 9: (np.uint32, 1, np.uint32), 10: (np.uint32, 1, np.uint32),
+}
+
+
+def saturate_cast_u8(f):
+    """cxp::saturate_cast<uchar>(float), FK/core/constexpr_libs/constexpr_saturate.h:91-113: NaN -> 0, round half to even, clamp."""
+    f = f.astype(np.float32)
+    with np.errstate(invalid="ignore"):
+        r = np.rint(f)
+        return np.where(np.isnan(f), 0, np.clip(r, 0, 255)).astype(np.uint8)
+
+
+def run_dual(which, a, b):
+    """Two-image chain number `which`: DualSourceRead -> the two-input form of the Operation (-> more) -> write."""
+    in_dtype, cn, out_dtype = DUAL_CASES[which]
+    assert a.dtype == in_dtype and b.dtype == in_dtype and a.shape == b.shape
+    wa, wb = _promote(a), _promote(b)
+    with np.errstate(all="ignore"):
+        if which == 0: return (a + b).astype(np.float32)
+        if which == 1: return np.abs(wa - wb).astype(np.int32)                 # uchar - uchar is an int; d < 0 ? -d : d
+        if which == 2: return (a * b).astype(np.float32)
+        if which == 3: return (a / b).astype(np.float32)
+        if which == 4: return (a - b).astype(np.float32)
+        if which == 5: return np.bitwise_xor(a, b)
+        if which == 6: return np.where(a < b, b, a)
+        if which == 7: return np.where(b < a, b, a)
+        if which == 8:
+            s = (wa + wb).astype(np.int32)                                      # Add<uchar3, uchar3, int3>
+            return saturate_cast_u8(s.astype(np.float32) * np.float32(0.5))
+        if which == 9: return np.bitwise_and(a, b)
+        if which == 10: return np.bitwise_or(a, b)
     raise KeyError(which)

@@ -441,6 +441,13 @@ int fklref_split_write(int which, const void* src, int w, int h, int pitch, int 
     s.sync();
     return rc;
 }
+// Two-image chain number `which` of tests/cases/pointwise_chains.h on the CPU backend.
+int fklref_dual(int which, const void* a, const void* b, int w, int h, int pitch_a, int pitch_b, void* out, int out_pitch) {
+    CpuStream s;
+    const int rc = pointwise_chains::Chains<CpuDPP, CpuStream>::dual(s, MemType::Host, which, a, b, w, h, pitch_a, pitch_b, out, out_pitch);
+    s.sync();
+    return rc;
+}
 #ifndef FKL_HARNESS_PUBLIC_API_ONLY
 // ccMatrix<range, primaries, direction, depth> as the reference computes it at compile time, row major.
 // to_rgb = 1 selects YCbCr2RGB.

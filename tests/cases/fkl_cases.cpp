@@ -614,6 +614,14 @@ extern "C" int fklcase_split_write(void* stream_, int which, const void* src, in
     });
 }
 
+extern "C" int fklcase_dual(void* stream_, int which, const void* a, const void* b, int w, int h, int pitch_a, int pitch_b, void* out,
+                            int out_pitch) {
+    return guarded_rc([&] {
+        Stream s(stream_);
+        return pointwise_chains::Chains<TransformDPP<>, Stream>::dual(s, MemType::Device, which, a, b, w, h, pitch_a, pitch_b, out, out_pitch);
+    });
+}
+
 // ---- padding through BorderReader (border_chains.h on the GPU) ----------------------------------------------------
 extern "C" int fklcase_pad(void* stream_, int elem, int border_type, const void* src, int w, int h, int pitch, int left, int top,
                            int out_w, int out_h, const float* value, void* out, int out_pitch) {

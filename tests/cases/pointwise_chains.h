@@ -115,6 +115,38 @@ template <class DPP, class StreamT> struct Chains {
         default: return 2;
         }
     }
+
+    // ---- DualSourceRead<_2D, T> -> the two-input form of an Operation -> write ------------------------------------
+    template <class T, class O, class... IOps>
+    static void two(StreamT& s, MemType mem, const void* a, const void* b, int w, int h, int pitch_a, int pitch_b, void* out, int out_pitch,
+                    const IOps&... iops) {
+        const auto pa = wrap<T>(a, w, h, pitch_a, mem);
+        const auto pb = wrap<T>(b, w, h, pitch_b, mem);
+        const auto o = wrap<O>(out, w, h, out_pitch, mem);
+        executeOperations<DPP>(s, DualSourceRead<ND::_2D, T>::build(pa, pb), iops..., PerThreadWrite<ND::_2D, O>::build(o.ptr()));
+    }
+    // 0 Add<float3>            1 AbsDiff<uchar3 -> int3>   2 Mul<float>              3 Div<float3>
+    // 4 Sub<float3>            5 BwXor<uint>               6 Max<float3>             7 Min<int>
+    // 8 the mean of two uchar3 images: Add<uchar3 -> int3> -> Cast<int3, float3> -> Mul{0.5} -> SaturateCast<float3, uchar3>
+    // 9 BwAnd<uint>           10 BwOr<uint>
+    static int dual(StreamT& s, MemType mem, int which, const void* a, const void* b, int w, int h, int pitch_a, int pitch_b,
+                    void* out, int out_pitch) {
+        switch (which) {
+        case 0: two<float3, float3>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Add<float3, float3, float3, UnaryType>::build()); return 0;
+        case 1: two<uchar3, int3>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, AbsDiff<uchar3, uchar3, int3, UnaryType>::build()); return 0;
+        case 2: two<float, float>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Mul<float, float, float, UnaryType>::build()); return 0;
+        case 3: two<float3, float3>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Div<float3, float3, float3, UnaryType>::build()); return 0;
+        case 4: two<float3, float3>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Sub<float3, float3, float3, UnaryType>::build()); return 0;
+        case 5: two<uint, uint>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, BwXor<uint, uint, uint, UnaryType>::build()); return 0;
+        case 6: two<float3, float3>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Max<float3, float3, float3, UnaryType>::build()); return 0;
+        case 7: two<int, int>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Min<int, int, int, UnaryType>::build()); return 0;
+        case 8: two<uchar3, uchar3>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, Add<uchar3, uchar3, int3, UnaryType>::build(),
+                                    Cast<int3, float3>::build(), Mul<float3>::build(make_set<float3>(0.5f)), SaturateCast<float3, uchar3>::build()); return 0;
+        case 9: two<uint, uint>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, BwAnd<uint, uint, uint, UnaryType>::build()); return 0;
+        case 10: two<uint, uint>(s, mem, a, b, w, h, pitch_a, pitch_b, out, out_pitch, BwOr<uint, uint, uint, UnaryType>::build()); return 0;
+        default: return 2;
+        }
+    }
 };
 
 } // namespace pointwise_chains

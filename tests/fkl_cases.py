@@ -319,6 +319,13 @@ def split_write(which, src_bytes, width, height, outs, dst=None, c=(1, 1, 1, 1))
                                     ptrs, pitches, cv.ctypes.data_as(C.c_void_p)))
 
 
+def dual(which, a_bytes, b_bytes, width, height, out_bytes):
+    """Two-image chain number `which` of tests/cases/pointwise_chains.h; the three arguments are 2-D u8 cuda tensors holding
+    the rows of the two inputs and of the output (each with a pitch of its own)."""
+    _ok(cases().fklcase_dual(_stream(), int(which), _p(a_bytes), _p(b_bytes), int(width), int(height), _pitch(a_bytes), _pitch(b_bytes),
+                             _p(out_bytes), _pitch(out_bytes)))
+
+
 def pad(src, border_type, left, top, out, value=(0, 0, 0)):
     """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out."""
     v = np.zeros(4, np.float32)

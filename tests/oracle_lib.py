@@ -717,6 +717,24 @@ def ref_pointwise(which, src, c=(0, 0, 0, 0), m=(1, 0, 0, 0, 1, 0, 0, 0, 1)):
     return out
 
 
+def ref_dual(which, a, b, pad=(0, 0)):
+    """Two-image chain `which` of tests/cases/pointwise_chains.h on the reference's CPU backend; `pad`: extra bytes at the end
+    of the rows of the first and of the second image (the two sources have pitches of their own)."""
+    in_dtype, cn, out_dtype = pointwise_oracle().DUAL_CASES[which]
+    h, w = a.shape[:2]
+    row = w * cn * np.dtype(in_dtype).itemsize
+    bufs = []
+    for img, extra in ((a, pad[0]), (b, pad[1])):
+        buf = np.zeros((h, row + extra), np.uint8)
+        buf[:, :row] = np.ascontiguousarray(img, dtype=in_dtype).view(np.uint8).reshape(h, row)
+        bufs.append(buf)
+    out = np.zeros(a.shape, out_dtype)
+    rc = ref().fklref_dual(int(which), C.c_void_p(_ptr(bufs[0])), C.c_void_p(_ptr(bufs[1])), w, h, bufs[0].strides[0], bufs[1].strides[0],
+                           C.c_void_p(_ptr(out)), out.strides[0])
+    assert rc == 0, rc
+    return out
+
+
 # SplitWrite chains of tests/cases/pointwise_chains.h: which -> (input dtype, channels, output dtype)
 SPLIT_WRITE_CASES = {0: (np.uint8, 3, np.uint8), 1: (np.uint8, 3, np.float32), 2: (np.float32, 4, np.float32),
                      3: (np.uint8, 3, np.float32), 4: (np.float32, 2, np.float32)}

@@ -57,3 +57,28 @@ def same(which, got, want, inexact):
     tiny = np.abs(w) < 1e-37                         # results in the denormal range: flushing is platform business
     sel = finite & ~tiny
     return bool(ok and np.all(np.abs(g[sel] - w[sel]) <= 1e-5 * np.abs(w[sel])) and np.all(np.abs(g[finite & tiny]) < 2e-37))
+
+
+def dual_inputs(which, cases, h, w, seed):
+    """Two images for the two-image chains: seeded values with zeros, NaN, infinities and the extreme integers mixed in."""
+    in_dtype, cn, _ = cases[which]
+    rng = np.random.default_rng(7000 + 10 * which + seed)
+    shape = (h, w, cn) if cn > 1 else (h, w)
+    n = h * w * cn
+    out = []
+    for k in range(2):
+        if in_dtype == np.float32:
+            v = rng.uniform(-50.0, 50.0, n).astype(np.float32)
+            special = [0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, 3.4e38, 1e-38][k:] + [2.0, -3.0]
+            v[: len(special)] = np.array(special, np.float32)
+        elif in_dtype == np.uint8:
+            v = rng.integers(0, 256, n, dtype=np.uint8)
+            v[:4] = [0, 255, 255, 1] if k == 0 else [255, 0, 255, 2]
+        elif in_dtype == np.int32:
+            v = rng.integers(-2**31, 2**31, n, dtype=np.int64).astype(np.int32)
+            v[:2] = [-2**31, 2**31 - 1] if k == 0 else [2**31 - 1, -2**31]
+        else:
+            v = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+            v[:2] = [0, 0xffffffff]
+        out.append(v.reshape(shape))
+    return out

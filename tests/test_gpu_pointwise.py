@@ -84,3 +84,37 @@ def test_split_write_matches_the_oracle(device, which):
             got = bufs[k].cpu().numpy()
             assert got[:, :dw].tobytes() == want[k].tobytes(), (which, seed, k)
             assert np.all(got[:, dw:] == 77), "padding columns were written"
+
+
+def _same_with_any_nan(got, want):
+    """Bit-exact, except that a NaN the operation itself produced (inf - inf, 0 / 0 ...) counts as equal to any NaN: which
+    quiet NaN an invalid operation returns is the platform's choice (x86 sets the sign bit, the GPU does not)."""
+    if got.dtype != np.float32:
+        return got.tobytes() == want.tobytes()
+    gn, wn = np.isnan(got), np.isnan(want)
+    return np.array_equal(gn, wn) and got[~gn].tobytes() == want[~wn].tobytes()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", sorted(po.DUAL_CASES))
+def test_two_image_chain_matches_the_oracle(device, which):
+    # DualSourceRead<_2D, T> -> the two-input form of Add / Sub / Mul / Div / AbsDiff / Max / Min / BwAnd / BwOr / BwXor -> write
+    import torch
+    in_dtype, cn, out_dtype = po.DUAL_CASES[which]
+    for seed, (h, w, pad_a, pad_b) in enumerate(((6, 11, 0, 0), (19, 34, 0, 8), (64, 256, 4, 0))):
+        a, b = pc.dual_inputs(which, po.DUAL_CASES, h, w, seed)
+        want = po.run_dual(which, a, b)
+        row = w * cn * np.dtype(in_dtype).itemsize
+        devs = []
+        for img, extra in ((a, pad_a), (b, pad_b)):
+            buf = np.zeros((h, row + extra), np.uint8)
+            buf[:, :row] = np.ascontiguousarray(img).view(np.uint8).reshape(h, row)
+            devs.append(torch.from_numpy(buf).to(device))
+        out_row = w * cn * np.dtype(out_dtype).itemsize
+        dev_out = torch.full((h, out_row + 4), 0xA5, dtype=torch.uint8, device=device)
+        cases.dual(which, devs[0], devs[1], w, h, dev_out)
+        torch.cuda.synchronize()
+        got = dev_out.cpu().numpy()
+        assert np.all(got[:, out_row:] == 0xA5)
+        got = np.ascontiguousarray(got[:, :out_row]).view(out_dtype).reshape(want.shape)
+        assert _same_with_any_nan(got, want), (which, seed)

@@ -131,3 +131,9 @@ def test_resize_geometry_of_every_aspect_ratio_mode():
 @pytest.mark.parametrize("which", sorted(ol.SPLIT_WRITE_CASES))
 def test_split_write(which):
     on_host_executor(t_pointwise.test_split_write_equals_the_reference_backend, which)
+
+
+@pytest.mark.parametrize("which", sorted(t_pointwise.po.DUAL_CASES))
+def test_two_image_chains(which):
+    # DualSourceRead and the two-input forms of Add ... BwOr on this repository's CPU executor
+    on_host_executor(t_pointwise.test_two_image_chains_equal_the_reference_backend, which)

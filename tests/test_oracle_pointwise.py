@@ -94,3 +94,28 @@ def test_split_write_equals_the_reference_backend(which):
         assert len(got) == len(want)
         for g, r in zip(got, want):
             assert g.dtype == r.dtype and g.tobytes() == r.tobytes(), (which, seed)
+
+
+def test_two_image_closed_forms():
+    a = np.array([[[1.0, 2.0, 3.0]]], np.float32)
+    b = np.array([[[0.5, -2.0, 4.0]]], np.float32)
+    assert po.run_dual(0, a, b).tolist() == [[[1.5, 0.0, 7.0]]] and po.run_dual(4, a, b).tolist() == [[[0.5, 4.0, -1.0]]]
+    assert po.run_dual(3, a, b).tolist() == [[[2.0, -1.0, 0.75]]] and po.run_dual(6, a, b).tolist() == [[[1.0, 2.0, 4.0]]]
+    u = np.array([[[0, 255, 7]]], np.uint8)
+    v = np.array([[[255, 0, 9]]], np.uint8)
+    assert po.run_dual(1, u, v).tolist() == [[[255, 255, 2]]]                    # the difference is taken in int
+    assert po.run_dual(8, u, v).tolist() == [[[128, 128, 8]]]                    # 127.5 rounds to the even 128, 8.0 stays
+    x = np.array([[0xff00ff00, 0x0f0f0f0f]], np.uint32)
+    y = np.array([[0x0ff00ff0, 0xffffffff]], np.uint32)
+    assert po.run_dual(5, x, y).tolist() == [[0xf0f0f0f0, 0xf0f0f0f0]] and po.run_dual(9, x, y).tolist() == [[0x0f000f00, 0x0f0f0f0f]]
+    assert po.run_dual(7, np.array([[5, -9]], np.int32), np.array([[-5, 9]], np.int32)).tolist() == [[-5, -9]]
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="oracle/_ref not built")
+@pytest.mark.parametrize("which", sorted(po.DUAL_CASES))
+def test_two_image_chains_equal_the_reference_backend(which):
+    for seed, (h, w) in enumerate(((6, 11), (19, 34))):
+        a, b = pc.dual_inputs(which, po.DUAL_CASES, h, w, seed)
+        want = ol.ref_dual(which, a, b, pad=(0, 8))
+        got = po.run_dual(which, a, b)
+        assert got.dtype == want.dtype and got.tobytes() == want.tobytes(), (which, seed)
