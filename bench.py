@@ -220,7 +220,15 @@ def main():
         record("circular_tensor_update_b8_720p", 8 * px, px * 3 + 2 * px * 12 + 7 * 2 * px * 12, lambda: cases.circular_update_b8(frames),
                max(10, args.steps // 4), max(2, args.warmup // 4))
         cases.circular_update_b8(frames, release=True)
-        del fo, po, uyvy, nv12, t4, d4, frames
+        # two images in, one out (DualSourceRead -> Add -> Cast -> Mul -> SaturateCast), and one image out as three planes
+        img2 = torch.from_numpy(rng.randint(0, 256, (H, W, 3)).astype(np.uint8)).to(dev)
+        mean = torch.zeros((H, W * 3), dtype=torch.uint8, device=dev)
+        record("mean_of_two_1080p_u8x3", W * H, 3 * W * H * 3, lambda: cases.dual(8, img.view(H, W * 3), img2.view(H, W * 3), W, H, mean),
+               args.steps, args.warmup)
+        planes = [torch.zeros((H, W), dtype=torch.float32, device=dev) for _ in range(3)]
+        record("u8x3_to_three_float_planes_1080p", W * H, W * H * (3 + 12),
+               lambda: cases.split_write(1, img.view(H, W * 3), W, H, planes, None, (1 / 255.0, 1 / 255.0, 1 / 255.0, 0)), args.steps, args.warmup)
+        del fo, po, uyvy, nv12, t4, d4, frames, img2, mean, planes
 
     # ---- configuration 3, the headline: W warm-up steps, then exactly K timed steps ---------------------------------
     r3 = record("c3", 64 * 224 * 224, a3, f3, args.steps, args.warmup)

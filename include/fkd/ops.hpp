@@ -1387,6 +1387,16 @@ template <class B> FKD_DEV void pin_base(B& b) {
     else if constexpr (sizeof(B) < 4) { u32 w = detail::to_bits(b); asm volatile("" : "+v"(w)); b = __builtin_bit_cast(B, decltype(detail::to_bits(b))(w)); }
     else { unsigned long long w = __builtin_bit_cast(unsigned long long, b); asm volatile("" : "+v"(w)); b = __builtin_bit_cast(B, w); }
 }
+// A channel value the optimiser may not look behind (free to schedule, unlike pin_base): keeps it from gluing the channels
+// of several 12-byte values into odd-sized vectors (<6 x float>) that it can then only shuffle through memory.
+template <class B> FKD_DEV B opaque(B b) {
+    if constexpr (sizeof(B) == 4) asm("" : "+v"(b));
+    return b;
+}
+constexpr int kSharedValues = 8;      // access-mode bit: see TeeWrite
+template <bool OPAQUE, class B> FKD_DEV B maybe_opaque(B b) {
+    if constexpr (OPAQUE) return opaque(b); else return b;
+}
 template <class V> FKD_DEV void pin_value(V& v) {
     pin_base(chan<0>(v));
     if constexpr (cn_v<V> > 1) pin_base(chan<1>(v));
@@ -2515,7 +2525,7 @@ template <class T> struct ReadSet {
 #if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int, int, int, const Params& p, Slot<T> (&out)[V]) {
 #pragma unroll
-        for (int i = 0; i < V; ++i) out[i].v = p.value;
+        for (int i = 0; i < V; ++i) out[i].v = map1<T>(p.value, [](auto c) { return opaque(c); });   // (see opaque)
     }
     FKD_HD static bool rows_aligned(const Params&, int) { return true; }
 #endif
@@ -2597,17 +2607,26 @@ template <class T> struct SplitWrite2D {
     }
 #endif
 #if defined(FKD_DEVICE_CODE)
-    template <int I, int V, int A> FKD_DEV static void channel_run(int x, int y, const Slot<T> (&v)[V], const Params& p) {
-        Slot<B> run[V];
-#pragma unroll
-        for (int i = 0; i < V; ++i) run[i].v = pick<I>(v[i].v);
-        detail::store_run<B, V, A>(detail::row_ptr(p.c[I].data, p.c[I].pitch, x, y), run);
-    }
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int, const Slot<T> (&v)[V], const Params& p) {
-        channel_run<0, V, A>(x, y, v, p);
-        channel_run<1, V, A>(x, y, v, p);
-        if constexpr (N > 2) channel_run<2, V, A>(x, y, v, p);
-        if constexpr (N > 3) channel_run<3, V, A>(x, y, v, p);
+        // (the channels are taken apart in one pass over the values, as TensorSplit does: taken apart channel by channel
+        // in separate passes, the value array stayed in memory)
+        Slot<B> c0[V], c1[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) { c0[i].v = chan<0>(v[i].v); c1[i].v = chan<1>(v[i].v); }
+        detail::store_run<B, V, A>(detail::row_ptr(p.c[0].data, p.c[0].pitch, x, y), c0);
+        detail::store_run<B, V, A>(detail::row_ptr(p.c[1].data, p.c[1].pitch, x, y), c1);
+        if constexpr (N > 2) {
+            Slot<B> c2[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) c2[i].v = chan<2>(v[i].v);
+            detail::store_run<B, V, A>(detail::row_ptr(p.c[2].data, p.c[2].pitch, x, y), c2);
+        }
+        if constexpr (N > 3) {
+            Slot<B> c3[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) c3[i].v = chan<3>(v[i].v);
+            detail::store_run<B, V, A>(detail::row_ptr(p.c[3].data, p.c[3].pitch, x, y), c3);
+        }
     }
     FKD_HD static bool rows_aligned(const Params& p) {
         bool ok = true;
@@ -2704,21 +2723,22 @@ template <class T, bool TRANSPOSED = false> struct TensorSplit {
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<T> (&v)[V], const Params& p) {
         B* w = at(p, x, y, z);
         const size_t px = G::channel_elements(p);
+        constexpr bool S = (A & kSharedValues) != 0;      // see TeeWrite
         Slot<B> c0[V], c1[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) { c0[i].v = chan<0>(v[i].v); c1[i].v = chan<1>(v[i].v); }
+        for (int i = 0; i < V; ++i) { c0[i].v = maybe_opaque<S>(chan<0>(v[i].v)); c1[i].v = maybe_opaque<S>(chan<1>(v[i].v)); }
         detail::store_run<B, V, A>(w, c0);
         detail::store_run<B, V, A>(w + px, c1);
         if constexpr (cn_v<T> > 2) {
             Slot<B> c2[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) c2[i].v = chan<2>(v[i].v);
+            for (int i = 0; i < V; ++i) c2[i].v = maybe_opaque<S>(chan<2>(v[i].v));
             detail::store_run<B, V, A>(w + 2 * px, c2);
         }
         if constexpr (cn_v<T> > 3) {
             Slot<B> c3[V];
 #pragma unroll
-            for (int i = 0; i < V; ++i) c3[i].v = chan<3>(v[i].v);
+            for (int i = 0; i < V; ++i) c3[i].v = maybe_opaque<S>(chan<3>(v[i].v));
             detail::store_run<B, V, A>(w + 3 * px, c3);
         }
     }
@@ -2934,8 +2954,11 @@ template <class W1, class W2> struct TeeWrite {
 #endif
 #if defined(FKD_DEVICE_CODE)
     template <int V, int A> FKD_DEV static void exec_row(int x, int y, int z, const Slot<In> (&v)[V], const Params& p) {
-        W1::template exec_row<V, A>(x, y, z, v, p.first);
-        W2::template exec_row<V, A>(x, y, z, v, p.second);
+        // Bit 8 of the access mode tells a planar write that another write reads the same values: it then takes the
+        // channels apart behind opaque points (see opaque).  Without them the array of 12-byte values that two writes take
+        // apart one after the other is kept in memory.
+        W1::template exec_row<V, A | kSharedValues>(x, y, z, v, p.first);
+        W2::template exec_row<V, A | kSharedValues>(x, y, z, v, p.second);
     }
     FKD_HD static bool rows_aligned(const Params& p) { return W1::rows_aligned(p.first) && W2::rows_aligned(p.second); }
 #endif

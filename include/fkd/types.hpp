@@ -99,7 +99,12 @@ template <class O, class A, class B, class F> FKD_HD O map2(const A& a, const B&
 struct Empty {};
 
 // Two values travelling through a chain side by side (what a read of two sources hands to a two-input operation).
-template <class A, class B> struct Two { A a; B b; };
+// Each half starts on a dword when its size is not a multiple of four (uchar3 ...), like an element of a per-thread array
+// (fkd::Slot): halves packed at byte offsets make the optimiser build 24-bit vectors that only scratch memory can hold.
+template <class A, class B> struct Two {
+    alignas(sizeof(A) % 4 != 0 ? 4 : alignof(A)) A a;
+    alignas(sizeof(B) % 4 != 0 ? 4 : alignof(B)) B b;
+};
 
 // Heterogeneous parameter pack with a layout both compilers agree on (plain nested aggregates).
 template <class... Ts> struct Tup;

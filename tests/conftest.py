@@ -9,6 +9,12 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
         sys.path.insert(0, p)
 
 
+# A chain compiled at run time that needs scratch memory (a per-thread array the optimiser could not keep in registers: an
+# order of magnitude slower, silently) is refused during the tests, like the ahead-of-time build refuses it; the reference's
+# programs that tests/test_gpu_reference_programs.py starts inherit the setting.
+os.environ.setdefault("FKLHIP_JIT_STRICT", "1")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
