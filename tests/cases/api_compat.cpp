@@ -269,3 +269,19 @@ static_assert(std::is_same_v<fk::TensorTSplit<float3>::ParamsType, fk::RawPtr<fk
               std::is_same_v<fk::TensorTPack<float3>::OutputType, float3> && !fk::TensorTSplit<float3>::THREAD_FUSION);
 static_assert(std::is_base_of_v<fk::TensorT<float>, fk::CircularTensor<float, 3, 4, fk::CircularTensorOrder::NewestFirst, fk::ColorPlanes::Transposed>> &&
               std::is_base_of_v<fk::Tensor<float>, fk::CircularTensor<float, 3, 4, fk::CircularTensorOrder::NewestFirst, fk::ColorPlanes::Standard>>);
+
+// ---- Two-image chains, SplitWrite and the per-channel Operations: the reference's types -------------------------------
+#include <fused_kernel/algorithms/basic_ops/basic_ops.h>
+static_assert(std::is_same_v<fk::DualSourceRead<fk::ND::_2D, uchar3>::OutputType, fk::Tuple<uchar3, uchar3>> &&
+              fk::opIs<fk::ReadType, fk::DualSourceRead<fk::ND::_2D, uchar3>> && !fk::DualSourceRead<fk::ND::_2D, uchar3>::THREAD_FUSION);
+static_assert(std::is_same_v<fk::Add<uchar3, uchar3, int3, fk::UnaryType>::InputType, fk::Tuple<uchar3, uchar3>> &&
+              fk::opIs<fk::UnaryType, fk::Add<uchar3, uchar3, int3, fk::UnaryType>> && fk::opIs<fk::BinaryType, fk::Add<float>>);
+static_assert(fk::opIs<fk::UnaryType, fk::AbsDiff<float, float, float, fk::UnaryType>> && fk::opIs<fk::BinaryType, fk::AbsDiff<float>> &&
+              fk::opIs<fk::UnaryType, fk::BwNot<uint>> && fk::opIs<fk::BinaryType, fk::ShiftLeft<uint>> && fk::opIs<fk::BinaryType, fk::Max<float3>>);
+static_assert(std::is_same_v<fk::SplitWrite<fk::ND::_2D, float3>::InputType, float3> && fk::opIs<fk::WriteType, fk::SplitWrite<fk::ND::_2D, float3>> &&
+              std::is_same_v<decltype(fk::SplitWriteParams<fk::ND::_2D, uchar4>::w), fk::RawPtr<fk::ND::_2D, uchar>>);
+static_assert(std::is_same_v<fk::MxVFloat3<>::ParamsType, fk::M3x3Float> && std::is_same_v<fk::Sqrt<uchar3, float3>::OutputType, float3>);
+constexpr auto twoImages = fk::DualSourceRead<fk::ND::_2D, float>::build(fk::DualSourceReadParams<fk::ND::_2D, float>{
+    fk::RawPtr<fk::ND::_2D, float>{nullptr, {8, 8, 32}}, fk::RawPtr<fk::ND::_2D, float>{nullptr, {8, 8, 32}}});
+constexpr auto summed = twoImages.then(fk::Add<float, float, float, fk::UnaryType>::build()).then(fk::Mul<float>::build(0.5f));
+static_assert(fk::opIs<fk::ReadType, decltype(summed)>, "the two-input form fuses onto the read of two images");
