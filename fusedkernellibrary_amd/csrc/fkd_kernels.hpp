@@ -84,6 +84,15 @@ constexpr int kRowsBX = 64;   // lanes along x: one wave per row segment
 constexpr int kRowsBY = 4;    // waves per workgroup
 constexpr unsigned long long kStreamElements = 1ull << 26;   // launches over more elements stream their input
 
+// For the test of what run-time compilation does with a chain whose per-thread array cannot stay in registers: with
+// FKD_TEST_UNRESOLVED_INDEX defined, the rows kernel indexes its values with an offset that is zero when the kernel runs
+// but unknown when it is compiled (an index the optimiser cannot resolve keeps the array in memory).  Zero otherwise.
+#ifdef FKD_TEST_UNRESOLVED_INDEX
+#define FKD_TEST_INDEX_OFFSET int(p.active_w >> 31)
+#else
+#define FKD_TEST_INDEX_OFFSET 0
+#endif
+
 // The full-width part of the rows kernel: every lane has V elements in each of its ROWS rows.  MODE as in
 // detail::load_run.
 template <class Chain, int V, int ROWS, int MODE>
@@ -111,7 +120,7 @@ __device__ __forceinline__ void rows_full(const typename Chain::Params& p, u32 k
         const int y = ybase + r;
         Slot<typename Chain::Value> row[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) row[i].v = out[r * V + i].v;
+        for (int i = 0; i < V; ++i) row[i].v = out[r * V + i + FKD_TEST_INDEX_OFFSET].v;
         if (y < ah) W::template exec_row<V, MODE>(x0, y, z, row, p.write);
     }
 }

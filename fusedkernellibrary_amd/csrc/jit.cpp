@@ -259,7 +259,9 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
 const char* jit_last_log() { return g_log.c_str(); }
 
 // Compile (or fetch from the cache directory) and register; the caller holds g_compile_mu.
-static int build_and_register(const char* signature, bool may_read_cache) {
+// `arrays_to_lds`: compile without the build's -disable-promote-alloca-to-lds, so that a per-thread array the optimiser
+// cannot keep in registers goes to LDS instead of scratch memory (the second attempt for such a chain, see below).
+static int build_and_register(const char* signature, bool may_read_cache, bool arrays_to_lds = false) {
     const std::string arch_name = device_arch();
     const std::string cached = cache_path(signature, arch_name);
     JitKernel* k = new JitKernel();   // lives as long as the registry entry: for the life of the process
@@ -281,7 +283,11 @@ static int build_and_register(const char* signature, bool may_read_cache) {
         const std::string arch = "--offload-arch=" + arch_name;
         std::vector<const char*> opts;
         opts.push_back(arch.c_str());
-        for (int i = 0; i < kJitFlagCount; ++i) opts.push_back(kJitFlags[i]);
+        for (int i = 0; i < kJitFlagCount; ++i) {
+            if (arrays_to_lds && strcmp(kJitFlags[i], "-mllvm") == 0 && i + 1 < kJitFlagCount &&
+                strncmp(kJitFlags[i + 1], "-disable-promote-alloca-to-lds", 30) == 0) { ++i; continue; }
+            opts.push_back(kJitFlags[i]);
+        }
         const std::vector<std::string> defines = extra_defines();
         for (const std::string& d : defines) opts.push_back(d.c_str());
         r = hiprtcCompileProgram(prog, int(opts.size()), opts.data());
@@ -317,14 +323,15 @@ static int build_and_register(const char* signature, bool may_read_cache) {
         delete k;
         if (from_cache) {
             // an unreadable or foreign file: compile afresh (which replaces it)
-            return build_and_register(signature, false);
+            return build_and_register(signature, false, arrays_to_lds);
         }
         g_log = std::string("loading the compiled chain failed: ") + hipGetErrorString(e);
         return int(e);
     }
     // The ahead-of-time build refuses kernels that need scratch memory (a private array the optimiser could not keep in
-    // registers, or spills: a silent slowdown of an order of magnitude).  A chain compiled here still runs, the note goes
-    // into the log; with FKLHIP_JIT_STRICT=1 it is refused like there.
+    // registers, or spills: a silent slowdown of an order of magnitude).  A chain compiled here still runs: it is compiled
+    // once more with such arrays moved to LDS, which is the faster of the two homes, and the note goes into the log; with
+    // FKLHIP_JIT_STRICT=1 it is refused like there.
     int scratch_bytes = 0;
     if (hipFuncGetAttribute(&scratch_bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, fn) != hipSuccess) scratch_bytes = 0;
     if (scratch_bytes > 0) {
@@ -335,6 +342,13 @@ static int build_and_register(const char* signature, bool may_read_cache) {
             delete k;
             g_log = note + " (refused: FKLHIP_JIT_STRICT=1)";
             return FKLHIP_EUNKNOWN_SIGNATURE;
+        }
+        if (!arrays_to_lds) {
+            hipModuleUnload(mod);
+            delete k;
+            const int rc = build_and_register(signature, false, true);
+            g_log = note + "; compiled again with per-thread arrays in LDS" + (g_log.empty() ? std::string() : ": " + g_log);
+            return rc;
         }
         g_log = note;
     } else if (from_cache) {

@@ -106,3 +106,25 @@ def test_code_objects_are_reused_from_the_cache_directory(device, tmp_path):
     r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(res)], env=env, capture_output=True, text=True, timeout=240)
     assert r.returncode == 0, r.stderr[-2000:]
     assert np.load(res).tobytes() == outs[0][0].tobytes() and os.path.getsize(path) > 1000
+
+
+def test_a_chain_that_would_need_scratch_memory_is_compiled_again_or_refused(device, tmp_path):
+    """A per-thread array that cannot stay in registers (forced here through the kernel's test hook): by default the chain is
+    compiled a second time with the array in LDS, runs, and the log says so; with FKLHIP_JIT_STRICT=1 it is refused."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    hook = "-DFKD_TEST_UNRESOLVED_INDEX=1"
+    res = tmp_path / "out.npy"
+    env = dict(os.environ, FKLHIP_JIT_DEFINES=hook, FKLHIP_JIT_STRICT="0")
+    r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(res)], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "bytes of scratch memory per lane; compiled again with per-thread arrays in LDS" in r.stdout, r.stdout
+    ref = tmp_path / "ref.npy"
+    r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(ref)], env=dict(os.environ), capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert np.load(res).tobytes() == np.load(ref).tobytes()
+    env["FKLHIP_JIT_STRICT"] = "1"
+    r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(res)], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode != 0 and "could not be compiled at run time" in r.stderr, r.stderr[-2000:]
