@@ -9,8 +9,9 @@ BGR->RGB -> (x - mean) / std -> planar float32 64x3x224x224), issued through the
 Every measurement is W warm-up steps, a synchronisation, and then exactly K timed steps back to back on one stream.  The
 events (and the host clock) that bracket the K steps are taken by the case driver itself, right before its first launch
 and right after its last: this script needs about 100 us of Python to marshal a call's arguments, and with the bracket
-around the Python call a short run (K = 20) would charge that idle time to the kernel.  `kernel_us_5_runs_min_mean_max`
-of the headline shows the K steps repeated four more times.
+around the Python call a short run (K = 20) would charge that idle time to the kernel.  Every measurement starts after
+30 ms of GPU idle (see Timer.run).  `kernel_us_5_runs_min_mean_max` of the headline shows the K steps repeated four more
+times, `kernel_us_1000_launches` one batch of 1000 launches (the first launches after idle are then a small part).
 
 Prints ONE JSON line.  `value` is output Mpix/s of the whole job; `roofline` prices the kernel's algorithmic bytes
 against the 8 TB/s HBM peak using the launch duration measured with HIP events on the launch stream;
@@ -60,9 +61,16 @@ class Timer:
         fkl.check(self.lib.fklhip_event_create(C.byref(self.e0)), "event_create")
         fkl.check(self.lib.fklhip_event_create(C.byref(self.e1)), "event_create")
 
-    def run(self, fn, steps, warmup):
+    def run(self, fn, steps, warmup, settle=0.03):
         torch = self.torch
         stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        # Every measurement starts from a GPU that has been idle for a moment.  A short batch of launches that follows the
+        # end of another burst within a few milliseconds catches the GPU on its way down to its idle state and reads up to
+        # 30 % slower (measured: 20 launches of configuration 3 right after 300 others, median 10.6 us per launch; after
+        # 20 ms of idle 8.37 us, and never above 8.8 us); which of the two a line got used to depend on what ran before it.
+        if settle > 0:
+            torch.cuda.synchronize()
+            time.sleep(settle)
         if warmup > 0:
             self.cases.set_reps(warmup)
             fn()
@@ -234,8 +242,12 @@ def main():
     r3 = record("c3", 64 * 224 * 224, a3, f3, args.steps, args.warmup)
     got3 = out3.cpu().numpy()
     # the same K steps four more times, for the spread (not used for `value`)
-    again = [timer.run(f3, args.steps, 0)[1] * 1e3 for _ in range(4)] + [r3["kernel_us"]]
+    again = [timer.run(f3, args.steps, args.warmup)[1] * 1e3 for _ in range(4)] + [r3["kernel_us"]]
     r3["kernel_us_5_runs_min_mean_max"] = [min(again), sum(again) / len(again), max(again)]
+    # and one long batch: what a launch costs once the first launches after the idle state are a small part of the batch
+    # (the second of two such batches: the first also pays for the launch queue's and the runtime's argument buffers growing)
+    timer.run(f3, 1000, 300, settle=0)
+    r3["kernel_us_1000_launches"] = timer.run(f3, 1000, 0, settle=0)[1] * 1e3
 
     if args.list_compiled:
         # kernel symbol of every chain compiled at run time ("fkd_jit_" + FNV-1a of the signature), for reading profiles
@@ -282,7 +294,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": r3["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": r3["frac_of_hbm_peak"], "traffic": TRAFFIC_C3_BYTES,
                      "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"],
-                     "kernel_us_5_runs_min_mean_max": r3["kernel_us_5_runs_min_mean_max"]},
+                     "kernel_us_5_runs_min_mean_max": r3["kernel_us_5_runs_min_mean_max"],
+                     "kernel_us_1000_launches": r3["kernel_us_1000_launches"],
+                     "frac_1000_launches": a3 / (r3["kernel_us_1000_launches"] * 1e-6) / 1e9 / HBM_PEAK_GBS},
         "cpu_baseline": cpu,
         "others": {k: v for k, v in results.items() if k != "c3"},
     }
