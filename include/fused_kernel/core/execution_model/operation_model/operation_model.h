@@ -54,7 +54,10 @@ struct OpenType {};
 struct ClosedType {};
 
 struct NullType {};
-template <typename... Ts> struct TypeList {};
+template <typename... Ts> struct TypeList {
+    static constexpr size_t size = sizeof...(Ts);
+    template <size_t I> using at = std::tuple_element_t<I, std::tuple<Ts...>>;
+};
 // one_of_v<T, TypeList<...>>: T is one of the listed types.  EquivalentType_t<T, ListA, ListB>: the type of ListB at the
 // position T has in ListA.  Interface counterpart: FK/core/utils/type_lists.h.
 template <typename T, typename TL> struct one_of;

@@ -23,7 +23,8 @@ TESTS = ["tests_algorithm_test_crop", "tests_algorithm_test_batchresize_build", 
          # ones this library computes) and of Deinterlace
          "utests_algorithm_image_processing_utest_color_conversion", "utests_algorithm_image_processing_utest_deinterlace"]
 # host-only logic (no device call): also run where there is no GPU
-HOST_TESTS = ["tests_thread_fusion_test_thread_fusion", "tests_string_test_struct_to_string", "tests_string_test_literal_to_string"]
+HOST_TESTS = ["tests_thread_fusion_test_thread_fusion", "tests_string_test_struct_to_string", "tests_string_test_literal_to_string",
+              "tests_data_test_typelist"]
 BENCHMARKS = ["benchmarks_fusion_benchmark_horizontal_fusion", "benchmarks_fusion_benchmark_thread_fusion",
               "benchmarks_latencyhiding_benchmark_latency_hiding", "benchmarks_numinstructions_benchmark_numinstructions_x_operation"]
 
