@@ -118,3 +118,27 @@ def test_two_image_chain_matches_the_oracle(device, which):
         assert np.all(got[:, out_row:] == 0xA5)
         got = np.ascontiguousarray(got[:, :out_row]).view(out_dtype).reshape(want.shape)
         assert _same_with_any_nan(got, want), (which, seed)
+
+
+@pytest.mark.gpu
+def test_two_image_and_split_properties_at_full_size(device):
+    # 4K: (a ^ b) ^ b = a through two launches of the two-image chain; the planes SplitWrite leaves recombine to the image
+    import torch
+    h, w = 2160, 3840
+    rng = np.random.default_rng(99)
+    a = rng.integers(0, 2**32, (h, w), dtype=np.uint64).astype(np.uint32)
+    b = rng.integers(0, 2**32, (h, w), dtype=np.uint64).astype(np.uint32)
+    da, db = (torch.from_numpy(x.view(np.uint8).reshape(h, w * 4)).to(device) for x in (a, b))
+    c = torch.zeros_like(da)
+    back = torch.zeros_like(da)
+    cases.dual(5, da, db, w, h, c)
+    cases.dual(5, c, db, w, h, back)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32).reshape(h, w), a ^ b)
+    assert back.cpu().numpy().tobytes() == a.tobytes()
+    img = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    dimg = torch.from_numpy(img.reshape(h, w * 3)).to(device)
+    planes = [torch.zeros((h, w), dtype=torch.uint8, device=device) for _ in range(3)]
+    cases.split_write(0, dimg, w, h, planes)
+    torch.cuda.synchronize()
+    assert np.stack([p.cpu().numpy() for p in planes], axis=-1).tobytes() == img.tobytes()
