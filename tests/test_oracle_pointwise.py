@@ -119,3 +119,18 @@ def test_two_image_chains_equal_the_reference_backend(which):
         want = ol.ref_dual(which, a, b, pad=(0, 8))
         got = po.run_dual(which, a, b)
         assert got.dtype == want.dtype and got.tobytes() == want.tobytes(), (which, seed)
+
+
+def test_two_image_and_split_chains_equal_the_committed_reference_vectors():
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "pointwise_reference_vectors.npz"))
+    for which in sorted(po.DUAL_CASES):
+        a, b = pc.dual_inputs(which, po.DUAL_CASES, 6, 11, 0)
+        assert a.tobytes() == g[f"dual_a_{which}"].tobytes() and b.tobytes() == g[f"dual_b_{which}"].tobytes()
+        assert po.run_dual(which, a, b).tobytes() == g[f"dual_out_{which}"].tobytes(), which
+    for which in sorted(ol.SPLIT_WRITE_CASES):
+        src = _split_input(which, 24, 40, 0)
+        assert src.tobytes() == g[f"split_in_{which}"].tobytes()
+        planes = ol.oracle_split_write(which, src, (29, 17) if which == 3 else None, (0.5, -2.0, 3.25, 0))
+        for k, plane in enumerate(planes):
+            assert plane.tobytes() == g[f"split_out_{which}_{k}"].tobytes(), (which, k)
