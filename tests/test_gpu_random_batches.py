@@ -86,3 +86,70 @@ def test_random_batch_equals_the_oracle(device, seed, batch, size, pad, least, d
     assert got.shape == want.shape
     same = got.view(np.uint32) == want.view(np.uint32)
     assert same.all(), f"{(~same).sum()} of {same.size} values differ; first at {np.argwhere(~same)[0]}"
+
+
+# (seed, source w x h, pitch padding, target w x h): crop -> bilinear resize that keeps the aspect ratio (bands of the
+# background colour) -> Mul -> Sub -> SaturateCast -> packed uchar3 tensor, five planes.
+LETTERBOX = [
+    (1, (97, 61), 0, (128, 64)),
+    (2, (97, 61), 1, (31, 17)),
+    (3, (200, 40), 0, (40, 200)),
+    (4, (33, 150), 3, (64, 9)),
+    (5, (64, 64), 0, (1, 1)),
+    (6, (300, 200), 0, (260, 70)),
+    (7, (12, 7), 0, (50, 50)),
+]
+
+
+@pytest.mark.parametrize("seed,size,pad,dst", LETTERBOX)
+def test_random_letterboxed_batch_equals_the_oracle(device, seed, size, pad, dst):
+    import torch
+    rng = np.random.RandomState(2000 + seed)
+    w, h = size
+    pitch = w * 3 + pad
+    backing = torch.from_numpy(rng.randint(0, 256, (h, pitch)).astype(np.uint8)).to(device)
+    src = backing.view(h, w, 3) if pad == 0 else torch.as_strided(backing, (h, w, 3), (pitch, 3, 1))
+    host = np.ascontiguousarray(backing.cpu().numpy()[:, :w * 3].reshape(h, w, 3))
+    rects = _rects(rng, 8, w, h, 1)[[0, 1, 4, 5, 6]]
+    bg = rng.uniform(0, 255, 3).astype(np.float32)
+    mul = rng.uniform(0.25, 3.0, 3).astype(np.float32)
+    sub = rng.uniform(-50, 200, 3).astype(np.float32)
+    out = torch.full((5, dst[1], dst[0], 3), 7, dtype=torch.uint8, device=device)
+    print(f"seed {seed} source {w}x{h} pitch {pitch} target {dst[0]}x{dst[1]}", flush=True)
+    cases.crop_resize_par_u8(src, rects, dst, bg, mul, sub, out)
+    torch.cuda.synchronize()
+    want = ol.oracle_crop_resize_par_u8(host, rects, dst, bg, mul, sub)
+    got = out.cpu().numpy()
+    assert got.shape == want.shape
+    assert got.tobytes() == want.tobytes(), f"{(got != want).sum()} of {got.size} bytes differ; first at {np.argwhere(got != want)[0]}"
+
+
+# (seed, frame w x h, pitch padding, target w x h): NV12 -> RGB -> bilinear resize -> Mul -> three float planes.
+FRAMES = [
+    (1, (64, 48), 0, (37, 19)),
+    (2, (66, 50), 2, (66, 50)),
+    (3, (130, 34), 0, (65, 17)),
+    (4, (34, 130), 6, (300, 5)),
+    (5, (2, 2), 0, (9, 9)),
+    (6, (256, 128), 0, (255, 127)),
+    (7, (40, 30), 0, (1, 1)),
+]
+
+
+@pytest.mark.parametrize("seed,size,pad,dst", FRAMES)
+def test_random_nv12_frame_equals_the_oracle(device, seed, size, pad, dst):
+    import torch
+    rng = np.random.RandomState(3000 + seed)
+    w, h = size
+    backing = torch.from_numpy(rng.randint(0, 256, (h * 3 // 2, w + pad)).astype(np.uint8)).to(device)
+    frame = backing[:, :w]
+    scale = float(np.float32(rng.uniform(0.001, 2.0)))
+    out = torch.full((3, dst[1], dst[0]), float("nan"), dtype=torch.float32, device=device)
+    print(f"seed {seed} frame {w}x{h} pitch {w + pad} target {dst[0]}x{dst[1]} scale {scale}", flush=True)
+    cases.nv12_rgb_resize_split(frame, w, h, dst, scale, out)
+    torch.cuda.synchronize()
+    want = ol.oracle_nv12_rgb_resize_split(np.ascontiguousarray(frame.cpu().numpy()), w, h, dst, scale)
+    got = out.cpu().numpy()
+    assert got.shape == want.shape
+    same = got.view(np.uint32) == want.view(np.uint32)
+    assert same.all(), f"{(~same).sum()} of {same.size} values differ; first at {np.argwhere(~same)[0]}"
