@@ -1,0 +1,113 @@
+"""Seeded random cases of the three resizing chains, shared by the GPU tests (tests/test_gpu_random_batches.py), the CPU
+test that pins the oracle on them (tests/test_oracle_random_batches.py) and the script that writes the reference's
+digests of them (tests/golden/make_random_batches_golden.py).  Every function returns host arrays only."""
+import hashlib
+
+import numpy as np
+
+
+def digest(a) -> str:
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def rects(rng, n, w, h, least):
+    out = []
+    for i in range(n):
+        kind = i % 8
+        if kind == 0:
+            cw, ch = min(w, least + rng.randint(0, 3)), 1 + rng.randint(0, 3)  # a few pixels
+        elif kind == 1:
+            cw, ch = w, h                                                   # the whole image
+        elif kind == 2:
+            cw, ch = w, 1 + rng.randint(0, h)                               # full width
+        elif kind == 3:
+            cw, ch = rng.randint(least, w + 1), h                           # full height
+        else:
+            cw, ch = rng.randint(least, w + 1), 1 + rng.randint(0, h)
+        x = rng.randint(0, w - cw + 1)
+        y = rng.randint(0, h - ch + 1)
+        if kind == 4:
+            x, y = w - cw, h - ch                                           # ends in the image's last pixel
+        out.append((x, y, cw, ch))
+    return np.array(out, np.int32)
+
+
+# crop -> bilinear resize -> channel swap -> (x - mean) / std -> three float planes per crop
+# (seed, batch, source w x h, pitch padding in bytes, narrowest crop, target w x h)
+NORMALISE = [
+    (1, 8, (97, 61), 1, 2, (32, 5)),        # pitch 292
+    (2, 8, (97, 61), 0, 1, (64, 9)),        # pitch 291: rows of every alignment
+    (3, 64, (131, 77), 3, 2, (96, 7)),      # pitch 396
+    (4, 8, (40, 33), 0, 2, (224, 3)),
+    (5, 8, (97, 61), 1, 2, (17, 11)),
+    (6, 64, (131, 77), 1, 1, (50, 6)),
+    (7, 8, (300, 9), 0, 2, (130, 13)),
+    (8, 8, (9, 200), 1, 2, (33, 31)),
+    (9, 8, (64, 64), 0, 2, (1, 1)),
+    (10, 64, (257, 129), 1, 2, (160, 10)),  # pitch 772
+    (11, 8, (5, 4), 1, 1, (64, 8)),
+    (12, 8, (512, 300), 0, 2, (256, 4)),
+    (13, 8, (512, 300), 0, 2, (260, 4)),    # wider than the strip form of the kernel takes
+]
+
+
+def normalise_inputs(seed, batch, size, pad, least):
+    """backing (h, pitch) u8, rects (batch, 4), sub (3), div (3); the image is backing[:, :w*3] seen as (h, w, 3)."""
+    rng = np.random.RandomState(1000 + seed)
+    w, h = size
+    backing = rng.randint(0, 256, (h, w * 3 + pad)).astype(np.uint8)
+    r = rects(rng, batch, w, h, least)
+    sub = rng.uniform(-20, 140, 3).astype(np.float32)
+    # 58.395 takes the two-instruction division, 0.7 the five-instruction one, a denormal-range divisor the generic one
+    div = np.array([[58.395, 57.12, 57.375], [0.7, 3.0, 1e-39], [1.0, 255.0, 0.1]][seed % 3], np.float32)
+    return backing, r, sub, div
+
+
+# crop -> bilinear resize that keeps the aspect ratio (bands of the background colour) -> Mul -> Sub -> SaturateCast ->
+# packed uchar3 tensor, five planes.  (seed, source w x h, pitch padding, target w x h)
+LETTERBOX = [
+    (1, (97, 61), 0, (128, 64)),
+    (2, (97, 61), 1, (31, 17)),
+    (3, (200, 40), 0, (40, 200)),
+    (4, (33, 150), 3, (64, 9)),
+    (5, (64, 64), 0, (1, 1)),
+    (6, (300, 200), 0, (260, 70)),
+    (7, (12, 7), 0, (50, 50)),
+]
+
+
+def letterbox_inputs(seed, size, pad):
+    rng = np.random.RandomState(2000 + seed)
+    w, h = size
+    backing = rng.randint(0, 256, (h, w * 3 + pad)).astype(np.uint8)
+    r = rects(rng, 8, w, h, 1)[[0, 1, 4, 5, 6]]
+    bg = rng.uniform(0, 255, 3).astype(np.float32)
+    mul = rng.uniform(0.25, 3.0, 3).astype(np.float32)
+    sub = rng.uniform(-50, 200, 3).astype(np.float32)
+    return backing, r, bg, mul, sub
+
+
+# NV12 -> RGB -> bilinear resize -> Mul -> three float planes.  (seed, frame w x h, pitch padding, target w x h)
+FRAMES = [
+    (1, (64, 48), 0, (37, 19)),
+    (2, (66, 50), 2, (66, 50)),
+    (3, (130, 34), 0, (65, 17)),
+    (4, (34, 130), 6, (300, 5)),
+    (5, (2, 2), 0, (9, 9)),
+    (6, (256, 128), 0, (255, 127)),
+    (7, (40, 30), 0, (1, 1)),
+]
+
+
+def frame_inputs(seed, size, pad):
+    rng = np.random.RandomState(3000 + seed)
+    w, h = size
+    backing = rng.randint(0, 256, (h * 3 // 2, w + pad)).astype(np.uint8)
+    scale = float(np.float32(rng.uniform(0.001, 2.0)))
+    return backing, scale
+
+
+def image_of(backing, w):
+    """The (h, w, 3) image at the start of every row of `backing`, as a view with the backing's pitch."""
+    h, pitch = backing.shape
+    return np.lib.stride_tricks.as_strided(backing, (h, w, 3), (pitch, 3, 1), writeable=False)

@@ -1,0 +1,50 @@
+"""The oracle on the seeded random cases of tests/random_cases.py: equal, bit for bit, to the digests the reference CPU
+backend gave (tests/golden/random_batches_reference_digests.json) and, where the reference backend is built, to its
+live output."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+import random_cases as rc
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "random_batches_reference_digests.json")) as f:
+    REFERENCE = json.load(f)
+
+
+def _check(key, want, live):
+    assert rc.digest(want) == REFERENCE[key], key
+    if ol.have_ref():
+        got = live()
+        assert got.tobytes() == want.tobytes(), key
+
+
+@pytest.mark.parametrize("seed,batch,size,pad,least,dst", rc.NORMALISE)
+def test_oracle_on_random_batches(seed, batch, size, pad, least, dst):
+    backing, rects, sub, div = rc.normalise_inputs(seed, batch, size, pad, least)
+    img = rc.image_of(backing, size[0])
+    want = ol.oracle_crop_resize_norm_split(np.ascontiguousarray(img), rects, dst, sub, div)
+    _check(f"normalise:{seed}", want, lambda: ol.ref_crop_resize_norm_split(img, rects, dst, sub, div))
+
+
+@pytest.mark.parametrize("seed,size,pad,dst", rc.LETTERBOX)
+def test_oracle_on_random_letterboxed_batches(seed, size, pad, dst):
+    backing, rects, bg, mul, sub = rc.letterbox_inputs(seed, size, pad)
+    img = rc.image_of(backing, size[0])
+    want = ol.oracle_crop_resize_par_u8(np.ascontiguousarray(img), rects, dst, bg, mul, sub)
+    _check(f"letterbox:{seed}", want, lambda: ol.ref_crop_resize_par_u8(img, rects, dst, bg, mul, sub))
+
+
+@pytest.mark.parametrize("seed,size,pad,dst", rc.FRAMES)
+def test_oracle_on_random_nv12_frames(seed, size, pad, dst):
+    backing, scale = rc.frame_inputs(seed, size, pad)
+    w, h = size
+    want = ol.oracle_nv12_rgb_resize_split(np.ascontiguousarray(backing[:, :w]), w, h, dst, scale)
+    _check(f"frame:{seed}", want, lambda: ol.ref_nv12_rgb_resize_split(backing[:, :w], w, h, dst, scale))
+
+
+def test_every_case_has_a_reference_digest():
+    keys = {f"normalise:{c[0]}" for c in rc.NORMALISE} | {f"letterbox:{c[0]}" for c in rc.LETTERBOX} | {f"frame:{c[0]}" for c in rc.FRAMES}
+    assert keys == set(REFERENCE)
