@@ -47,6 +47,9 @@ def parse():
                     help="run the stand-alone instruction-issue measurement (fusedkernellibrary_amd/probe_issue_rate) and exit")
     ap.add_argument("--uchar3-access", action="store_true",
                     help="run the stand-alone comparison of access forms for uchar3 rows (fusedkernellibrary_amd/probe_uchar3_rows) and exit")
+    ap.add_argument("--rows-sweep", action="store_true",
+                    help="time configuration 3's chain for 8 to 448 output rows per plane (224 wide, the same 64 crops), print one "
+                         "line per height and the straight line through the heights that fill the GPU, and exit")
     ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
@@ -140,6 +143,24 @@ def main():
     src3 = torch.from_numpy(c3["src"]).to(dev)
     out3 = torch.zeros((64, 3, 224, 224), dtype=torch.float32, device=dev)
     f3 = lambda: cases.crop_resize_norm_split(src3, c3["rects"], c3["dst"], c3["sub"], c3["div"], out3)
+    if args.rows_sweep:
+        heights = (8, 56, 112, 168, 224, 336, 448, 672, 896)
+        best = {}
+        for _ in range(3):
+            for hh in heights:
+                o = torch.zeros((64, 3, hh, 224), dtype=torch.float32, device=dev)
+                us = timer.run(lambda: cases.crop_resize_norm_split(src3, c3["rects"], (224, hh), c3["sub"], c3["div"], o),
+                               args.steps, args.warmup)[1] * 1e3
+                best[hh] = min(best.get(hh, 1e9), us)
+                del o
+        for hh in heights:
+            print(f"rows per plane {hh:4d}   workgroups {64 * ((hh + 7) // 8):5d}   output {64 * 3 * hh * 224 * 4 / 1e6:7.2f} MB   "
+                  f"{best[hh]:7.2f} us per launch")
+        hs = np.array([hh for hh in heights if hh % 224 == 0], dtype=np.float64)   # whole rounds of 7 workgroups per compute unit
+        slope, fixed = np.polyfit(hs, np.array([best[int(hh)] for hh in hs]), 1)
+        print(f"through the heights that are whole multiples of 224: {fixed:.2f} us + {slope * 224:.2f} us per 224 rows "
+              f"(38.54 MB of output: {64 * 3 * 224 * 224 * 4 / (slope * 224 * 1e-6) / 1e12:.2f} TB/s)")
+        return
     # (timed after the other configurations, further down: the first launches of a process run on a GPU that has not
     # reached its working clocks yet, and the headline should not depend on what happened to be measured first)
 
@@ -248,6 +269,16 @@ def main():
     # (the second of two such batches: the first also pays for the launch queue's and the runtime's argument buffers growing)
     timer.run(f3, 1000, 300, settle=0)
     r3["kernel_us_1000_launches"] = timer.run(f3, 1000, 0, settle=0)[1] * 1e3
+    # the same 64 crops to planes of twice the rows (224 x 448): what a launch costs that does not depend on its size, and what
+    # 38.5 MB more of output cost once the kernel runs (the source bytes are the same, so they count for nothing here)
+    out3x2 = torch.zeros((64, 3, 448, 224), dtype=torch.float32, device=dev)
+    f3x2 = lambda: cases.crop_resize_norm_split(src3, c3["rects"], (224, 448), c3["sub"], c3["div"], out3x2)
+    twice = min(timer.run(f3x2, args.steps, args.warmup)[1] * 1e3 for _ in range(3))
+    once = min(again)
+    r3["twice_the_rows"] = {"kernel_us": twice, "marginal_us": twice - once, "fixed_us": 2 * once - twice,
+                            "marginal_gbs": 64 * 3 * 224 * 224 * 4 / ((twice - once) * 1e-6) / 1e9,
+                            "marginal_frac": 64 * 3 * 224 * 224 * 4 / ((twice - once) * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    del out3x2
 
     if args.list_compiled:
         # kernel symbol of every chain compiled at run time ("fkd_jit_" + FNV-1a of the signature), for reading profiles
@@ -296,7 +327,8 @@ def main():
                      "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"],
                      "kernel_us_5_runs_min_mean_max": r3["kernel_us_5_runs_min_mean_max"],
                      "kernel_us_1000_launches": r3["kernel_us_1000_launches"],
-                     "frac_1000_launches": a3 / (r3["kernel_us_1000_launches"] * 1e-6) / 1e9 / HBM_PEAK_GBS},
+                     "frac_1000_launches": a3 / (r3["kernel_us_1000_launches"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                     "twice_the_rows": r3["twice_the_rows"]},
         "cpu_baseline": cpu,
         "others": {k: v for k, v in results.items() if k != "c3"},
     }
