@@ -1,10 +1,10 @@
 // CircularTensor: a Tensor of BATCH planes that always shows the last BATCH images handed to update(), newest first
 // or oldest first, the temporal window of a video pipeline.  update() runs the caller's chain (read ... write) on the
 // new image and shifts the others by one plane in ONE launch: a DivergentBatchTransformDPP of two sequences, the
-// caller's chain with a store into a hidden circular copy put before its write, and a copy of the other BATCH - 1
-// planes out of that hidden copy.
+// caller's chain with a store into a hidden ring of BATCH planes put before its write, and a copy of the other
+// BATCH - 1 planes out of that ring.
 // Interface counterpart: FK/core/data/circular_tensor.h:24-168.  With ColorPlanes::Transposed the window is a TensorT
-// (all first channel planes, then all second ones, ...) and the chain must end in Write<TensorTSplit<StoreT>>.
+// (all first channel planes, then all second ones, ...) and the chain must end in Write<TensorTSplit<...>>.
 #ifndef FK_AMD_CIRCULAR_TENSOR_H
 #define FK_AMD_CIRCULAR_TENSOR_H
 
@@ -14,96 +14,91 @@
 #include <fused_kernel/algorithms/basic_ops/memory_operations.h>
 
 #include <stdexcept>
+#include <type_traits>
 
 namespace fk {
 
 enum class CircularTensorOrder { NewestFirst, OldestFirst };
-
-// Which sequence of update() a plane belongs to: 0 the caller's chain (the newest image), 1 the copy.
-template <CircularTensorOrder CTO, int BATCH> struct SequenceSelectorType {
-    static constexpr uint at(const uint& index) {
-        if constexpr (CTO == CircularTensorOrder::NewestFirst) return index > 0 ? 1u : 0u;
-        else return index != BATCH - 1 ? 1u : 0u;
-    }
-};
-
-template <CircularTensorOrder CT_ORDER> struct CTReadDirection;
-template <> struct CTReadDirection<CircularTensorOrder::NewestFirst> { static constexpr CircularDirection dir{CircularDirection::Descendent}; };
-template <> struct CTReadDirection<CircularTensorOrder::OldestFirst> { static constexpr CircularDirection dir{CircularDirection::Ascendent}; };
-template <CircularTensorOrder CT_ORDER> static constexpr CircularDirection CTReadDirection_v = CTReadDirection<CT_ORDER>::dir;
-
 enum class ColorPlanes { Standard, Transposed };
 
-template <typename T, ColorPlanes CP_MODE> struct CoreType;
-template <typename T> struct CoreType<T, ColorPlanes::Standard> { using type = Tensor<T>; };
-template <typename T> struct CoreType<T, ColorPlanes::Transposed> { using type = TensorT<T>; };
-template <typename T, ColorPlanes CP_MODE> using CoreType_t = typename CoreType<T, CP_MODE>::type;
+namespace amd {
 
-template <typename T, int COLOR_PLANES, typename Enabler = void> struct CircularTensorStoreType {};
-template <typename T, int COLOR_PLANES> struct CircularTensorStoreType<T, COLOR_PLANES, std::enable_if_t<std::is_aggregate_v<T> && COLOR_PLANES == 1>> {
-    using type = T;
-};
-template <typename T, int COLOR_PLANES> struct CircularTensorStoreType<T, COLOR_PLANES, std::enable_if_t<!std::is_aggregate_v<T> && (COLOR_PLANES > 1)>> {
-    using type = VectorType_t<T, COLOR_PLANES>;
+// The reader that fetches back, element for element, what a tensor writer stored.
+template <typename Writer> struct StoredBy;
+template <typename E> struct StoredBy<TensorWrite<E>> { using Reader = TensorRead<E>; };
+template <typename E> struct StoredBy<TensorSplit<E>> { using Reader = TensorPack<E>; };
+template <typename E> struct StoredBy<TensorTSplit<E>> { using Reader = TensorTPack<E>; };
+
+template <typename T, int N> struct LazyVector { using type = VectorType_t<T, N>; };
+
+// Everything the template arguments of a CircularTensor decide.
+template <typename T, int CHANNELS, int BATCH, CircularTensorOrder ORDER, ColorPlanes LAYOUT> struct WindowTraits {
+    // an element of the window: T itself when T already is a pixel in one plane, CHANNELS values of T otherwise
+    static constexpr bool kPixelInOnePlane = std::is_aggregate_v<T> && CHANNELS == 1;
+    static_assert(kPixelInOnePlane || (!std::is_aggregate_v<T> && CHANNELS > 1),
+                  "CircularTensor<T, COLOR_PLANES, ...>: either a vector T in one plane or a scalar T in several");
+    using Element = typename std::conditional_t<kPixelInOnePlane, std::type_identity<T>, LazyVector<T, CHANNELS>>::type;
+    using Window = std::conditional_t<LAYOUT == ColorPlanes::Transposed, TensorT<T>, Tensor<T>>;
+
+    static constexpr uint kNewestPlane = ORDER == CircularTensorOrder::NewestFirst ? 0u : uint(BATCH) - 1u;
+    // the ring is filled upwards; showing the newest image first means walking it downwards
+    static constexpr CircularDirection kWalk =
+        ORDER == CircularTensorOrder::NewestFirst ? CircularDirection::Descendent : CircularDirection::Ascendent;
+    // plane of the launch -> sequence: the caller's chain (0) for the plane that shows the newest image, the copy (1) elsewhere
+    struct PlaneToSequence {
+        static constexpr uint at(const uint& plane) { return plane == kNewestPlane ? 0u : 1u; }
+    };
+    template <typename WriteIOp> static constexpr bool accepts() {
+        if constexpr (LAYOUT == ColorPlanes::Transposed) return std::is_same_v<WriteIOp, Write<TensorTSplit<Element>>>;
+        else return std::is_same_v<WriteIOp, Write<TensorWrite<Element>>> || std::is_same_v<WriteIOp, Write<TensorSplit<Element>>>;
+    }
 };
 
-template <typename T, int COLOR_PLANES, int BATCH, CircularTensorOrder CT_ORDER, ColorPlanes CP_MODE> class CircularTensor : public CoreType_t<T, CP_MODE> {
-    using ParentType = CoreType_t<T, CP_MODE>;
-    using StoreT = typename CircularTensorStoreType<T, COLOR_PLANES>::type;
-    using WriteInstantiableOperations = TypeList<Write<TensorWrite<StoreT>>, Write<TensorSplit<StoreT>>, Write<TensorTSplit<StoreT>>>;
-    using ReadInstantiableOperations = TypeList<Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorRead<StoreT>, BATCH>>,
-                                                Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorPack<StoreT>, BATCH>>,
-                                                Read<CircularTensorRead<CTReadDirection_v<CT_ORDER>, TensorTPack<StoreT>, BATCH>>>;
+} // namespace amd
+
+template <typename T, int COLOR_PLANES, int BATCH, CircularTensorOrder CT_ORDER, ColorPlanes CP_MODE>
+class CircularTensor : public amd::WindowTraits<T, COLOR_PLANES, BATCH, CT_ORDER, CP_MODE>::Window {
+    using Traits = amd::WindowTraits<T, COLOR_PLANES, BATCH, CT_ORDER, CP_MODE>;
+    using Window = typename Traits::Window;
 
 public:
-    CircularTensor() {}
-    CircularTensor(const uint& width_, const uint& height_, const MemType& type_ = defaultMemType, const int& deviceID_ = 0)
-        : ParentType(width_, height_, BATCH, COLOR_PLANES, type_, deviceID_), m_tempTensor(width_, height_, BATCH, COLOR_PLANES, type_, deviceID_) {}
+    CircularTensor() = default;
+    CircularTensor(const uint& width, const uint& height, const MemType& mem = defaultMemType, const int& device = 0)
+        : Window(width, height, BATCH, COLOR_PLANES, mem, device), ring_(width, height, BATCH, COLOR_PLANES, mem, device) {}
 
-    void Alloc(const uint& width_, const uint& height_, const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
-        this->allocTensor(width_, height_, BATCH, COLOR_PLANES, type_, deviceID_);
-        m_tempTensor.allocTensor(width_, height_, BATCH, COLOR_PLANES, type_, deviceID_);
+    void Alloc(const uint& width, const uint& height, const MemType& mem = defaultMemType, const int& device = 0) {
+        this->allocTensor(width, height, BATCH, COLOR_PLANES, mem, device);
+        ring_.allocTensor(width, height, BATCH, COLOR_PLANES, mem, device);
     }
 
-    // The IOps are a complete chain whose write is TensorWrite<StoreT> or TensorSplit<StoreT> on this tensor's ptr().
-    template <ParArch PA, typename... IOpTypes> void update(Stream_<PA>& stream, const IOpTypes&... instantiableOperationInstances) {
-        const auto writeInstantiableOperation = ppLast(instantiableOperationInstances...);
-        using writeDFType = std::decay_t<decltype(writeInstantiableOperation)>;
-        using writeOpType = typename writeDFType::Operation;
-        if constexpr (CP_MODE == ColorPlanes::Transposed) {
-            static_assert(std::is_same_v<writeDFType, Write<TensorTSplit<StoreT>>>,
-                          "Need to use TensorTSplitWrite as write function because you are using a transposed CircularTensor (CP_MODE = Transposed)");
-        } else {
-            static_assert(one_of_v<writeDFType, TypeList<Write<TensorWrite<StoreT>>, Write<TensorSplit<StoreT>>>>,
-                          "the chain given to CircularTensor::update must end in Write<TensorWrite<StoreT>> or Write<TensorSplit<StoreT>>");
-        }
-        using equivalentReadDFType = EquivalentType_t<writeDFType, WriteInstantiableOperations, ReadInstantiableOperations>;
+    // `chain` is a complete chain (read ... write) whose write stores one image into this tensor's ptr().
+    template <ParArch PA, typename... IOps> void update(Stream_<PA>& stream, const IOps&... chain) {
+        using WriteIOp = std::decay_t<decltype(ppLast(chain...))>;
+        static_assert(Traits::template accepts<WriteIOp>(),
+                      "the chain given to CircularTensor::update must end in Write<TensorWrite<E>> or Write<TensorSplit<E>> "
+                      "(ColorPlanes::Standard) or in Write<TensorTSplit<E>> (ColorPlanes::Transposed), E being the window's element");
+        using Writer = typename WriteIOp::Operation;
+        if (PA == ParArch::GPU_AMD && this->getMemType() != MemType::Device && this->getMemType() != MemType::DeviceAndPinned)
+            throw std::runtime_error("CircularTensor::update on the GPU needs a window in MemType::Device or MemType::DeviceAndPinned");
 
-        // The launch's planes are the planes of both sequences together: one for the new image, BATCH - 1 copied.
-        constexpr uint COPY_PLANES = static_cast<uint>(BATCH) - 1u;
+        // sequence 0: the caller's chain; its result also goes into slot head_ of the ring, just before its own write
+        MidWrite<CircularTensorWrite<CircularDirection::Ascendent, Writer, BATCH>> keep;
+        keep.params.first = head_;
+        keep.params.opData.params = ring_.ptr();
+        // sequence 1: the other BATCH - 1 images, read back out of the ring in the window's order, through the same write
+        Read<CircularTensorRead<Traits::kWalk, typename amd::StoredBy<Writer>::Reader, BATCH>> others;
+        others.params.first = head_;
+        others.params.opData.params = ring_.ptr();
+        others.params.opData.params.dims.planes = uint(BATCH) - 1u;
 
-        MidWrite<CircularTensorWrite<CircularDirection::Ascendent, writeOpType, BATCH>> updateWriteToTemp;
-        updateWriteToTemp.params.first = m_nextUpdateIdx;
-        updateWriteToTemp.params.opData.params = m_tempTensor.ptr();
-        const auto updateOps = buildOperationSequence_tup(insert_before_last(updateWriteToTemp, instantiableOperationInstances...));
-
-        equivalentReadDFType nonUpdateRead;
-        nonUpdateRead.params.first = m_nextUpdateIdx;
-        nonUpdateRead.params.opData.params = m_tempTensor.ptr();
-        nonUpdateRead.params.opData.params.dims.planes = COPY_PLANES;
-        const auto copyOps = buildOperationSequence(nonUpdateRead, writeInstantiableOperation);
-
-        if (PA == ParArch::GPU_AMD && !(this->getMemType() == MemType::Device || this->getMemType() == MemType::DeviceAndPinned)) {
-            throw std::runtime_error("CircularTensor operations on Device memory only supported "
-                                     "if the CircularTensor is MemType::Device or MemType::DeviceAndPinned");
-        }
-        Executor<DivergentBatchTransformDPP<PA, SequenceSelectorType<CT_ORDER, BATCH>>>::executeOperations(stream, updateOps, copyOps);
-        m_nextUpdateIdx = (m_nextUpdateIdx + 1) % BATCH;
+        Executor<DivergentBatchTransformDPP<PA, typename Traits::PlaneToSequence>>::executeOperations(
+            stream, buildOperationSequence_tup(insert_before_last(keep, chain...)), buildOperationSequence(others, ppLast(chain...)));
+        head_ = (head_ + 1) % BATCH;
     }
 
 private:
-    CoreType_t<T, CP_MODE> m_tempTensor;
-    int m_nextUpdateIdx{0};
+    Window ring_;     // every image ever stored, slot head_ next
+    int head_{0};
 };
 
 } // namespace fk

@@ -158,7 +158,7 @@ void fklo_yuv2rgb_709_full(const uint8_t yuv[3], float rgb[3]);
 float fklo_bilinear(float p00, float p10, float p01, float p11, float sx, float sy);
 
 /* Circular-buffer plane of logical plane z (computeCircularThreadIdx, FK/algorithms/basic_ops/memory_operations.h:422-432):
- * direction 0 Ascendent, 1 Descendent.  Sequence of CircularTensor::update that owns plane z (SequenceSelectorType::at,
+ * direction 0 Ascendent, 1 Descendent.  Sequence of CircularTensor::update that owns plane z (the selector of CircularTensor::update,
  * FK/core/data/circular_tensor.h:26-35): 0 the caller's chain, 1 the copy; order 0 NewestFirst, 1 OldestFirst. */
 int32_t fklo_circular_plane(int32_t direction, int32_t batch, int32_t z, int32_t first);
 int32_t fklo_window_sequence(int32_t order, int32_t batch, int32_t z);
