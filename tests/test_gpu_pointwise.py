@@ -45,6 +45,22 @@ def test_operation_matches_the_oracle(device, which):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("which", [9, 6, 4, 14, 23, 13])
+def test_widths_around_a_wave_of_runs(device, which):
+    # A wave moves 256 elements of a row (64 lanes x 4).  Waves that lie wholly inside a row take the dense form of the
+    # accesses for 32- to 64-byte runs, the wave at the row's end and rows narrower than a wave the per-lane form; odd
+    # heights leave the last thread row half used; padded pitches of byte images put rows on odd addresses.
+    in_dtype, _, out_dtype = po.CASES[which]
+    wide = np.dtype(in_dtype).itemsize > 1 or np.dtype(out_dtype).itemsize > 1
+    for seed, (w, h, pad) in enumerate(((255, 5, 0), (256, 4, 0), (257, 3, 1), (260, 5, 0), (511, 2, 3), (512, 5, 0), (515, 1, 0),
+                                        (768, 3, 2), (1021, 5, 0), (1024, 2, 0), (1283, 3, 0))):
+        src = pc.inputs(which, po.CASES, h, w, 40 + seed)
+        want = po.run(which, src, pc.constants(which), pc.MATRIX)
+        got = run_on_gpu(device, which, src, pad * (4 if wide else 1), pad * (4 if wide else 1))
+        assert pc.same(which, got, want, po.INEXACT), (which, w, h, pad)
+
+
+@pytest.mark.gpu
 def test_full_size_properties(device):
     # 4K: Abs is idempotent, Max then Min with the same constants clamps, x ^ c ^ c = x, (x << 5) >> 5 keeps the low bits
     h, w = 2160, 3840
