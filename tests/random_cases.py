@@ -15,7 +15,7 @@ def rects(rng, n, w, h, least):
     for i in range(n):
         kind = i % 8
         if kind == 0:
-            cw, ch = min(w, least + rng.randint(0, 3)), 1 + rng.randint(0, 3)  # a few pixels
+            cw, ch = min(w, least + rng.randint(0, 3)), min(h, 1 + rng.randint(0, 3))  # a few pixels
         elif kind == 1:
             cw, ch = w, h                                                   # the whole image
         elif kind == 2:
@@ -111,3 +111,35 @@ def image_of(backing, w):
     """The (h, w, 3) image at the start of every row of `backing`, as a view with the backing's pitch."""
     h, pitch = backing.shape
     return np.lib.stride_tricks.as_strided(backing, (h, w, 3), (pitch, 3, 1), writeable=False)
+
+
+def sweep_case(i):
+    """Case i of an open-ended seeded sweep over the three chains: (family, arguments) with family 0 normalise (batch 8),
+    1 letterbox, 2 NV12 frame; sizes from one or two pixels to a few hundred, pitches of every alignment, target sizes
+    that take either form of the bilinear kernel, whole and fractional factors, divisors of every division sequence."""
+    rng = np.random.RandomState(50000 + i)
+    w, h = int(rng.randint(2, 400)), int(rng.randint(1, 300))
+    pad = int(rng.choice([0, 0, 1, 2, 3, 4]))
+    family = i % 3
+    if family == 0:
+        dst = (int(rng.choice([rng.randint(1, 300), 32 * rng.randint(1, 9), 224])), int(rng.randint(1, 40)))
+        backing = rng.randint(0, 256, (h, w * 3 + pad)).astype(np.uint8)
+        r = rects(rng, 8, w, h, min(int(rng.choice([1, 2])), w))
+        sub = rng.uniform(-20, 140, 3).astype(np.float32)
+        div = rng.choice([58.395, 57.12, 57.375, 0.7, 3.0, 1.0, 255.0, 0.1, 1e-39, 7.0, 1.5e10], 3).astype(np.float32)
+        return family, dict(backing=backing, w=w, rects=r, dst=dst, sub=sub, div=div)
+    if family == 1:
+        dst = (int(rng.randint(1, 300)), int(rng.randint(1, 80)))
+        backing = rng.randint(0, 256, (h, w * 3 + pad)).astype(np.uint8)
+        r = rects(rng, 8, w, h, 1)[[0, 1, 4, 5, 6]]
+        bg = rng.uniform(0, 255, 3).astype(np.float32)
+        mul = rng.uniform(0.25, 3.0, 3).astype(np.float32)
+        sub = rng.uniform(-50, 200, 3).astype(np.float32)
+        return family, dict(backing=backing, w=w, rects=r, dst=dst, bg=bg, mul=mul, sub=sub)
+    w, h = 2 * int(rng.randint(1, 200)), 2 * int(rng.randint(1, 120))
+    pad = 2 * int(rng.randint(0, 4))
+    k = int(rng.choice([0, 1, 2, 3]))
+    dst = (w // k, h // k) if k in (1, 2) else (int(rng.randint(1, 300)), int(rng.randint(1, 100)))
+    backing = rng.randint(0, 256, (h * 3 // 2, w + pad)).astype(np.uint8)
+    scale = float(np.float32(rng.uniform(0.001, 2.0)))
+    return family, dict(backing=backing, w=w, h=h, dst=dst, scale=scale)

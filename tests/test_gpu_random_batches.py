@@ -84,3 +84,30 @@ def test_random_nv12_frame_equals_the_oracle(device, seed, size, pad, dst):
     torch.cuda.synchronize()
     want = ol.oracle_nv12_rgb_resize_split(np.ascontiguousarray(backing[:, :w]), w, h, dst, scale)
     _same_bits(out.cpu().numpy(), want, f"frame:{seed}")
+
+
+def test_sweep_of_random_cases_equals_the_oracle(device):
+    # 1 500 cases of random_cases.sweep_case, a few seconds; the first differing case is named
+    import torch
+    kernels = set()
+    for i in range(1500):
+        family, c = rc.sweep_case(i)
+        backing, w, dst = c["backing"], c["w"], c["dst"]
+        if family == 0:
+            out = torch.full((8, 3, dst[1], dst[0]), float("nan"), dtype=torch.float32, device=device)
+            cases.crop_resize_norm_split(_image_on(device, backing, w), c["rects"], dst, c["sub"], c["div"], out)
+            want = ol.oracle_crop_resize_norm_split(np.ascontiguousarray(rc.image_of(backing, w)), c["rects"], dst, c["sub"], c["div"])
+        elif family == 1:
+            out = torch.full((5, dst[1], dst[0], 3), 7, dtype=torch.uint8, device=device)
+            cases.crop_resize_par_u8(_image_on(device, backing, w), c["rects"], dst, c["bg"], c["mul"], c["sub"], out)
+            want = ol.oracle_crop_resize_par_u8(np.ascontiguousarray(rc.image_of(backing, w)), c["rects"], dst, c["bg"], c["mul"], c["sub"])
+        else:
+            out = torch.full((3, dst[1], dst[0]), float("nan"), dtype=torch.float32, device=device)
+            cases.nv12_rgb_resize_split(torch.from_numpy(backing).to(device)[:, :w], w, c["h"], dst, c["scale"], out)
+            want = ol.oracle_nv12_rgb_resize_split(np.ascontiguousarray(backing[:, :w]), w, c["h"], dst, c["scale"])
+        torch.cuda.synchronize()
+        kernels.add((family, last_launch()["kernel"]))
+        got = out.cpu().numpy()
+        assert got.shape == want.shape and got.tobytes() == want.tobytes(), \
+            f"case {i} (family {family}, source {backing.shape}, target {dst}, kernel {last_launch()['kernel']}) differs from the oracle"
+    assert {(0, "strip"), (0, "gather"), (1, "gather"), (2, "gather")} <= kernels

@@ -48,3 +48,24 @@ def test_oracle_on_random_nv12_frames(seed, size, pad, dst):
 def test_every_case_has_a_reference_digest():
     keys = {f"normalise:{c[0]}" for c in rc.NORMALISE} | {f"letterbox:{c[0]}" for c in rc.LETTERBOX} | {f"frame:{c[0]}" for c in rc.FRAMES}
     assert keys == set(REFERENCE)
+
+
+def test_oracle_equals_the_reference_backend_on_the_sweep():
+    # the 1 500 cases of the sweep the GPU test runs, against the live reference CPU backend
+    if not ol.have_ref():
+        pytest.skip("the reference CPU backend is not built here")
+    for i in range(1500):
+        family, c = rc.sweep_case(i)
+        backing, w, dst = c["backing"], c["w"], c["dst"]
+        if family == 0:
+            img = rc.image_of(backing, w)
+            want = ol.oracle_crop_resize_norm_split(np.ascontiguousarray(img), c["rects"], dst, c["sub"], c["div"])
+            got = ol.ref_crop_resize_norm_split(img, c["rects"], dst, c["sub"], c["div"])
+        elif family == 1:
+            img = rc.image_of(backing, w)
+            want = ol.oracle_crop_resize_par_u8(np.ascontiguousarray(img), c["rects"], dst, c["bg"], c["mul"], c["sub"])
+            got = ol.ref_crop_resize_par_u8(img, c["rects"], dst, c["bg"], c["mul"], c["sub"])
+        else:
+            want = ol.oracle_nv12_rgb_resize_split(np.ascontiguousarray(backing[:, :w]), w, c["h"], dst, c["scale"])
+            got = ol.ref_nv12_rgb_resize_split(backing[:, :w], w, c["h"], dst, c["scale"])
+        assert got.tobytes() == want.tobytes(), f"case {i} (family {family})"
