@@ -143,3 +143,37 @@ def sweep_case(i):
     backing = rng.randint(0, 256, (h * 3 // 2, w + pad)).astype(np.uint8)
     scale = float(np.float32(rng.uniform(0.001, 2.0)))
     return family, dict(backing=backing, w=w, h=h, dst=dst, scale=scale)
+
+
+def reader_sweep_case(i):
+    """Case i of a seeded sweep over the read-back operations either side of the path: family 0 Warping of a uchar3 image,
+    1 Warping of a float image (affine or perspective, rotation by any angle, scale 0.3 to 3, shifts that move part of the
+    target outside the source), 2 Deinterlace of a uchar3 image (all three modes), 3 BorderReader under a Crop that leaves
+    the image by up to three image sizes (all five border types, uchar3 or float)."""
+    import math
+    rng = np.random.RandomState(70000 + i)
+    family = i % 4
+    w, h = int(rng.randint(2, 300)), int(rng.randint(2, 200))
+    if family < 2:
+        perspective = bool(rng.randint(0, 2))
+        angle, s = rng.uniform(-math.pi, math.pi), rng.uniform(0.3, 3.0)
+        m = [[s * math.cos(angle), -s * math.sin(angle), rng.uniform(-50, 50)], [s * math.sin(angle), s * math.cos(angle), rng.uniform(-50, 50)]]
+        if perspective:
+            m.append([rng.uniform(-1e-3, 1e-3), rng.uniform(-1e-3, 1e-3), 1.0])
+        dst = (int(rng.randint(1, 300)), int(rng.randint(1, 120)))
+        if family == 0:
+            img = rng.randint(0, 256, (h, w, 3)).astype(np.uint8)
+        else:
+            img = (rng.random_sample((h, w)) * 200 - 100).astype(np.float32)
+        return family, dict(img=img, matrix=m, perspective=perspective, dst=dst)
+    if family == 2:
+        mode = int(rng.randint(1, 4))
+        return family, dict(img=rng.randint(0, 256, (h, w, 3)).astype(np.uint8), mode=mode)
+    border = int(rng.randint(0, 5))
+    left, top = int(rng.randint(-w // 2, 3 * w)), int(rng.randint(-h // 2, 3 * h))
+    out_w, out_h = int(rng.randint(1, 400)), int(rng.randint(1, 150))
+    if rng.randint(0, 2):
+        img, value = rng.randint(0, 256, (h, w, 3)).astype(np.uint8), (9, 8, 7)
+    else:
+        img, value = (rng.random_sample((h, w)) * 100 - 50).astype(np.float32), (-1.5,)
+    return family, dict(img=img, border=border, left=left, top=top, out_w=out_w, out_h=out_h, value=value)

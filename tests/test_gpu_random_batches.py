@@ -111,3 +111,34 @@ def test_sweep_of_random_cases_equals_the_oracle(device):
         assert got.shape == want.shape and got.tobytes() == want.tobytes(), \
             f"case {i} (family {family}, source {backing.shape}, target {dst}, kernel {last_launch()['kernel']}) differs from the oracle"
     assert {(0, "strip"), (0, "gather"), (1, "gather"), (2, "gather")} <= kernels
+
+
+BORDERS = [ol.BORDER_CONSTANT, ol.BORDER_REPLICATE, ol.BORDER_REFLECT, ol.BORDER_WRAP, ol.BORDER_REFLECT_101]
+
+
+def test_sweep_of_random_reader_cases_equals_the_oracle(device):
+    # 1 000 cases of random_cases.reader_sweep_case: Warping, Deinterlace, BorderReader (reference warping.h:42-96,
+    # deinterlace.h, border_reader.h:177-327)
+    import torch
+    for i in range(1000):
+        family, c = rc.reader_sweep_case(i)
+        img = c["img"]
+        src = torch.from_numpy(img).to(device)
+        if family < 2:
+            dst = c["dst"]
+            out = torch.full((dst[1], dst[0], 3) if family == 0 else (dst[1], dst[0]), -1.0, dtype=torch.float32, device=device)
+            cases.warp(src, c["matrix"], c["perspective"], dst, out)
+            want = ol.oracle_warp(img, 3 if family == 0 else 1, c["matrix"], dst, c["perspective"])
+        elif family == 2:
+            out = torch.full(img.shape, -1.0, dtype=torch.float32, device=device)
+            cases.deinterlace(src, c["mode"], out)
+            want = ol.oracle_deinterlace(img, 3, c["mode"])
+        else:
+            shape = (c["out_h"], c["out_w"], 3) if img.ndim == 3 else (c["out_h"], c["out_w"])
+            out = torch.zeros(shape, dtype=torch.uint8 if img.dtype == np.uint8 else torch.float32, device=device)
+            cases.pad(src, BORDERS[c["border"]], c["left"], c["top"], out, value=c["value"])
+            want = ol.oracle_pad(img, BORDERS[c["border"]], c["left"], c["top"], c["out_w"], c["out_h"], value=c["value"])
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert got.shape == want.shape and got.tobytes() == want.tobytes(), \
+            f"case {i} (family {family}, source {img.shape}) differs from the oracle: " + str({k: v for k, v in c.items() if k != "img"})

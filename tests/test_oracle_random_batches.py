@@ -69,3 +69,29 @@ def test_oracle_equals_the_reference_backend_on_the_sweep():
             want = ol.oracle_nv12_rgb_resize_split(np.ascontiguousarray(backing[:, :w]), w, c["h"], dst, c["scale"])
             got = ol.ref_nv12_rgb_resize_split(backing[:, :w], w, c["h"], dst, c["scale"])
         assert got.tobytes() == want.tobytes(), f"case {i} (family {family})"
+
+
+def test_oracle_equals_the_reference_backend_on_the_reader_sweep():
+    # the cases of the reader sweep the GPU test runs that the reference harness has a chain for (uchar3 Warping and
+    # Deinterlace, BorderReader of both element types), against the live reference CPU backend
+    if not ol.have_ref():
+        pytest.skip("the reference CPU backend is not built here")
+    borders = [ol.BORDER_CONSTANT, ol.BORDER_REPLICATE, ol.BORDER_REFLECT, ol.BORDER_WRAP, ol.BORDER_REFLECT_101]
+    for i in range(1000):
+        family, c = rc.reader_sweep_case(i)
+        img = c["img"]
+        if family == 0:
+            want = ol.oracle_warp(img, 3, c["matrix"], c["dst"], c["perspective"])
+            got = ol.ref_warp_u8x3(img, c["matrix"], c["dst"], c["perspective"])
+        elif family == 2:
+            want = ol.oracle_deinterlace(img, 3, c["mode"])
+            got = ol.ref_deinterlace_u8x3(img, c["mode"])
+            if c["mode"] == ol.DEINTERLACE_LINEAR_ODD and img.shape[0] % 2:
+                # outside the reference's domain: its last line reads past the image (here it is defined as the last line)
+                want, got = want[:-1], got[:-1]
+        elif family == 3:
+            want = ol.oracle_pad(img, borders[c["border"]], c["left"], c["top"], c["out_w"], c["out_h"], value=c["value"])
+            got = ol.ref_pad(img, borders[c["border"]], c["left"], c["top"], c["out_w"], c["out_h"], value=c["value"])
+        else:
+            continue
+        assert got.tobytes() == want.tobytes(), f"case {i} (family {family})"
