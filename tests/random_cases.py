@@ -177,3 +177,38 @@ def reader_sweep_case(i):
     else:
         img, value = (rng.random_sample((h, w)) * 100 - 50).astype(np.float32), (-1.5,)
     return family, dict(img=img, border=border, left=left, top=top, out_w=out_w, out_h=out_h, value=value)
+
+
+def color_sweep_case(i, y2r, r2y, resize_formats):
+    """Case i of a seeded sweep over the pixel-format chains: family 0 ReadYUV -> ConvertYUVToRGB, 1 ConvertRGBToYUV ->
+    WriteYUV (odd sizes leave the last chroma block to one column or row), 2 ReadYUV under a bilinear resize.  `y2r`, `r2y`:
+    the (pixel format, range, primaries) combinations the case driver has chains for; `resize_formats`: pixel formats."""
+    import oracle_lib as ol
+    rng = np.random.RandomState(90000 + i)
+    family = i % 3
+
+    def frame(pf, w, h, pad):
+        rows, cols = ol.frame_shape(pf, w, h)
+        if ol.PF_WIDE[pf]:
+            return rng.randint(0, 1024, (rows, cols + pad)).astype(np.uint16)
+        return rng.randint(0, 256, (rows, cols + pad)).astype(np.uint8)
+
+    if family == 0:
+        pf, cr, cp = y2r[int(rng.randint(0, len(y2r)))]
+        w, h = 2 * int(rng.randint(1, 400)), 2 * int(rng.randint(1, 100))
+        return family, dict(pf=pf, cr=cr, cp=cp, w=w, h=h, frame=frame(pf, w, h, int(rng.randint(0, 6))))
+    if family == 1:
+        pf, cr, cp = r2y[int(rng.randint(0, len(r2y)))]
+        wide = ol.PF_WIDE[pf]
+        w, h = int(rng.randint(1, 500)), int(rng.randint(1, 120))
+        if pf in (ol.PF_Y210, ol.PF_UYVY):
+            w += w & 1
+        rgb = rng.randint(0, 1024 if wide else 256, (h, w, 3)).astype(np.uint16 if wide else np.uint8)
+        rows, cols = ol.frame_shape(pf, w + (w & 1), h + (h & 1))
+        if pf in (ol.PF_NV12, ol.PF_NV21, ol.PF_P010, ol.PF_P210):
+            rows = h + (h + 1) // 2 if pf != ol.PF_P210 else 2 * h     # chroma rows start right after `height` luma rows
+        return family, dict(pf=pf, cr=cr, cp=cp, rgb=rgb, start=np.full((rows, cols + 4), 9, rgb.dtype))
+    pf = resize_formats[int(rng.randint(0, len(resize_formats)))]
+    w, h = 2 * int(rng.randint(1, 200)), 2 * int(rng.randint(1, 100))
+    dst = (int(rng.randint(1, 300)), int(rng.randint(1, 100)))
+    return family, dict(pf=pf, w=w, h=h, dst=dst, frame=frame(pf, w, h, 0))

@@ -80,6 +80,35 @@ def test_yuv_resize(device, pf):
         assert out.cpu().numpy().tobytes() == ol.oracle_yuv_resize(pf, buf, w, h, dst, 0.5).tobytes(), dst
 
 
+RESIZED = [ol.PF_NV21, ol.PF_UYVY, ol.PF_P010]
+
+
+def test_sweep_of_random_sizes(device):
+    """900 seeded cases of the three chain kinds above (tests/random_cases.py) at random sizes and pitches."""
+    import torch
+    import random_cases as rc
+    for i in range(900):
+        family, c = rc.color_sweep_case(i, Y2R, R2Y, RESIZED)
+        pf = c["pf"]
+        if family == 0:
+            out = torch.full((c["h"], c["w"], 3), -7.0, dtype=torch.float32, device=device)
+            cases.yuv_to_rgb(pf, c["cr"], c["cp"], to_dev(c["frame"], device), c["w"], c["h"], out)
+            torch.cuda.synchronize()
+            same = out.cpu().numpy().tobytes() == ol.oracle_yuv_to_rgb(pf, c["cr"], c["cp"], c["frame"], c["w"], c["h"]).tobytes()
+        elif family == 1:
+            dev = to_dev(c["start"].copy(), device)
+            cases.rgb_to_yuv(pf, c["cr"], c["cp"], to_dev(c["rgb"], device), dev)
+            torch.cuda.synchronize()
+            same = np.array_equal(to_host(dev, c["rgb"].dtype), ol.oracle_rgb_to_yuv(pf, c["cr"], c["cp"], c["rgb"], c["start"].copy()))
+        else:
+            dst = c["dst"]
+            out = torch.zeros((dst[1], dst[0], 3), dtype=torch.float32, device=device)
+            cases.yuv_resize(pf, to_dev(c["frame"], device), c["w"], c["h"], dst, 0.5, out)
+            torch.cuda.synchronize()
+            same = out.cpu().numpy().tobytes() == ol.oracle_yuv_resize(pf, c["frame"], c["w"], c["h"], dst, 0.5).tobytes()
+        assert same, f"case {i} (family {family}): " + str({k: v for k, v in c.items() if not isinstance(v, np.ndarray)})
+
+
 @pytest.mark.parametrize("cd,cr,cp", DEPTHS)
 def test_depth_conversions(device, cd, cr, cp):
     import torch

@@ -304,3 +304,26 @@ def test_normalize_matches_reference_backend(which):
     dt, mx = ol.NORMALIZE[which]
     src = rng(700 + which).integers(0, int(mx) + 1, (6, 27, 3)).astype(dt)
     assert ol.oracle_normalize(which, src).tobytes() == ol.ref_normalize(which, src).tobytes()
+
+
+@needs_ref
+def test_oracle_equals_the_reference_backend_on_the_sweep_of_random_sizes():
+    # the 900 cases tests/test_gpu_color.py runs on the GPU (tests/random_cases.py); RGB -> YUV only at even sizes, odd
+    # ones being outside what the reference's writers define
+    import random_cases as rc
+    for i in range(900):
+        family, c = rc.color_sweep_case(i, Y2R, R2Y, [ol.PF_NV21, ol.PF_UYVY, ol.PF_P010])
+        pf = c["pf"]
+        if family == 0:
+            same = ol.oracle_yuv_to_rgb(pf, c["cr"], c["cp"], c["frame"], c["w"], c["h"]).tobytes() == \
+                ol.ref_yuv_to_rgb(pf, c["cr"], c["cp"], c["frame"], c["w"], c["h"]).tobytes()
+        elif family == 1:
+            h, w = c["rgb"].shape[:2]
+            if (w | h) & 1:
+                continue
+            same = np.array_equal(ol.oracle_rgb_to_yuv(pf, c["cr"], c["cp"], c["rgb"], c["start"].copy()),
+                                  ol.ref_rgb_to_yuv(pf, c["cr"], c["cp"], c["rgb"], c["start"].copy()))
+        else:
+            same = ol.oracle_yuv_resize(pf, c["frame"], c["w"], c["h"], c["dst"], 0.5).tobytes() == \
+                ol.ref_yuv_resize(pf, c["frame"], c["w"], c["h"], c["dst"], 0.5).tobytes()
+        assert same, f"case {i} (family {family})"
