@@ -82,3 +82,16 @@ def dual_inputs(which, cases, h, w, seed):
             v[:2] = [0, 0xffffffff]
         out.append(v.reshape(shape))
     return out
+
+
+def sweep_case(i, cases, dual_cases):
+    """Case i of a seeded sweep over the per-channel chains (even i) and the two-image chains (odd i): which chain, image
+    size (40 to 900 wide, 1 to 12 rows) and the padding of each pitch in elements of the wider of input and output."""
+    rng = np.random.RandomState(110000 + i)
+    w, h = int(rng.randint(40, 900)), int(rng.randint(1, 12))
+    table = cases if i % 2 == 0 else dual_cases
+    keys = sorted(table)
+    which = keys[int(rng.randint(0, len(keys)))]
+    in_dtype, _, out_dtype = table[which]
+    unit = max(np.dtype(in_dtype).itemsize, np.dtype(out_dtype).itemsize)
+    return i % 2, which, w, h, [int(rng.randint(0, 4)) * unit for _ in range(2)]

@@ -158,3 +158,34 @@ def test_two_image_and_split_properties_at_full_size(device):
     cases.split_write(0, dimg, w, h, planes)
     torch.cuda.synchronize()
     assert np.stack([p.cpu().numpy() for p in planes], axis=-1).tobytes() == img.tobytes()
+
+
+@pytest.mark.gpu
+def test_sweep_of_random_sizes(device):
+    # 800 seeded cases (tests/pointwise_cases.py: sweep_case): every per-channel and two-image chain at random sizes and pitches
+    import torch
+    for i in range(800):
+        two, which, w, h, pads = pc.sweep_case(i, po.CASES, po.DUAL_CASES)
+        if not two:
+            src = pc.inputs(which, po.CASES, h, w, i)
+            want = po.run(which, src, pc.constants(which), pc.MATRIX)
+            got = run_on_gpu(device, which, src, pads[0], pads[1])
+            assert pc.same(which, got, want, po.INEXACT), (i, which, w, h, pads)
+            continue
+        in_dtype, cn, out_dtype = po.DUAL_CASES[which]
+        a, b = pc.dual_inputs(which, po.DUAL_CASES, h, w, i)
+        want = po.run_dual(which, a, b)
+        row = w * cn * np.dtype(in_dtype).itemsize
+        devs = []
+        for img, extra in ((a, pads[0]), (b, pads[1])):
+            buf = np.zeros((h, row + extra), np.uint8)
+            buf[:, :row] = np.ascontiguousarray(img).view(np.uint8).reshape(h, row)
+            devs.append(torch.from_numpy(buf).to(device))
+        out_row = w * cn * np.dtype(out_dtype).itemsize
+        dev_out = torch.full((h, out_row + 4), 0xA5, dtype=torch.uint8, device=device)
+        cases.dual(which, devs[0], devs[1], w, h, dev_out)
+        torch.cuda.synchronize()
+        got = dev_out.cpu().numpy()
+        assert np.all(got[:, out_row:] == 0xA5), (i, which, w, h, pads)
+        got = np.ascontiguousarray(got[:, :out_row]).view(out_dtype).reshape(want.shape)
+        assert _same_with_any_nan(got, want), (i, which, w, h, pads)

@@ -134,3 +134,21 @@ def test_two_image_and_split_chains_equal_the_committed_reference_vectors():
         planes = ol.oracle_split_write(which, src, (29, 17) if which == 3 else None, (0.5, -2.0, 3.25, 0))
         for k, plane in enumerate(planes):
             assert plane.tobytes() == g[f"split_out_{which}_{k}"].tobytes(), (which, k)
+
+
+@pytest.mark.skipif(not ol.have_ref(), reason="oracle/_ref not built")
+def test_oracle_equals_the_reference_backend_on_the_sweep_of_random_sizes():
+    # the 800 cases tests/test_gpu_pointwise.py runs on the GPU (pointwise_cases.sweep_case)
+    for i in range(800):
+        two, which, w, h, pads = pc.sweep_case(i, po.CASES, po.DUAL_CASES)
+        if not two:
+            src = pc.inputs(which, po.CASES, h, w, i)
+            want = ol.ref_pointwise(which, src, pc.constants(which), pc.MATRIX)
+            assert pc.same(which, po.run(which, src, pc.constants(which), pc.MATRIX), want, po.INEXACT), (i, which, w, h)
+        else:
+            a, b = pc.dual_inputs(which, po.DUAL_CASES, h, w, i)
+            want = ol.ref_dual(which, a, b, pad=tuple(pads))
+            got = po.run_dual(which, a, b)
+            same = got.tobytes() == want.tobytes() or np.array_equal(np.isnan(got), np.isnan(want)) and \
+                np.array_equal(got[~np.isnan(got)].view(np.uint8), want[~np.isnan(want)].view(np.uint8))
+            assert got.dtype == want.dtype and same, (i, which, w, h)
