@@ -212,3 +212,35 @@ def color_sweep_case(i, y2r, r2y, resize_formats):
     w, h = 2 * int(rng.randint(1, 200)), 2 * int(rng.randint(1, 100))
     dst = (int(rng.randint(1, 300)), int(rng.randint(1, 100)))
     return family, dict(pf=pf, w=w, h=h, dst=dst, frame=frame(pf, w, h, 0))
+
+
+def chain_sweep_case(i):
+    """Case i of a seeded sweep over the rest of the benchmark chains: family 0 the float chain of N alternating Add / Mul
+    (N in 1, 2, 3, 10, 50, 100; with and without the thread-fusion spelling), 1 four uchar3 images with their own Mul and Add
+    in one launch, 2 the normalising chain on eight crops of which only the first `used` are read, 3 an array of four images
+    of which only the first `active` are read.  Sizes from 1 x 1 to 700 x 40, padded pitches."""
+    rng = np.random.RandomState(130000 + i)
+    family = i % 4
+    w, h = int(rng.randint(1, 700)), int(rng.randint(1, 40))
+    if family == 0:
+        n = int(rng.choice([1, 2, 3, 10, 50, 100]))
+        pads = (int(rng.randint(0, 4)), int(rng.randint(0, 4)))
+        src = (rng.random_sample((h, w + pads[0])) * 2 - 1).astype(np.float32)
+        return family, dict(n=n, w=w, src=src, out_pad=pads[1], tf=int(rng.randint(0, 2)))
+    if family == 1:
+        pad = int(rng.randint(0, 4))
+        backings = [rng.randint(0, 256, (h, w * 3 + pad)).astype(np.uint8) for _ in range(4)]
+        return family, dict(w=w, backings=backings, mul=rng.uniform(0.5, 2, (4, 3)).astype(np.float32),
+                            add=rng.uniform(-64, 64, (4, 3)).astype(np.float32))
+    if family == 2:
+        w = max(w, 2)
+        used = int(rng.randint(0, 9))
+        dst = (int(rng.randint(1, 200)), int(rng.randint(1, 30)))
+        img = rng.randint(0, 256, (h, w, 3)).astype(np.uint8)
+        r = rects(rng, 8, w, h, 1)
+        default = rng.uniform(-5, 300, 3).astype(np.float32)
+        sub = rng.uniform(0, 130, 3).astype(np.float32)
+        div = rng.choice([58.395, 57.12, 0.7, 3.0, 255.0], 3).astype(np.float32)
+        return family, dict(img=img, rects=r, dst=dst, used=used, default=default, sub=sub, div=div)
+    active = int(rng.randint(0, 5))
+    return family, dict(active=active, imgs=[rng.randint(0, 256, (h, w, 3)).astype(np.uint8) for _ in range(4)])

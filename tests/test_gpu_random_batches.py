@@ -142,3 +142,41 @@ def test_sweep_of_random_reader_cases_equals_the_oracle(device):
         got = out.cpu().numpy()
         assert got.shape == want.shape and got.tobytes() == want.tobytes(), \
             f"case {i} (family {family}, source {img.shape}) differs from the oracle: " + str({k: v for k, v in c.items() if k != "img"})
+
+
+def test_sweep_of_random_chain_cases_equals_the_oracle(device):
+    # 1 200 cases of random_cases.chain_sweep_case: the float chain, the horizontal batch, the two conditional batches
+    import torch
+    for i in range(1200):
+        family, c = rc.chain_sweep_case(i)
+        if family == 0:
+            w, src = c["w"], c["src"]
+            o = torch.full((src.shape[0], w + c["out_pad"]), 5.0, dtype=torch.float32, device=device)
+            cases.add_mul_chain(torch.from_numpy(src).to(device)[:, :w], c["n"], 0.5, 1.0001, o[:, :w], tf=c["tf"])
+            torch.cuda.synchronize()
+            got = o.cpu().numpy()
+            want = ol.oracle_add_mul_chain(np.ascontiguousarray(src[:, :w]), c["n"], 0.5, 1.0001)
+            same = got[:, :w].tobytes() == want.tobytes() and bool((got[:, w:] == 5.0).all())
+        elif family == 1:
+            w, h = c["w"], c["backings"][0].shape[0]
+            srcs = [_image_on(device, b, w) for b in c["backings"]]
+            outs = [torch.zeros((h, w, 3), dtype=torch.uint8, device=device) for _ in range(4)]
+            cases.batch_muladd_sat(srcs, c["mul"], c["add"], outs)
+            torch.cuda.synchronize()
+            want = ol.oracle_batch_muladd_sat([np.ascontiguousarray(rc.image_of(b, w)) for b in c["backings"]], c["mul"], c["add"])
+            same = np.stack([o.cpu().numpy() for o in outs]).tobytes() == np.stack(want).tobytes()
+        elif family == 2:
+            dst = c["dst"]
+            out = torch.full((8, 3, dst[1], dst[0]), 7.0, dtype=torch.float32, device=device)
+            cases.crop_resize_default_norm_split(torch.from_numpy(c["img"]).to(device), c["rects"], dst, c["used"], c["default"],
+                                                 c["sub"], c["div"], out)
+            torch.cuda.synchronize()
+            want = ol.oracle_crop_resize_default_norm_split(c["img"], c["rects"], dst, c["used"], c["default"], c["sub"], c["div"])
+            same = out.cpu().numpy().tobytes() == want.tobytes()
+        else:
+            h, w = c["imgs"][0].shape[:2]
+            out = torch.zeros((4, h, w, 3), dtype=torch.float32, device=device)
+            cases.batch_default_cast_mul([torch.from_numpy(s).to(device) for s in c["imgs"]], c["active"], (7, 200, 33), (0.5, 2.0, 1.25), out)
+            torch.cuda.synchronize()
+            same = out.cpu().numpy().tobytes() == ol.oracle_batch_default_cast_mul(c["imgs"], c["active"], (7, 200, 33), (0.5, 2.0, 1.25)).tobytes()
+        assert same, f"case {i} (family {family}) differs from the oracle: " + str({k: v for k, v in c.items() if not isinstance(v, (np.ndarray, list))})

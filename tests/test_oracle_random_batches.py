@@ -95,3 +95,26 @@ def test_oracle_equals_the_reference_backend_on_the_reader_sweep():
         else:
             continue
         assert got.tobytes() == want.tobytes(), f"case {i} (family {family})"
+
+
+def test_oracle_equals_the_reference_backend_on_the_chain_sweep():
+    # the 1 200 cases of the chain sweep the GPU test runs, against the live reference CPU backend
+    if not ol.have_ref():
+        pytest.skip("the reference CPU backend is not built here")
+    for i in range(1200):
+        family, c = rc.chain_sweep_case(i)
+        if family == 0:
+            src = c["src"][:, :c["w"]]
+            same = ol.oracle_add_mul_chain(np.ascontiguousarray(src), c["n"], 0.5, 1.0001).tobytes() == \
+                ol.ref_add_mul_chain(src, c["n"], 0.5, 1.0001, c["tf"]).tobytes()
+        elif family == 1:
+            imgs = [rc.image_of(b, c["w"]) for b in c["backings"]]
+            want = ol.oracle_batch_muladd_sat([np.ascontiguousarray(x) for x in imgs], c["mul"], c["add"])
+            same = np.stack(ol.ref_batch_muladd_sat(imgs, c["mul"], c["add"])).tobytes() == np.stack(want).tobytes()
+        elif family == 2:
+            args = (c["img"], c["rects"], c["dst"], c["used"], c["default"], c["sub"], c["div"])
+            same = ol.oracle_crop_resize_default_norm_split(*args).tobytes() == ol.ref_crop_resize_default_norm_split(*args).tobytes()
+        else:
+            args = (c["imgs"], c["active"], (7, 200, 33), (0.5, 2.0, 1.25))
+            same = ol.oracle_batch_default_cast_mul(*args).tobytes() == ol.ref_batch_default_cast_mul(*args).tobytes()
+        assert same, f"case {i} (family {family})"
