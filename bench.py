@@ -50,6 +50,9 @@ def parse():
     ap.add_argument("--rows-sweep", action="store_true",
                     help="time configuration 3's chain for 8 to 448 output rows per plane (224 wide, the same 64 crops), print one "
                          "line per height and the straight line through the heights that fill the GPU, and exit")
+    ap.add_argument("--two-streams", action="store_true",
+                    help="time configuration 3's launches as two independent sequences on two streams (each with its own output), "
+                         "against one sequence of the same number of launches on one stream, print both and exit")
     ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
@@ -143,6 +146,34 @@ def main():
     src3 = torch.from_numpy(c3["src"]).to(dev)
     out3 = torch.zeros((64, 3, 224, 224), dtype=torch.float32, device=dev)
     f3 = lambda: cases.crop_resize_norm_split(src3, c3["rects"], c3["dst"], c3["sub"], c3["div"], out3)
+    if args.two_streams:
+        # Launches on one stream run one after the other: each pays the start and the end of a launch by itself.  Two
+        # sequences that do not depend on each other (two halves of a stream of batches, each writing its own tensor) may
+        # overlap on the GPU.  Wall clock around K launches per sequence, enqueued by the C++ case driver.
+        k = max(args.steps, 200)
+        outs = [torch.zeros((64, 3, 224, 224), dtype=torch.float32, device=dev) for _ in range(2)]
+        streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
+        def sequence(i):
+            with torch.cuda.stream(streams[i]):
+                cases.set_reps(k)
+                cases.crop_resize_norm_split(src3, c3["rects"], c3["dst"], c3["sub"], c3["div"], outs[i])
+        def timed(which):
+            torch.cuda.synchronize(); time.sleep(0.03)
+            t0 = time.perf_counter()
+            for i in which:
+                sequence(i)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e6 / (k * len(which))
+        for i in (0, 1):
+            sequence(i)
+        one = min(timed([0, 0]) for _ in range(5))
+        two = min(timed([0, 1]) for _ in range(5))
+        want = outs[0].cpu().numpy().tobytes()
+        assert outs[1].cpu().numpy().tobytes() == want
+        print(f"{2 * k} launches of configuration 3 on one stream:  {one:.2f} us per launch (wall clock)")
+        print(f"{k} + {k} launches on two streams:                {two:.2f} us per launch ({a3 / (two * 1e-6) / 1e12:.2f} TB/s of algorithmic bytes, "
+              f"{100 * a3 / (two * 1e-6) / 1e9 / HBM_PEAK_GBS:.0f} % of peak)")
+        return
     if args.rows_sweep:
         heights = (8, 56, 112, 168, 224, 336, 448, 672, 896)
         best = {}
