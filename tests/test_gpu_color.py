@@ -163,3 +163,50 @@ def test_normalize(device, which):
     cases.normalize(which, to_dev(src, device), out)
     torch.cuda.synchronize()
     assert out.cpu().numpy().tobytes() == ol.oracle_normalize(which, src).tobytes()
+
+
+def test_sweep_of_random_sizes_of_the_per_pixel_conversions(device):
+    """400 seeded cases at random sizes (1 x 1 to 600 x 12): the depth conversions in both directions, every ColorConversion
+    code, NormalizePixel.  Inputs as in the tests above."""
+    import torch
+    codes = sorted(ol.COLOR_CODES)
+    for i in range(400):
+        r = np.random.default_rng(150000 + i)
+        h, w = int(r.integers(1, 13)), int(r.integers(1, 601))
+        kind = i % 3
+        if kind == 0:
+            cd, cr, cp = DEPTHS[int(r.integers(0, len(DEPTHS)))]
+            to_rgb = bool(r.integers(0, 2))
+            if cd >= 3:
+                src = (r.random((h, w, 3), dtype=np.float32) * np.float32(1.2) - np.float32(0.1)).astype(np.float32)
+            elif cd == 0:
+                src = r.integers(0, 256, (h, w, 3), dtype=np.uint8)
+            else:
+                src = r.integers(0, 4096, (h, w, 3)).astype(np.uint16)
+            out = torch.zeros((h, w, 3), dtype=torch.float32, device=device)
+            cases.convert_depth(cd, cr, cp, to_rgb, to_dev(src, device), out)
+            torch.cuda.synchronize()
+            same = out.cpu().numpy().tobytes() == ol.oracle_convert_depth(cd, cr, cp, to_rgb, src).tobytes()
+            what = ("depth", cd, cr, cp, to_rgb)
+        elif kind == 1:
+            which = codes[int(r.integers(0, len(codes)))]
+            idt, cin, odt, cout, _ = ol.COLOR_CODES[which]
+            if idt == np.float32:
+                src = (r.random((h, w, cin), dtype=np.float32) * np.float32(255.0)).astype(np.float32)
+            else:
+                src = r.integers(0, 256 if idt == np.uint8 else 1024, (h, w, cin)).astype(idt)
+            out = to_dev(np.zeros((h, w, cout) if cout > 1 else (h, w), odt), device)
+            cases.convert_code(which, to_dev(src, device), out)
+            torch.cuda.synchronize()
+            same = to_host(out, odt).tobytes() == ol.oracle_convert_code(which, src).tobytes()
+            what = ("code", which)
+        else:
+            which = int(r.integers(0, 2))
+            dt, mx = ol.NORMALIZE[which]
+            src = r.integers(0, int(mx) + 1, (h, w, 3)).astype(dt)
+            out = torch.zeros((h, w, 3), dtype=torch.float32, device=device)
+            cases.normalize(which, to_dev(src, device), out)
+            torch.cuda.synchronize()
+            same = out.cpu().numpy().tobytes() == ol.oracle_normalize(which, src).tobytes()
+            what = ("normalize", which)
+        assert same, (i, what, w, h)
