@@ -61,3 +61,40 @@ def test_circular_tensor_reference_scenario(device):
     got = cases.circular(batch, False, imgs, 10.0)
     for z in range(batch):
         assert (got[-1, z] == float(iters - z)).all()
+
+
+def test_sweep_of_random_sizes(device):
+    """150 seeded cases at random sizes: the two divergent launches above, and the window for every batch size and
+    order the case driver has (2, 3, 4, 15; newest or oldest first) with a random number of updates."""
+    import torch
+    for i in range(150):
+        r = np.random.default_rng(170000 + i)
+        h, w = int(r.integers(1, 60)), int(r.integers(1, 400))
+        kind = i % 3
+        if kind == 0:
+            a = r.integers(0, 2**32, (h, w), dtype=np.uint32)
+            b = r.integers(0, 2**32, (h, w), dtype=np.uint32)
+            add = int(r.integers(0, 1000))
+            out = torch.zeros((2, h, w), dtype=torch.int32, device=device)
+            cases.divergent_two(torch.from_numpy(a.view(np.int32)).to(device), torch.from_numpy(b.view(np.int32)).to(device), add, out)
+            torch.cuda.synchronize()
+            got = out.cpu().numpy().view(np.uint32)
+            same = np.array_equal(got[0], a + np.uint32(add)) and np.array_equal(got[1], b)
+        elif kind == 1:
+            ih, iw = int(r.integers(1, 200)), int(r.integers(2, 300))
+            t = (r.random((4, h, w, 3), dtype=np.float32) * 10 - 5).astype(np.float32)
+            img = r.integers(0, 256, (ih, iw, 3), dtype=np.uint8)
+            mul = float(np.float32(r.uniform(0.1, 4.0)))
+            out = torch.full((4, h, w, 3), -1.0, dtype=torch.float32, device=device)
+            cases.divergent_mixed(torch.from_numpy(t).to(device), mul, torch.from_numpy(img).to(device), out)
+            torch.cuda.synchronize()
+            same = out.cpu().numpy().tobytes() == ol.oracle_divergent_mixed(t, mul, img).tobytes()
+        else:
+            batch = int(r.choice([2, 3, 4, 15]))
+            oldest_first = bool(r.integers(0, 2))
+            imgs = [r.integers(0, 256, (h, w, 3), dtype=np.uint8) for _ in range(batch + int(r.integers(0, 6)))]
+            got = cases.circular(batch, oldest_first, [torch.from_numpy(x).to(device) for x in imgs], 10.0)
+            want = ol.oracle_circular(batch, oldest_first, imgs, 10.0)
+            defined = ~np.isnan(want)
+            same = np.array_equal(got[defined], want[defined])
+        assert same, (i, kind, w, h)
