@@ -137,3 +137,13 @@ def test_split_write(which):
 def test_two_image_chains(which):
     # DualSourceRead and the two-input forms of Add ... BwOr on this repository's CPU executor
     on_host_executor(t_pointwise.test_two_image_chains_equal_the_reference_backend, which)
+
+
+def test_sweeps_of_random_cases():
+    # the seeded sweeps that hold the oracle to the reference backend (and the GPU to the oracle), on this executor
+    import test_oracle_random_batches as t_random
+    on_host_executor(t_random.test_oracle_equals_the_reference_backend_on_the_sweep)
+    on_host_executor(t_random.test_oracle_equals_the_reference_backend_on_the_reader_sweep)
+    on_host_executor(t_random.test_oracle_equals_the_reference_backend_on_the_chain_sweep)
+    on_host_executor(t_color.test_oracle_equals_the_reference_backend_on_the_sweep_of_random_sizes)
+    on_host_executor(t_pointwise.test_oracle_equals_the_reference_backend_on_the_sweep_of_random_sizes)
