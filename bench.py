@@ -43,16 +43,6 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--list-compiled", action="store_true",
                     help="print to stderr the kernel symbol and signature of every chain compiled at run time")
-    ap.add_argument("--issue-rate", action="store_true",
-                    help="run the stand-alone instruction-issue measurement (fusedkernellibrary_amd/probe_issue_rate) and exit")
-    ap.add_argument("--uchar3-access", action="store_true",
-                    help="run the stand-alone comparison of access forms for uchar3 rows (fusedkernellibrary_amd/probe_uchar3_rows) and exit")
-    ap.add_argument("--rows-sweep", action="store_true",
-                    help="time configuration 3's chain for 8 to 448 output rows per plane (224 wide, the same 64 crops), print one "
-                         "line per height and the straight line through the heights that fill the GPU, and exit")
-    ap.add_argument("--two-streams", action="store_true",
-                    help="time configuration 3's launches as two independent sequences on two streams (each with its own output), "
-                         "against one sequence of the same number of launches on one stream, print both and exit")
     ap.add_argument("--only", default="", help="comma separated subset of c1,c2,c3,c4,c5,ext (c3 is always run)")
     return ap.parse_args()
 
@@ -96,13 +86,6 @@ class Timer:
 
 def main():
     args = parse()
-    if args.issue_rate or args.uchar3_access:
-        import subprocess
-        probe = os.path.join(ROOT, "fusedkernellibrary_amd", "probe_issue_rate" if args.issue_rate else "probe_uchar3_rows")
-        if not os.path.exists(probe):
-            print(f"bench.py: {probe} is missing: build it with `python -m fusedkernellibrary_amd.build`", file=sys.stderr)
-            sys.exit(1)
-        sys.exit(subprocess.run([probe]).returncode)
     if args.gpus != 1:
         print(f"bench.py: this path runs on ONE GPU (asked for {args.gpus}); every output pixel is independent, "
               "so more GPUs would only split the batch. Run with --gpus 1.", file=sys.stderr)
@@ -146,52 +129,6 @@ def main():
     src3 = torch.from_numpy(c3["src"]).to(dev)
     out3 = torch.zeros((64, 3, 224, 224), dtype=torch.float32, device=dev)
     f3 = lambda: cases.crop_resize_norm_split(src3, c3["rects"], c3["dst"], c3["sub"], c3["div"], out3)
-    if args.two_streams:
-        # Launches on one stream run one after the other: each pays the start and the end of a launch by itself.  Two
-        # sequences that do not depend on each other (two halves of a stream of batches, each writing its own tensor) may
-        # overlap on the GPU.  Wall clock around K launches per sequence, enqueued by the C++ case driver.
-        k = max(args.steps, 200)
-        outs = [torch.zeros((64, 3, 224, 224), dtype=torch.float32, device=dev) for _ in range(2)]
-        streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
-        def sequence(i):
-            with torch.cuda.stream(streams[i]):
-                cases.set_reps(k)
-                cases.crop_resize_norm_split(src3, c3["rects"], c3["dst"], c3["sub"], c3["div"], outs[i])
-        def timed(which):
-            torch.cuda.synchronize(); time.sleep(0.03)
-            t0 = time.perf_counter()
-            for i in which:
-                sequence(i)
-            torch.cuda.synchronize()
-            return (time.perf_counter() - t0) * 1e6 / (k * len(which))
-        for i in (0, 1):
-            sequence(i)
-        one = min(timed([0, 0]) for _ in range(5))
-        two = min(timed([0, 1]) for _ in range(5))
-        want = outs[0].cpu().numpy().tobytes()
-        assert outs[1].cpu().numpy().tobytes() == want
-        print(f"{2 * k} launches of configuration 3 on one stream:  {one:.2f} us per launch (wall clock)")
-        print(f"{k} + {k} launches on two streams:                {two:.2f} us per launch ({a3 / (two * 1e-6) / 1e12:.2f} TB/s of algorithmic bytes, "
-              f"{100 * a3 / (two * 1e-6) / 1e9 / HBM_PEAK_GBS:.0f} % of peak)")
-        return
-    if args.rows_sweep:
-        heights = (8, 56, 112, 168, 224, 336, 448, 672, 896)
-        best = {}
-        for _ in range(3):
-            for hh in heights:
-                o = torch.zeros((64, 3, hh, 224), dtype=torch.float32, device=dev)
-                us = timer.run(lambda: cases.crop_resize_norm_split(src3, c3["rects"], (224, hh), c3["sub"], c3["div"], o),
-                               args.steps, args.warmup)[1] * 1e3
-                best[hh] = min(best.get(hh, 1e9), us)
-                del o
-        for hh in heights:
-            print(f"rows per plane {hh:4d}   workgroups {64 * ((hh + 7) // 8):5d}   output {64 * 3 * hh * 224 * 4 / 1e6:7.2f} MB   "
-                  f"{best[hh]:7.2f} us per launch")
-        hs = np.array([hh for hh in heights if hh % 224 == 0], dtype=np.float64)   # whole rounds of 7 workgroups per compute unit
-        slope, fixed = np.polyfit(hs, np.array([best[int(hh)] for hh in hs]), 1)
-        print(f"through the heights that are whole multiples of 224: {fixed:.2f} us + {slope * 224:.2f} us per 224 rows "
-              f"(38.54 MB of output: {64 * 3 * 224 * 224 * 4 / (slope * 224 * 1e-6) / 1e12:.2f} TB/s)")
-        return
     # (timed after the other configurations, further down: the first launches of a process run on a GPU that has not
     # reached its working clocks yet, and the headline should not depend on what happened to be measured first)
 
@@ -218,7 +155,7 @@ def main():
                    args.steps, args.warmup)
             if n >= 50:
                 # n dependent fp32 instructions per element that no contraction or packing may merge: 8.3 M elements are
-                # 129 600 wave-wide elements, at the 2.45 cycles per instruction and SIMD this chip issues (--issue-rate)
+                # 129 600 wave-wide elements, at the 2.45 cycles per instruction and SIMD this chip was measured to issue
                 results[f"c2_n{n}"]["valu_issue_floor_us"] = 129600 * n * 2.45 / 1024 / 2.3e3
         record("copy_f32_4k", 3840 * 2160, 2 * 3840 * 2160 * 4, lambda: cases.copy_f32(s, o), args.steps, args.warmup)
     if "c5" in only:
