@@ -23,7 +23,7 @@ ABI_SYMBOLS = (
     "fklhip_free", "fklhip_host_alloc", "fklhip_host_free", "fklhip_memcpy_async", "fklhip_memcpy2d_async",
     "fklhip_memset_async", "fklhip_event_create", "fklhip_event_destroy", "fklhip_event_record", "fklhip_event_sync",
     "fklhip_event_elapsed_ms", "fklhip_lookup", "fklhip_launch_handle", "fklhip_launch", "fklhip_last_launch",
-    "fklhip_signature_count", "fklhip_signature_at", "fklhip_jit_log",
+    "fklhip_signature_count", "fklhip_signature_at", "fklhip_jit_log", "fklhip_strip_form",
 )
 
 

@@ -15,6 +15,7 @@ namespace fklhip {
 
 template <class Chain> int aot_launch(const void*, const void* blob, size_t bytes, void* stream, fkd::LaunchInfo* info) {
     using Params = typename Chain::Params;
+    static_assert(sizeof(Params) <= size_t(FKLHIP_MAX_BLOB_BYTES), "the chain's parameter block exceeds FKLHIP_MAX_BLOB_BYTES: use a smaller batch per launch");
     if (!blob) return FKLHIP_EINVAL;
     if (bytes != sizeof(Params)) return FKLHIP_EBLOB_SIZE;
     // The runtime copies the block into its kernel-argument buffer during the launch call, so the caller's block may go

@@ -570,17 +570,14 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
 // pixels.  So the fixed work of a wave is spread over seven pixels per lane instead of four, nearly all of it on the
 // vector unit (the scalar unit is shared by the four SIMDs of a compute unit and was as busy as they were).
 // What the form asks of every plane -- source rows that share their alignment (pitch a multiple of 4), source smaller
-// than 4 GB and at least two columns wide, output plane smaller than 2 GB -- is checked on the host when the parameter
+// than 2 GB and at least two columns wide, output plane smaller than 2 GB -- is checked on the host when the parameter
 // block is made (Chain::finalize_write, bit 0 of Params::reserved); launchers take the tile form when the bit is clear.
 // Taps come through a buffer resource whose extent ends with the image, so windows that reach past the last row read
 // zeros in bytes nobody uses and no lane needs a narrower access; the row is part of the lane's offset.
-#ifndef FKD_STRIP_DEPTH
-#define FKD_STRIP_DEPTH 1
-#endif
-constexpr int kStripRows = kGatherBY * FKD_GATHER_YI, kStripStep = 32, kStripMaxWidth = 256, kStripDepth = FKD_STRIP_DEPTH;
-constexpr int kStripThreads = kStripRows * kStripStep;
+constexpr int kStripRows = kGatherBY * FKD_GATHER_YI, kStripStep = 32, kStripMaxWidth = 256;
+constexpr int kStripThreads = kStripRows * kStripStep, kStripMaxSteps = kStripMaxWidth / kStripStep;
 static_assert(kStripThreads == kGatherBX * kGatherBY, "the two forms of the bilinear kernel share their workgroup shape");
-static_assert(kStripThreads == kStripMaxWidth && (kStripDepth + 1) * kStripStep <= kStripThreads, "one table column per thread");
+static_assert(kStripThreads == kStripMaxWidth, "one table column per thread");
 
 template <class Chain> constexpr bool strip_capable() {
     using Root = ResizeRoot<typename Chain::Read>;
@@ -604,10 +601,8 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     using Raw = typename Back::Raw;
     using W = typename Chain::Write;
     using WP = typename W::Plane;
-    constexpr int D = kStripDepth;
-    constexpr int kEntries = kStripMaxWidth + (D + 1) * kStripStep;
     // per column: ax, bx, window offset, bytes to drop from the window (bits 0-1) | flags
-    __shared__ detail::u32x4_t column[kEntries];
+    __shared__ detail::u32x4_t column[kStripMaxWidth];
     __shared__ u32 wave_clamped[kStripThreads / 64];
     constexpr u32 kClamped = 0x80000000u, kOutsideX = 0x40000000u;
 
@@ -628,6 +623,7 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     const int sw = Back::width(q.back), sh = Back::height(q.back);
     const detail::TapImage image = Back::tap_image_bounded(z, q.back);
     const int steps = (aw + kStripStep - 1) / kStripStep;
+    if (steps == 0) return;                                             // no columns: nothing to write (the whole workgroup leaves)
 
     const int t = int(threadIdx.y) * 64 + int(threadIdx.x);
     // What depends on the column: the horizontal weights, the window's byte offset in a row, and flags beside the bytes to drop.
@@ -685,19 +681,16 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
         fetch(first);
     }
 
-    // ---- the column table: one column per thread (the workgroup has as many threads as the form has columns); the
-    // D + 1 steps after the last one hold a window offset beyond the image's extent, so requesting them touches no
-    // memory.  Each wave notes whether it met a clamped column. ----
+    // ---- the column table: one column per thread (the workgroup has as many threads as the form has columns).  Columns
+    // of the steps after the last one hold a window offset of 2 GB: the image is smaller than that (checked on the host), so
+    // the sum with the lane's row offset neither wraps nor comes back below the image's extent, and requesting such a
+    // column touches no memory.  Each wave notes whether it met a clamped column. ----
+    constexpr u32 kNoWindow = 0x80000000u;
     {
         bool clamped = false;
         detail::u32x4_t e = column_entry(t, clamped);
-        if (t >= steps * kStripStep) { e.z = 0xfffffff0u; clamped = false; }
+        if (t >= steps * kStripStep) { e.z = kNoWindow; clamped = false; }
         column[t] = e;
-        if (t < (D + 1) * kStripStep) {
-            detail::u32x4_t none;
-            none.x = 0u; none.y = 0u; none.z = 0xfffffff0u; none.w = 0u;
-            column[kStripMaxWidth + t] = none;
-        }
         const bool any = __builtin_amdgcn_ballot_w64(clamped) != 0ull;
         if (threadIdx.x == 0) wave_clamped[threadIdx.y] = any ? 1u : 0u;
     }
@@ -715,7 +708,7 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     auto run = [&](auto static_tag, auto clamp_tag) {
         constexpr bool STATIC = decltype(static_tag)::value != 0;
         constexpr bool CLAMP = decltype(clamp_tag)::value != 0;
-        auto produce = [&](int k, const StepTaps& s, bool beyond) {
+        auto produce = [&](int k, const StepTaps& s) {
             // (the words are copied out first: a bit cast applied directly to an element of the vector reads element 0)
             const u32 ax_bits = s.e.x, bx_bits = s.e.y;
             const f32 ax = __builtin_bit_cast(f32, ax_bits), bx = __builtin_bit_cast(f32, bx_bits);
@@ -737,48 +730,27 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
             if constexpr (STATIC) res = Chain::compute_static_ops(v, ops);
             else res = Chain::compute_checked_ops(v, ops);
             u32 off = out0 + u32(k) * WP::lane_offset(kStripStep, true);
-            if (beyond) off = WP::kMaskedOut;                         // a step of the prologue that does not exist
             if (partial && k == steps - 1) {                          // wave uniform, kept a branch
                 asm volatile("" : "+v"(off));
                 if (g + kStripStep * k >= aw) off = WP::kMaskedOut;
             }
             WP::put_masked(oplane, 0u, off, res);
         };
-        // D steps of taps are in flight behind the step being blended.  Every pass through the loop issues the same
-        // accesses in the same order as the prologue did, and the only branches leave the loop: the compiler's wait for
-        // a step's taps can then leave all later accesses in flight.  (Written out per depth with named tap sets: with
-        // an array of sets the compiler rotates registers instead, and a copy of a register waits for its load.)
-        if constexpr (D == 1) {
-            StepTaps s0 = first, s1;
-            request(1, s1);
-            produce(0, s0, false);
-#pragma unroll 1
-            for (int k = 1; k < steps; k += 2) {
-                request(k + 1, s0);
-                produce(k, s1, false);
-                if (k + 1 >= steps) break;
-                request(k + 2, s1);
-                produce(k + 1, s0, false);
-            }
-        } else {
-            static_assert(D == 2, "depths 1 and 2 are written out");
-            StepTaps s0 = first, s1, s2;
-            request(1, s1);
-            request(2, s2);
-            produce(0, s0, false);
-            request(3, s0);
-            produce(1, s1, steps < 2);
-#pragma unroll 1
-            for (int k = 2; k < steps; k += 3) {
-                request(k + 2, s1);
-                produce(k, s2, false);
-                if (k + 1 >= steps) break;
-                request(k + 3, s2);
-                produce(k + 1, s0, false);
-                if (k + 2 >= steps) break;
-                request(k + 4, s0);
-                produce(k + 2, s1, false);
-            }
+        // One step of taps is in flight behind the step being blended.  The steps are written out (a plane has at most
+        // kStripMaxSteps of them) and the only branches leave the kernel: every step issues the same accesses in the same
+        // order, so the compiler's wait for a step's taps leaves all later accesses in flight, table reads carry their step
+        // in the instruction's immediate offset, and there is no loop bookkeeping.  The request behind the last step meets
+        // a column without a window.
+        StepTaps sa = first, sb;
+        request(1, sb);
+#pragma unroll
+        for (int k = 0; k < kStripMaxSteps; k += 2) {
+            if (k > 0) request(k + 1, sb);
+            produce(k, sa);
+            if (k + 1 >= steps) return;
+            if (k + 2 < kStripMaxSteps) request(k + 2, sa);
+            produce(k + 1, sb);
+            if (k + 2 >= steps) return;
         }
     };
     auto run_static = [&](auto static_tag) {

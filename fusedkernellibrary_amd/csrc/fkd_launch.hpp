@@ -56,9 +56,10 @@ hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, La
     constexpr int TW = kGatherBX * XI, TH = kGatherBY * YI;
     if constexpr (strip_capable<Chain>()) {
         // Narrow outputs (batches of small planes): the strip form, whose workgroups own 8 whole rows of a plane.
-        if (p.active_w <= unsigned(kStripMaxWidth) && (p.reserved & 1u) != 0 && fklhip::strip_enabled()) {
+        // (an output without columns has no workgroup in the tile form's grid: it falls through and launches nothing)
+        if (p.active_w != 0 && p.active_w <= unsigned(kStripMaxWidth) && (p.reserved & 1u) != 0 && fklhip::strip_enabled()) {
             const dim3 grid((p.active_h + kStripRows - 1) / kStripRows, 1, p.active_z), block(kGatherBX, kStripThreads / kGatherBX, 1);
-            if (info) *info = LaunchInfo{"strip", {grid.x, 1, grid.z}, {block.x, block.y, 1}, unsigned((kStripMaxWidth + (kStripDepth + 1) * kStripStep) * 16 + 4)};
+            if (info) *info = LaunchInfo{"strip", {grid.x, 1, grid.z}, {block.x, block.y, 1}, unsigned(kStripMaxWidth * 16 + (kStripThreads / 64) * 4)};
             if (grid.x == 0 || grid.z == 0) return hipSuccess;
             if (grid.z > 65535u) return hipErrorInvalidConfiguration;
             return launch_by_pointer(&k_strip<Chain>, grid, block, stream, p);

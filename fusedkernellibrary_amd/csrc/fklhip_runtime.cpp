@@ -8,6 +8,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -29,7 +30,18 @@ Table& table() {
 
 thread_local fkd::LaunchInfo g_last = {"", {0, 0, 0}, {0, 0, 0}, 0};
 
+// The environment is looked at once (a function-local static: thread safe), afterwards only the atomic is read.
+std::atomic<int>& strip_setting() {
+    static std::atomic<int> setting = [] {
+        const char* e = getenv("FKLHIP_STRIP");
+        return (e && e[0] == '0' && e[1] == 0) ? 0 : 1;
+    }();
+    return setting;
+}
+
 } // namespace
+
+bool strip_enabled() { return strip_setting().load(std::memory_order_relaxed) != 0; }
 
 void register_chain(const char* signature, size_t blob_bytes, LaunchFn fn, const void* ctx) {
     Table& t = table();
@@ -53,7 +65,9 @@ const char* fklhip_error_string(int code) {
     case FKLHIP_EUNKNOWN_SIGNATURE:
         return "no kernel was compiled for this chain signature (add it to aot_signatures.txt and rebuild libfklhip.so)"
                " and it could not be compiled at run time (fklhip_jit_log has the compiler's messages)";
-    case FKLHIP_EBLOB_SIZE: return "parameter block size does not match the chain signature";
+    case FKLHIP_EBLOB_SIZE:
+        return "parameter block size does not match the chain signature, or exceeds FKLHIP_MAX_BLOB_BYTES (1 MiB less 64 bytes:"
+               " the most the library passes on as by-value kernel arguments; split the batch into several launches)";
     case FKLHIP_EINVAL: return "invalid argument";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
     }
@@ -146,7 +160,14 @@ int fklhip_jit_log(const char** log) {
     return FKLHIP_OK;
 }
 
+int fklhip_strip_form(int enable) {
+    std::atomic<int>& s = strip_setting();
+    if (enable < 0) return s.load(std::memory_order_relaxed);
+    return s.exchange(enable != 0 ? 1 : 0, std::memory_order_relaxed);
+}
+
 int fklhip_launch_handle(const void* handle, const void* blob, size_t blob_bytes, void* stream) {
+    if (blob_bytes > size_t(FKLHIP_MAX_BLOB_BYTES)) return FKLHIP_EBLOB_SIZE;   // before anything reaches the runtime
     const size_t idx = reinterpret_cast<size_t>(handle);
     Entry e;
     {

@@ -213,7 +213,7 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
     TileGeom g{0, 0, 0, 0};
     unsigned grid[3], block[3] = {64, 4, 1};
     const char* kind = m.gather ? "gather_jit" : "rows_jit";
-    if (m.gather && m.strip_width != 0 && active[0] <= m.strip_width && (active[3] & 1u) != 0 && strip_enabled()) {
+    if (m.gather && m.strip_width != 0 && active[0] != 0 && active[0] <= m.strip_width && (active[3] & 1u) != 0 && strip_enabled()) {
         // strip form: one workgroup per m.by * m.yi output rows of a plane; the all-zero TileGeom tells the kernel
         kind = "strip_jit";
         grid[0] = (active[1] + m.by * m.yi - 1) / (m.by * m.yi);
@@ -328,6 +328,15 @@ static int build_and_register(const char* signature, bool may_read_cache, bool a
         g_log = std::string("loading the compiled chain failed: ") + hipGetErrorString(e);
         return int(e);
     }
+    if (k->meta.params_bytes > unsigned(FKLHIP_MAX_BLOB_BYTES)) {
+        // by-value kernel arguments beyond what the library passes on to the runtime: refused here, with a sentence,
+        // instead of failing inside the launch call
+        g_log = "the chain's parameter block is " + std::to_string(k->meta.params_bytes) + " bytes; a launch accepts at most " +
+                std::to_string(FKLHIP_MAX_BLOB_BYTES) + " (FKLHIP_MAX_BLOB_BYTES): use a smaller batch per launch";
+        hipModuleUnload(mod);
+        delete k;
+        return FKLHIP_EBLOB_SIZE;
+    }
     // The ahead-of-time build refuses kernels that need scratch memory (a private array the optimiser could not keep in
     // registers, or spills: a silent slowdown of an order of magnitude).  A chain compiled here still runs: it is compiled
     // once more with such arrays moved to LDS, which is the faster of the two homes, and the note goes into the log; with
@@ -354,7 +363,9 @@ static int build_and_register(const char* signature, bool may_read_cache, bool a
     } else if (from_cache) {
         g_log = "loaded from " + cached;
     }
-    if (!from_cache && !cached.empty()) write_file(cached, k->code);
+    // (an object compiled with per-thread arrays in LDS is not kept: the file's name does not say how it was compiled, and
+    // a later process running with FKLHIP_JIT_STRICT=1 would take it for a clean one)
+    if (!from_cache && !cached.empty() && !arrays_to_lds) write_file(cached, k->code);
     int dev = 0;
     hipGetDevice(&dev);
     k->per_device.emplace(dev, fn);

@@ -19,12 +19,9 @@ struct Entry {
     const void* ctx;
 };
 
-// Narrow outputs of bilinear chains are launched in strip form unless FKLHIP_STRIP=0 (read at every launch, so one process
-// can run both forms on the same input; the two give identical results).
-inline bool strip_enabled() {
-    const char* e = getenv("FKLHIP_STRIP");
-    return !(e && e[0] == '0' && e[1] == 0);
-}
+// Narrow outputs of bilinear chains are launched in strip form unless that was switched off: by FKLHIP_STRIP=0 in the
+// environment when the setting is first needed, or by fklhip_strip_form(0) (the two forms give identical results).
+bool strip_enabled();
 
 // Called from static initialisers of the generated instance files, and by the run-time compiler.
 void register_chain(const char* signature, size_t blob_bytes, LaunchFn fn, const void* ctx = nullptr);

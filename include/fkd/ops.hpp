@@ -1467,9 +1467,10 @@ template <class T> struct Read2D {
     static constexpr bool kBoundedOut = small_integer_base<T>();
     FKD_NAME("Read2D<" + type_name<T>() + ">")
     // What the strip form of the bilinear kernel asks of a source image (checked on the host, see Chain::finalize): rows
-    // that share their alignment, 32-bit offsets, two columns.
+    // that share their alignment, byte offsets below 2 GB (the offset 2 GB itself marks a column without a window), two
+    // columns.
     FKD_HD static bool strip_ok(const Params& p) {
-        return p.pitch % 4 == 0 && size_t(p.pitch) * p.height < 0xfffffff0ull && p.width >= 2 && p.height >= 1;
+        return p.pitch % 4 == 0 && size_t(p.pitch) * p.height < 0x7ffffff0ull && p.width >= 2 && p.height >= 1;
     }
 #if defined(FKD_EXEC_CODE)
     FKD_DEV static int width(const Params& p) { return int(p.width); }

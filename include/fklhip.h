@@ -26,11 +26,19 @@ extern "C" {
 enum {
     FKLHIP_OK = 0,
     FKLHIP_EUNKNOWN_SIGNATURE = 10001, /* no kernel was built for this chain signature */
-    FKLHIP_EBLOB_SIZE = 10002,         /* parameter block size does not match the signature */
+    FKLHIP_EBLOB_SIZE = 10002,         /* parameter block size does not match the signature, or exceeds FKLHIP_MAX_BLOB_BYTES */
     FKLHIP_EINVAL = 10003              /* null pointer / malformed argument */
 };
 
 enum { FKLHIP_COPY_H2H = 0, FKLHIP_COPY_H2D = 1, FKLHIP_COPY_D2H = 2, FKLHIP_COPY_D2D = 3 };
+
+/* Largest parameter block a launch accepts.  A chain's parameters travel as by-value kernel arguments, like the
+ * reference's __grid_constant__ arguments (FK/core/execution_model/executor_details/executor_kernels.h:26-30), and
+ * grow with the batch (FK/core/execution_model/operation_model/batch_operations.h:164-219: one entry per plane).
+ * Measured on an MI355X with ROCm 7.2: the HIP runtime accepts 1 048 584 bytes of kernel arguments and the kernel reads
+ * them correctly; with 4 MiB the launch call crashes inside the runtime.  The library therefore refuses anything above
+ * 1 MiB less 64 bytes (room for its own trailing arguments) with FKLHIP_EBLOB_SIZE instead of passing it on. */
+#define FKLHIP_MAX_BLOB_BYTES 1048512
 
 /* Library identity: FKLHIP_ABI_VERSION the library was built with. */
 int fklhip_abi_version(void);
@@ -99,6 +107,13 @@ int fklhip_launch(const char *signature, const void *blob, size_t blob_bytes, vo
  * compiled code objects are kept there (file name = hash of signature, architecture, flags and header text) and
  * reused by later processes; after such a reuse the log reads "loaded from <file>". */
 int fklhip_jit_log(const char **log);
+
+/* The bilinear kernel has two forms that give identical results: tiles, and for outputs up to 256 pixels wide whole
+ * rows ("strip").  fklhip_strip_form(0) makes every later launch of the process take the tile form, fklhip_strip_form(1)
+ * restores the choice by shape, a negative argument changes nothing; the return value is the previous setting (0 or 1).
+ * The initial setting is 1 unless the environment variable FKLHIP_STRIP is "0" when the library first needs it.  No
+ * counterpart in the reference; it exists so that tests can compare the two forms in one process. */
+int fklhip_strip_form(int enable);
 
 /* Introspection for tests and benchmarks: what the last fklhip_launch* on this thread launched.
  * kernel receives "rows", "rows_unaligned", "gather", or "rows_jit" / "gather_jit" for chains compiled at run time; grid/block receive 3 values each. */

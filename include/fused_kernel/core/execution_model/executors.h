@@ -95,6 +95,9 @@ template <typename... IOps> struct FusedChain {
 template <typename... IOps> void launch_fused(void* stream, const IOps&... iOps) {
     using F = FusedChain<IOps...>;
     static_assert(!F::kTee, "a MidWrite operation is only supported inside the sequences of a DivergentBatchTransformDPP launch");
+    static_assert(sizeof(typename F::Chain::Params) <= size_t(FKLHIP_MAX_BLOB_BYTES),
+                  "the fused chain's parameters exceed FKLHIP_MAX_BLOB_BYTES (1 MiB of by-value kernel arguments): every plane of a "
+                  "BatchRead or BatchWrite adds its own parameters, so use a smaller BATCH per launch");
     const typename F::Chain::Params p = F::params(iOps...);
     gpuErrchk(fklhip_launch_handle(kernel_handle<typename F::Chain>(), &p, sizeof(p), stream));
 }
@@ -102,6 +105,8 @@ template <typename... IOps> void launch_fused(void* stream, const IOps&... iOps)
 // Several already back-fused sequences in one launch.
 template <typename SequenceSelector, typename... Seqs> void launch_divergent(void* stream, const Seqs&... seqs) {
     using D = fkd::Divergent<typename Seqs::Fused::Chain...>;
+    static_assert(sizeof(typename D::Params) <= size_t(FKLHIP_MAX_BLOB_BYTES),
+                  "the sequences' parameters together exceed FKLHIP_MAX_BLOB_BYTES (1 MiB of by-value kernel arguments)");
     typename D::Params p{};
     uint w = 0, h = 0, z = 0;
     auto fill = [&](auto& self, auto& node, const auto& first, const auto&... rest) -> void {

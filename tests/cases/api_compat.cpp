@@ -285,3 +285,12 @@ constexpr auto twoImages = fk::DualSourceRead<fk::ND::_2D, float>::build(fk::Dua
     fk::RawPtr<fk::ND::_2D, float>{nullptr, {8, 8, 32}}, fk::RawPtr<fk::ND::_2D, float>{nullptr, {8, 8, 32}}});
 constexpr auto summed = twoImages.then(fk::Add<float, float, float, fk::UnaryType>::build()).then(fk::Mul<float>::build(0.5f));
 static_assert(fk::opIs<fk::ReadType, decltype(summed)>, "the two-input form fuses onto the read of two images");
+
+// ---- A batch whose parameters would not fit the by-value kernel arguments: tests/test_abi.py compiles this file once more
+// with FK_API_COMPAT_HUGE_BATCH and expects the static_assert that names FKLHIP_MAX_BLOB_BYTES (reference: every plane of a
+// BatchRead carries its own parameters, FK/core/execution_model/operation_model/batch_operations.h:164-219) ----------
+#ifdef FK_API_COMPAT_HUGE_BATCH
+inline void launch_huge_batch(fk::Stream& s, const std::array<fk::Ptr2D<uchar3>, 45000>& in, const std::array<fk::Ptr2D<uchar3>, 45000>& out) {
+    fk::executeOperations<fk::TransformDPP<>>(s, fk::PerThreadRead<fk::ND::_2D, uchar3>::build(in), fk::PerThreadWrite<fk::ND::_2D, uchar3>::build(out));
+}
+#endif

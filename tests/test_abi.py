@@ -76,3 +76,60 @@ def test_launching_a_user_defined_operation_without_a_lowering_is_a_compile_time
                        capture_output=True, text=True)
     assert r.returncode != 0
     assert "this Operation has no MI355X lowering: specialise fk::amd::Lower<Operation>" in r.stderr
+
+
+def test_a_batch_whose_parameters_exceed_the_kernel_argument_limit_is_a_compile_time_message():
+    """The host executor bounds sizeof(Chain::Params), a compile-time constant, by FKLHIP_MAX_BLOB_BYTES: 45 000 planes of
+    24-byte pointers twice over are 2 MB of by-value kernel arguments, which stops the build with a sentence."""
+    src = os.path.join(ROOT, "tests", "cases", "api_compat.cpp")
+    r = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-DFK_API_COMPAT_HUGE_BATCH", "-I", os.path.join(ROOT, "include"), src],
+                       capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "exceed FKLHIP_MAX_BLOB_BYTES" in r.stderr and "smaller BATCH per launch" in r.stderr
+
+
+def max_blob_bytes():
+    text = open(os.path.join(ROOT, "include", "fklhip.h")).read()
+    return int(re.search(r"#define\s+FKLHIP_MAX_BLOB_BYTES\s+(\d+)", text).group(1))
+
+
+def test_a_parameter_block_above_the_limit_is_refused_before_it_reaches_the_runtime():
+    lib = fkl.lib()
+    limit = max_blob_bytes()
+    assert 64 * 1024 <= limit <= 1024 * 1024
+    sig = [s for s, _ in fkl.signatures() if s.startswith("Chain<Read2D<f32>,OpList<Add<f32,f32,f32>>,")][0]
+    h = C.c_void_p()
+    assert lib.fklhip_lookup(sig.encode(), C.byref(h)) == 0
+    blob = (C.c_char * (limit + 1))()
+    assert lib.fklhip_launch_handle(h, blob, limit + 1, None) == 10002
+    assert b"FKLHIP_MAX_BLOB_BYTES" in lib.fklhip_error_string(10002)
+    # every chain compiled into the library is far below it
+    assert max(b for _, b in fkl.signatures()) <= limit
+
+
+def test_strip_form_switch_round_trip():
+    lib = fkl.lib()
+    first = lib.fklhip_strip_form(-1)
+    assert first in (0, 1)
+    assert lib.fklhip_strip_form(0) == first and lib.fklhip_strip_form(-1) == 0
+    assert lib.fklhip_strip_form(1) == 0 and lib.fklhip_strip_form(-1) == 1
+    lib.fklhip_strip_form(first)
+
+
+def test_an_output_without_columns_launches_nothing_in_either_form():
+    """Configuration 3's chain with an active extent of 0 x 8 x 1: the strip form's grid (rows / 8 workgroups) would not be
+    empty, so the launcher must not take it; the tile form's grid has no workgroup and nothing is launched (no GPU call is
+    made, so this runs without one)."""
+    lib = fkl.lib()
+    sig, size = [(s, b) for s, b in fkl.signatures() if s.startswith("Chain<BatchRead<64,ResizeLinear<1,Crop<Read2D<Vec<u8,3>>>>>,OpList<Reorder<")][0]
+    blob = (C.c_uint32 * (size // 4))()
+    for w, h in ((0, 8), (0, 224), (8, 0)):
+        blob[0], blob[1], blob[2], blob[3] = w, h, 1, 1      # active_w, active_h, active_z, strip form allowed
+        for form in (1, 0):
+            old = lib.fklhip_strip_form(form)
+            try:
+                assert lib.fklhip_launch(sig.encode(), blob, size, None) == 0
+            finally:
+                lib.fklhip_strip_form(old)
+            ll = fkl.last_launch()
+            assert ll["grid"][0] * ll["grid"][1] * ll["grid"][2] == 0, ll

@@ -1,15 +1,13 @@
 """The strip form of the bilinear kernel (narrow planar outputs: a workgroup owns 8 whole rows of a plane, half a wave
-one row) against the oracle and against the tile form on the same inputs.  FKLHIP_STRIP=0 switches the strip form off at
-the next launch, so one process runs both."""
-import os
-
+one row) against the oracle and against the tile form on the same inputs.  fklhip_strip_form(0) switches the strip form
+off for the launches that follow, so one process runs both."""
 import numpy as np
 import pytest
 
 import fkl_cases as cases
 import oracle_lib as ol
 import workloads as wl
-from fusedkernellibrary_amd import last_launch
+from fusedkernellibrary_amd import last_launch, lib
 
 pytestmark = pytest.mark.gpu
 
@@ -22,17 +20,13 @@ def device():
 
 class strip_switched:
     def __init__(self, on):
-        self.value = "1" if on else "0"
+        self.value = 1 if on else 0
 
     def __enter__(self):
-        self.old = os.environ.get("FKLHIP_STRIP")
-        os.environ["FKLHIP_STRIP"] = self.value
+        self.old = lib().fklhip_strip_form(self.value)
 
     def __exit__(self, *exc):
-        if self.old is None:
-            os.environ.pop("FKLHIP_STRIP", None)
-        else:
-            os.environ["FKLHIP_STRIP"] = self.old
+        lib().fklhip_strip_form(self.old)
 
 
 def _c3(src, rects, dst, sub, div, device):

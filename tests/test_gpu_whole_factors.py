@@ -44,15 +44,15 @@ def test_normalise_batch_with_whole_and_fractional_planes(device):
     want = ol.oracle_crop_resize_norm_split(src, rects, (dw, dh), sub, div)
     # a 32-pixel-wide planar output goes to the strip form of the kernel (which always blends four taps); with that form
     # switched off the tile form runs, whose waves pick the one-tap path plane by plane
-    import os
-    for form, kernel in (("1", "strip"), ("0", "gather")):
-        os.environ["FKLHIP_STRIP"] = form
+    from fusedkernellibrary_amd import lib
+    for form, kernel in ((1, "strip"), (0, "gather")):
+        old = lib().fklhip_strip_form(form)
         try:
             out = torch.zeros((64, 3, dh, dw), dtype=torch.float32, device=device)
             cases.crop_resize_norm_split(_dev(src, device), rects, (dw, dh), sub, div, out)
             torch.cuda.synchronize()
         finally:
-            del os.environ["FKLHIP_STRIP"]
+            lib().fklhip_strip_form(old)
         assert last_launch()["kernel"] == kernel
         assert out.cpu().numpy().tobytes() == want.tobytes()
     # a 1x plane is the crop itself, channels swapped, normalised
