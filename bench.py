@@ -108,8 +108,8 @@ def main():
     only = set(filter(None, args.only.split(","))) or {"c1", "c2", "c3", "c4", "c5", "ext"}
     results = {}
 
-    def record(name, out_px, alg_bytes, fn, steps, warmup):
-        wall_ms, dev_ms = timer.run(fn, steps, warmup)
+    def record(name, out_px, alg_bytes, fn, steps, warmup, best_of=1):
+        wall_ms, dev_ms = min((timer.run(fn, steps, warmup) for _ in range(best_of)), key=lambda t: t[1])
         ll = fkl.last_launch()
         results[name] = {
             "mpix_per_s": out_px / 1e6 / (wall_ms * 1e-3),
@@ -150,14 +150,30 @@ def main():
         c = wl.config2()
         s = torch.from_numpy(c["src"]).to(dev)
         o = torch.zeros_like(s)
-        for n in c["n_ops"]:
+        for n in c["n_ops_sweep"]:
+            # (best of three batches each: the crossover below compares launches that differ by a few percent)
             record(f"c2_n{n}", 3840 * 2160, 2 * 3840 * 2160 * 4, lambda n=n: cases.add_mul_chain(s, n, c["add"], c["mul"], o),
-                   args.steps, args.warmup)
+                   args.steps, args.warmup, best_of=3)
             if n >= 50:
                 # n dependent fp32 instructions per element that no contraction or packing may merge: 8.3 M elements are
                 # 129 600 wave-wide elements, at the 2.45 cycles per instruction and SIMD this chip was measured to issue
                 results[f"c2_n{n}"]["valu_issue_floor_us"] = 129600 * n * 2.45 / 1024 / 2.3e3
-        record("copy_f32_4k", 3840 * 2160, 2 * 3840 * 2160 * 4, lambda: cases.copy_f32(s, o), args.steps, args.warmup)
+        record("copy_f32_4k", 3840 * 2160, 2 * 3840 * 2160 * 4, lambda: cases.copy_f32(s, o), args.steps, args.warmup, best_of=3)
+        # Where instruction issue takes over from bandwidth (the sweep of the reference's instruction-count benchmark,
+        # benchmarks/numinstructions/benchmark_numinstructions_x_operation.h:33-43): the first N of the sweep whose launch
+        # takes 5 % longer than the plain copy of the same image, the straight line through the launches beyond it
+        # (what a launch costs whatever its length + what one more operation costs), and the N at which that line meets
+        # the copy's duration.
+        copy_us = results["copy_f32_4k"]["kernel_us"]
+        sweep = [(n, results[f"c2_n{n}"]["kernel_us"]) for n in c["n_ops_sweep"]]
+        beyond = [(n, us) for n, us in sweep if us > 1.05 * copy_us]
+        cross = {"copy_us": copy_us, "sweep_n": [n for n, _ in sweep], "sweep_us": [us for _, us in sweep],
+                 "first_n_5_percent_above_copy": beyond[0][0] if beyond else None}
+        if len(beyond) >= 2:
+            per_op, fixed = np.polyfit(np.array([n for n, _ in beyond], np.float64), np.array([us for _, us in beyond]), 1)
+            cross.update({"fit_through_n": [n for n, _ in beyond], "fixed_us": float(fixed), "per_op_us": float(per_op),
+                          "line_meets_copy_at_n": float((copy_us - fixed) / per_op)})
+        results["c2_crossover"] = cross
     if "c5" in only:
         c = wl.config5()
         s = torch.from_numpy(c["nv12"]).to(dev)
@@ -226,6 +242,19 @@ def main():
         record("u8x3_to_three_float_planes_1080p", W * H, W * H * (3 + 12),
                lambda: cases.split_write(1, img.view(H, W * 3), W, H, planes, None, (1 / 255.0, 1 / 255.0, 1 / 255.0, 0)), args.steps, args.warmup)
         del fo, po, uyvy, nv12, t4, d4, frames, img2, mean, planes
+        # the same four chains at 3840 x 2160, where the launch floor is a smaller part of a launch
+        W, H = 3840, 2160
+        img4k = torch.from_numpy(rng.randint(0, 256, (H, W, 3)).astype(np.uint8)).to(dev)
+        fo = torch.zeros((H, W, 3), dtype=torch.float32, device=dev)
+        affine4k = [[math.cos(th), -math.sin(th), 80.0], [math.sin(th), math.cos(th), -120.0]]
+        record("warp_affine_2160p_u8x3", W * H, W * H * (3 + 12), lambda: cases.warp(img4k, affine4k, False, (W, H), fo), args.steps, args.warmup)
+        record("deinterlace_blend_2160p_u8x3", W * H, W * H * (3 + 12), lambda: cases.deinterlace(img4k, 1, fo), args.steps, args.warmup)
+        uyvy = torch.from_numpy(rng.randint(0, 256, (H, 2 * W)).astype(np.uint8)).to(dev)
+        record("uyvy_to_rgb_full709_2160p", W * H, W * H * (2 + 12), lambda: cases.yuv_to_rgb(10, 1, 1, uyvy, W, H, fo), args.steps, args.warmup)
+        po = torch.zeros((H + 32, W + 32, 3), dtype=torch.uint8, device=dev)
+        record("pad_reflect101_16px_2160p_u8x3", (W + 32) * (H + 32), W * H * 3 + (W + 32) * (H + 32) * 3,
+               lambda: cases.pad(img4k, 4, 16, 16, po), args.steps, args.warmup)
+        del img4k, fo, uyvy, po
 
     # ---- configuration 3, the headline: W warm-up steps, then exactly K timed steps ---------------------------------
     r3 = record("c3", 64 * 224 * 224, a3, f3, args.steps, args.warmup)
@@ -233,10 +262,44 @@ def main():
     # the same K steps four more times, for the spread (not used for `value`)
     again = [timer.run(f3, args.steps, args.warmup)[1] * 1e3 for _ in range(4)] + [r3["kernel_us"]]
     r3["kernel_us_5_runs_min_mean_max"] = [min(again), sum(again) / len(again), max(again)]
+    # The same K steps recorded once into a HIP graph (kernel nodes only: the launch path allocates nothing and records no
+    # memset) and replayed: what the steps cost when the host issues one graph launch instead of K kernel launches.
+    graph = torch.cuda.CUDAGraph()
+    cases.set_reps(args.steps)
+    with torch.cuda.graph(graph):
+        f3()
+    torch.cuda.synchronize()
+    graph_runs = []
+    for _ in range(5):
+        graph.replay()                                   # warm-up replay
+        torch.cuda.synchronize()
+        time.sleep(0.03)
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        t0 = time.perf_counter()
+        fkl.check(timer.lib.fklhip_event_record(timer.e0, stream), "event_record")
+        graph.replay()
+        fkl.check(timer.lib.fklhip_event_record(timer.e1, stream), "event_record")
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / args.steps
+        ms = C.c_float()
+        fkl.check(timer.lib.fklhip_event_elapsed_ms(C.byref(ms), timer.e0, timer.e1), "event_elapsed")
+        graph_runs.append((wall, ms.value / args.steps))
+    if out3.cpu().numpy().tobytes() != got3.tobytes():
+        print("bench.py: the graph replay's output differs from the eager launches'", file=sys.stderr)
+        sys.exit(3)
+    r3["graph_replay"] = {"ms_per_step_graph": min(w for w, _ in graph_runs), "kernel_us_graph": min(d for _, d in graph_runs) * 1e3,
+                          "runs_wall_ms_per_step": [w for w, _ in graph_runs], "runs_kernel_us": [d * 1e3 for _, d in graph_runs],
+                          "note": "K steps captured once into a HIP graph of K kernel nodes, one replay timed (wall clock around replay + "
+                                  "synchronise, events around the replay); best of 5"}
+    del graph
     # and one long batch: what a launch costs once the first launches after the idle state are a small part of the batch
     # (the second of two such batches: the first also pays for the launch queue's and the runtime's argument buffers growing)
     timer.run(f3, 1000, 300, settle=0)
-    r3["kernel_us_1000_launches"] = timer.run(f3, 1000, 0, settle=0)[1] * 1e3
+    long_wall_ms, long_dev_ms = timer.run(f3, 1000, 0, settle=0)
+    r3["kernel_us_1000_launches"] = long_dev_ms * 1e3
+    # wall clock per step of the same batch: the one synchronisation at the end of a timed region (10 - 20 us) is then a
+    # thousandth of a step instead of a twentieth
+    r3["ms_per_step_1000_launches"] = long_wall_ms
     # the same 64 crops to planes of twice the rows (224 x 448): what a launch costs that does not depend on its size, and what
     # 38.5 MB more of output cost once the kernel runs (the source bytes are the same, so they count for nothing here)
     out3x2 = torch.zeros((64, 3, 448, 224), dtype=torch.float32, device=dev)
@@ -299,7 +362,8 @@ def main():
                      "kernel_us_5_runs_min_mean_max": r3["kernel_us_5_runs_min_mean_max"],
                      "kernel_us_1000_launches": r3["kernel_us_1000_launches"],
                      "frac_1000_launches": a3 / (r3["kernel_us_1000_launches"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                     "twice_the_rows": r3["twice_the_rows"]},
+                     "ms_per_step_1000_launches": r3["ms_per_step_1000_launches"],
+                     "twice_the_rows": r3["twice_the_rows"], "graph_replay": r3["graph_replay"]},
         "cpu_baseline": cpu,
         "others": {k: v for k, v in results.items() if k != "c3"},
     }

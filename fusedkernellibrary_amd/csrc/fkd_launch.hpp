@@ -29,12 +29,22 @@ template <class Chain, int V, int ROWS>
 hipError_t launch_rows_with(const typename Chain::Params& p, hipStream_t stream, LaunchInfo* info, bool aligned) {
     const unsigned gx = (p.active_w + kRowsBX * V - 1) / (kRowsBX * V);
     const unsigned gy = (p.active_h + kRowsBY * ROWS - 1) / (kRowsBY * ROWS);
-    const dim3 grid(gx, gy, p.active_z), block(kRowsBX, kRowsBY, 1);
+    dim3 grid(gx, gy, p.active_z);
+    const dim3 block(kRowsBX, kRowsBY, 1);
+    TileGeom g{0u, 0u, 0u, 0u};
+    if constexpr (rows_in_bands<Chain>()) {
+        // gathering reads, larger launches: a one-dimensional grid whose workgroups the kernel renumbers into one band per XCD
+        if ((unsigned long long)gx * gy > 0x7fffff00ull) return hipErrorInvalidConfiguration;
+        if (gx * gy >= kRowsBandBlocks) {
+            grid = dim3(rows_band_chunk(gx * gy) * 8u, 1, p.active_z);
+            g = TileGeom{gx, gy, gx * gy * p.active_z, division_magic(gx, gx * gy)};
+        }
+    }
     if (info) *info = LaunchInfo{aligned_name(aligned), {grid.x, grid.y, grid.z}, {block.x, block.y, 1}, 0};
     if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
     if (grid.y > 65535u || grid.z > 65535u) return hipErrorInvalidConfiguration;
-    if (aligned) return launch_by_pointer(&k_rows<Chain, V, ROWS, true>, grid, block, stream, p);
-    return launch_by_pointer(&k_rows<Chain, V, ROWS, false>, grid, block, stream, p);
+    if (aligned) return launch_by_pointer(&k_rows<Chain, V, ROWS, true>, grid, block, stream, p, g);
+    return launch_by_pointer(&k_rows<Chain, V, ROWS, false>, grid, block, stream, p, g);
 }
 
 template <class Chain>

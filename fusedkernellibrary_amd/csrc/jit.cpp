@@ -35,13 +35,14 @@
 namespace fklhip {
 namespace {
 
-// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): nine and four 32-bit words.
+// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): ten and four 32-bit words.
 struct JitMeta {
-    unsigned gather, params_bytes, v, rows, xi, yi, by, max_planes, strip_width;
+    unsigned gather, params_bytes, v, rows, xi, yi, by, max_planes, strip_width, bands;
 };
 struct TileGeom {
     unsigned tiles_x, tiles_y, n_tiles, tiles_x_magic;
 };
+constexpr unsigned kRowsBandBlocks = 4096;     // as fkd::kRowsBandBlocks
 // As fkd::division_magic: floor(2^32 / d) + 1 when it divides every number below `limit` exactly, else 0.
 unsigned division_magic(unsigned d, unsigned limit) {
     if (d == 0) return 0;
@@ -234,6 +235,16 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
         grid[0] = (active[0] + 64 * m.v - 1) / (64 * m.v);
         grid[1] = (active[1] + 4 * m.rows - 1) / (4 * m.rows);
         grid[2] = active[2];
+        if (m.bands && (unsigned long long)grid[0] * grid[1] >= kRowsBandBlocks) {
+            // as launch_rows_with: one-dimensional, eight equal runs of the plane's blocks
+            if ((unsigned long long)grid[0] * grid[1] > 0x7fffff00ull) return int(hipErrorInvalidConfiguration);
+            g.tiles_x = grid[0];
+            g.tiles_y = grid[1];
+            g.n_tiles = grid[0] * grid[1] * grid[2];
+            g.tiles_x_magic = division_magic(g.tiles_x, g.tiles_x * g.tiles_y);
+            grid[0] = (grid[0] * grid[1] + 7u) / 8u * 8u;
+            grid[1] = 1;
+        }
     }
     if (info) *info = fkd::LaunchInfo{kind, {grid[0], grid[1], grid[2]}, {block[0], block[1], 1}, 0};
     if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return FKLHIP_OK;

@@ -288,6 +288,9 @@ int fklref_add_mul_chain(const float* in, int w, int h, int pitch, int n_ops, fl
     case 2: return add_mul_n<2>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
     case 3: return add_mul_n<3>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
     case 10: return add_mul_n<10>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 20: return add_mul_n<20>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 30: return add_mul_n<30>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
+    case 40: return add_mul_n<40>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
     case 50: return add_mul_n<50>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
     case 100: return add_mul_n<100>(in, w, h, pitch, addv, mulv, out, out_pitch, tf);
     default: return 1;

@@ -261,6 +261,9 @@ int fklcase_add_mul_chain(void* stream, const float* in, int w, int h, int pitch
         case 2: add_mul_n<2>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
         case 3: add_mul_n<3>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
         case 10: add_mul_n<10>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 20: add_mul_n<20>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 30: add_mul_n<30>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
+        case 40: add_mul_n<40>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
         case 50: add_mul_n<50>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
         case 100: add_mul_n<100>(stream, in, w, h, pitch, addv, mulv, out, out_pitch, tf); break;
         default: throw std::runtime_error("add_mul_chain: unsupported operation count");

@@ -68,7 +68,7 @@ def main():
     out["c1_full"] = r   # 122 880 bytes: small enough to keep whole
     digests["c1_full"] = sha(r)
     c = wl.config2()
-    for n in c["n_ops"]:
+    for n in c["n_ops_sweep"]:
         r = ol.ref_add_mul_chain(c["src"], n, c["add"], c["mul"])
         assert sha(r) == sha(ol.oracle_add_mul_chain(c["src"], n, c["add"], c["mul"]))
         digests[f"c2_full_n{n}"] = sha(r)

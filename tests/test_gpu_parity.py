@@ -123,7 +123,7 @@ def test_config1_reduced(device):
 
 # ---- configuration 2: pure vertical fusion ----------------------------------------------------------------------
 
-@pytest.mark.parametrize("n", [1, 10, 50, 100])
+@pytest.mark.parametrize("n", [1, 10, 20, 30, 40, 50, 100])
 def test_config2_full_size(device, n):
     c = wl.config2()
     got = run_c2(c, n, device)

@@ -128,3 +128,17 @@ def test_a_chain_that_would_need_scratch_memory_is_compiled_again_or_refused(dev
     env["FKLHIP_JIT_STRICT"] = "1"
     r = subprocess.run([sys.executable, "-c", _CACHE_SCRIPT, root, str(res)], env=env, capture_output=True, text=True, timeout=240)
     assert r.returncode != 0 and "could not be compiled at run time" in r.stderr, r.stderr[-2000:]
+
+
+def test_a_chain_whose_parameters_exceed_the_kernel_argument_limit_is_refused_with_a_sentence(device):
+    """45 000 planes of 24-byte pointers on either side are 2 MB of by-value kernel arguments: the run-time compiler
+    refuses the chain (FKLHIP_EBLOB_SIZE) and its log names the limit, instead of the launch call failing later."""
+    import ctypes as C
+    from fusedkernellibrary_amd import lib
+    sig = b"Chain<BatchRead<45000,Read2D<Vec<u8,3>>>,OpList<>,BatchWrite<45000,Write2D<Vec<u8,3>>>>"
+    h = C.c_void_p()
+    assert lib().fklhip_lookup(sig, C.byref(h)) == 10002
+    log = C.c_char_p()
+    lib().fklhip_jit_log(C.byref(log))
+    assert b"FKLHIP_MAX_BLOB_BYTES" in log.value and b"smaller batch" in log.value
+    assert sig.decode() not in [s for s, _ in signatures()]

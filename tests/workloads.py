@@ -66,7 +66,8 @@ def config1(width: int = 3840, height: int = 2160, seed: int = 1):
 def config2(width: int = 3840, height: int = 2160, seed: int = 2):
     """Pure vertical fusion: float image, N alternating Add(0.5f)/Mul(1.0001f)."""
     src = RawMT(seed).unit_floats(width * height).reshape(height, width)
-    return {"src": src, "add": np.float32(0.5), "mul": np.float32(1.0001), "n_ops": (1, 10, 50, 100)}
+    return {"src": src, "add": np.float32(0.5), "mul": np.float32(1.0001), "n_ops": (1, 10, 50, 100),
+            "n_ops_sweep": (1, 10, 20, 30, 40, 50, 100)}       # the benchmark's sweep for the instruction-vs-bandwidth crossover
 
 
 def config3_rects(batch: int = 64, width: int = 1920, height: int = 1080, seed: int = 33,
