@@ -74,25 +74,44 @@ constexpr int round_to_int(float v) {
     return v < 0.f ? -r : r;
 }
 
-template <AspectRatio AR> constexpr Size target_size(const Size& srcSize, const Size& dstSize) {
-    const float scaleFactor = dstSize.height / (float)srcSize.height;
-    const int targetHeight = dstSize.height;
-    const int targetWidth = round_to_int(scaleFactor * srcSize.width);
-    if constexpr (AR == AspectRatio::PRESERVE_AR_RN_EVEN) {
-        const int evenWidth = targetWidth - (targetWidth % 2);
-        if (evenWidth > dstSize.width) {
-            const float scaleW = dstSize.width / (float)srcSize.width;
-            const int h = round_to_int(scaleW * srcSize.height);
-            return Size(dstSize.width, h - (h % 2));
-        }
-        return Size(evenWidth, targetHeight);
-    } else {
-        if (targetWidth > dstSize.width) {
-            const float scaleW = dstSize.width / (float)srcSize.width;
-            return Size(dstSize.width, round_to_int(scaleW * srcSize.height));
-        }
-        return Size(targetWidth, targetHeight);
-    }
+// Size of the resized image on a canvas when the aspect ratio is kept: the source is fitted to the canvas height, and to
+// the canvas width instead if that comes out wider than the canvas.  Scale factors and products are single precision, the
+// rounding is half away from zero; PRESERVE_AR_RN_EVEN then takes the even number at or below the rounded side.
+template <AspectRatio AR> constexpr Size target_size(const Size& source, const Size& canvas) {
+    constexpr bool kEven = AR == AspectRatio::PRESERVE_AR_RN_EVEN;
+    auto even_floor = [](int v) { return kEven ? v - (v % 2) : v; };
+    // the free side of an image scaled so that `fitted` source pixels become `to` output pixels
+    auto free_side = [](int to, int fitted, int other) { return round_to_int((to / static_cast<float>(fitted)) * other); };
+    const int width_by_height = even_floor(free_side(canvas.height, source.height, source.width));
+    if (width_by_height <= canvas.width) return Size(width_by_height, canvas.height);
+    return Size(canvas.width, even_floor(free_side(canvas.width, source.width, source.height)));
+}
+
+// How far the source advances per output pixel along one axis: the single-precision value of 1 / (outputs / inputs),
+// both divisions in double, which is the rounding the device's coordinates are checked against.
+constexpr float source_step(int outputs, int inputs) {
+    const double enlargement = static_cast<double>(outputs) / static_cast<double>(inputs);
+    return static_cast<float>(1.0 / enlargement);
+}
+
+// Where the resized image sits on the output canvas: its size under the aspect-ratio mode and its first column and row
+// (centred, halves truncated; PRESERVE_AR_LEFT pins it to column 0).
+struct Letterbox {
+    Size image;
+    int left, top;
+    constexpr int right() const { return left + image.width - 1; }
+    constexpr int bottom() const { return top + image.height - 1; }
+};
+template <AspectRatio AR> constexpr Letterbox place_on_canvas(const Size& source, const Size& canvas) {
+    const Size image = target_size<AR>(source, canvas);
+    const int left = AR == AspectRatio::PRESERVE_AR_LEFT ? 0 : (canvas.width - image.width) / 2;
+    return Letterbox{image, left, (canvas.height - image.height) / 2};
+}
+
+// The extent of whatever a complete read IOp delivers.
+template <typename ReadIOp> constexpr Size extent_of(const ReadIOp& read) {
+    static_assert(isCompleteOperation<ReadIOp>, "a Resize can only be completed against a complete read IOp (one that knows its source)");
+    return NumElems::size(Point{0, 0, 0}, read);
 }
 } // namespace resize_detail
 
@@ -116,31 +135,26 @@ struct Resize : IncompleteReadBackOperation<NullType, IncompleteResizeParams<AR,
         return Resize<IType, AR, DefaultType_>::build(IncompleteResizeParams<AR, DefaultType_>{dstSize, backgroundValue}, NullType{});
     }
 
-    // Completion against the read behind it.
-    template <typename NewBackIOp, std::enable_if_t<isOperation<NewBackIOp>, int> = 0>
-    static constexpr auto build(const NewBackIOp& backIOp, const InstantiableType& iOp) {
-        static_assert(isCompleteOperation<NewBackIOp>, "NewBackIOp must be a complete IOp");
-        using NewDefaultType = float_<cn<typename NewBackIOp::Operation::OutputType>>;
-        static_assert(std::is_same_v<NewDefaultType, DefaultType>, "Default value type and Op::OutputType must be the same.");
-        return build(backIOp, iOp.params.dstSize, iOp.params.defaultValue);
+    // Completion of the incomplete IOp against the read it was fused onto.
+    template <typename SourceIOp, std::enable_if_t<isOperation<SourceIOp>, int> = 0>
+    static constexpr auto build(const SourceIOp& source, const InstantiableType& pending) {
+        static_assert(std::is_same_v<float_<cn<typename SourceIOp::Operation::OutputType>>, DefaultType>,
+                      "the background value of a letterboxing Resize must be the float vector with the channel count of the pixels it reads");
+        return build(source, pending.params.dstSize, pending.params.defaultValue);
     }
 
-    template <typename NewBackIOp, std::enable_if_t<isOperation<NewBackIOp>, int> = 0>
-    static constexpr auto build(const NewBackIOp& backIOp, const Size& dstSize,
-                                const VectorType_t<float, cn<typename NewBackIOp::Operation::OutputType>>& backgroundValue) {
-        static_assert(isCompleteOperation<NewBackIOp>, "NewBackIOp must be a complete IOp");
-        const Size srcSize = NumElems::size(Point{0, 0, 0}, backIOp);
-        const Size targetSize = resize_detail::target_size<AR>(srcSize, dstSize);
-        const double cfx = static_cast<double>(targetSize.width) / srcSize.width;
-        const double cfy = static_cast<double>(targetSize.height) / srcSize.height;
-        using NewOutputType = float_<cn<typename NewBackIOp::Operation::OutputType>>;
-        const int x1 = AR == AspectRatio::PRESERVE_AR_LEFT ? 0 : static_cast<int>((dstSize.width - targetSize.width) / 2);
-        const int y1 = static_cast<int>((dstSize.height - targetSize.height) / 2);
-        const ResizeParams<AR, NewOutputType> resizeParams{dstSize,
-                                                           {static_cast<float>(1.0 / cfx), static_cast<float>(1.0 / cfy)},
-                                                           x1, y1, x1 + targetSize.width - 1, y1 + targetSize.height - 1,
-                                                           backgroundValue};
-        return NewInstantiableType<NewBackIOp>::build(resizeParams, Interpolate<IType>::build(backIOp));
+    // Complete in one call: the letterbox is placed on the canvas, the band around it takes the background value.
+    template <typename SourceIOp, std::enable_if_t<isOperation<SourceIOp>, int> = 0>
+    static constexpr auto build(const SourceIOp& source, const Size& canvas,
+                                const VectorType_t<float, cn<typename SourceIOp::Operation::OutputType>>& background) {
+        using Pixel = float_<cn<typename SourceIOp::Operation::OutputType>>;
+        const Size from = resize_detail::extent_of(source);
+        const resize_detail::Letterbox box = resize_detail::place_on_canvas<AR>(from, canvas);
+        return NewInstantiableType<SourceIOp>::build(
+            ResizeParams<AR, Pixel>{canvas,
+                                    {resize_detail::source_step(box.image.width, from.width), resize_detail::source_step(box.image.height, from.height)},
+                                    box.left, box.top, box.right(), box.bottom(), background},
+            Interpolate<IType>::build(source));
     }
 };
 
@@ -161,20 +175,20 @@ template <> struct Resize<InterpolationType::INTER_LINEAR, AspectRatio::IGNORE_A
     using Parent::build;
     static constexpr auto build(const Size& dstSize) { return InstantiableType{{ParamsType{dstSize}, BackIOp{}}}; }
 
-    template <typename NewBackIOp, std::enable_if_t<isOperation<NewBackIOp>, int> = 0>
-    static constexpr auto build(const NewBackIOp& backIOp, const Size& dstSize) {
-        static_assert(isCompleteOperation<NewBackIOp>, "NewBackIOp must be a complete IOp");
-        const Size srcSize = NumElems::size(Point{0, 0, 0}, backIOp);
-        const double cfx = static_cast<double>(dstSize.width) / static_cast<double>(srcSize.width);
-        const double cfy = static_cast<double>(dstSize.height) / static_cast<double>(srcSize.height);
-        const typename NewInstantiableType<NewBackIOp>::ParamsType resizeParams{
-            dstSize, {static_cast<float>(1.0 / cfx), static_cast<float>(1.0 / cfy)}};
-        return NewInstantiableType<NewBackIOp>::build(resizeParams, Interpolate<IType>::build(backIOp));
+    // The whole source stretched over the whole output.
+    template <typename SourceIOp, std::enable_if_t<isOperation<SourceIOp>, int> = 0>
+    static constexpr auto build(const SourceIOp& source, const Size& outputSize) {
+        const Size from = resize_detail::extent_of(source);
+        using Completed = NewInstantiableType<SourceIOp>;
+        return Completed::build(
+            typename Completed::ParamsType{outputSize, {resize_detail::source_step(outputSize.width, from.width),
+                                                        resize_detail::source_step(outputSize.height, from.height)}},
+            Interpolate<IType>::build(source));
     }
 
-    template <typename NewBackIOp, std::enable_if_t<isOperation<NewBackIOp>, int> = 0>
-    static constexpr auto build(const NewBackIOp& backIOp, const InstantiableType& selfIOp) {
-        return build(backIOp, selfIOp.params.dstSize);
+    template <typename SourceIOp, std::enable_if_t<isOperation<SourceIOp>, int> = 0>
+    static constexpr auto build(const SourceIOp& source, const InstantiableType& pending) {
+        return build(source, pending.params.dstSize);
     }
 
     // Resize straight from a pointer: destination size, or scale factors when the size is empty.
