@@ -357,7 +357,7 @@ def main():
                    "output_pixels_per_step": 64 * 224 * 224, "union_source_pixels": union_px,
                    "sum_of_crop_areas_bytes": int(sum(int(r[2]) * int(r[3]) for r in c3["rects"])) * 3},
         "roofline": {"bound": "hbm", "achieved": r3["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": r3["frac_of_hbm_peak"], "traffic": TRAFFIC_C3_BYTES,
+                     "frac": r3["frac_of_hbm_peak"], "traffic": traffic_c3()[0], "traffic_note": traffic_c3()[1],
                      "algorithmic_bytes": a3, "kernel_us": r3["kernel_us"], "kernel": "fkd::k_" + r3["kernel"],
                      "kernel_us_5_runs_min_mean_max": r3["kernel_us_5_runs_min_mean_max"],
                      "kernel_us_1000_launches": r3["kernel_us_1000_launches"],
@@ -371,9 +371,32 @@ def main():
 
 
 # HBM bytes one launch of configuration 3 moves: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this script, scaled by what the
-# same counters read for its plain copy chain of known size.  Measured once, not in this run (the counters need the
-# profiler attached): profiles/k_strip_config3.txt holds the commands and the readings (run of 2026-11-25, fkd::k_strip).
-TRAFFIC_C3_BYTES = 52599000
+# same counters read for its plain copy chain of known size.  Measured under the profiler, not in this run (the counters
+# need it attached): profiles/k_strip_config3.txt holds the commands and the readings.  The figure belongs to the kernel
+# sources it was measured on: their digest is kept beside it, and a run on other sources reports no traffic figure rather
+# than a stale one.
+TRAFFIC_C3_BYTES = 52058000
+TRAFFIC_C3_SOURCES = ("fusedkernellibrary_amd/csrc/fkd_kernels.hpp", "fusedkernellibrary_amd/csrc/fkd_launch.hpp",
+                      "include/fkd/ops.hpp", "include/fkd/types.hpp")
+TRAFFIC_C3_SOURCES_SHA256 = "9dbd5965dcd4e5016b6575c398e291308713d9dff6254e6323de5078da10cbff"
+
+
+def device_sources_sha256():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in TRAFFIC_C3_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def traffic_c3():
+    """(bytes, note): the measured figure while the kernel sources are the ones it was measured on, else (None, why)."""
+    now = device_sources_sha256()
+    if now == TRAFFIC_C3_SOURCES_SHA256:
+        return TRAFFIC_C3_BYTES, "rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated (profiles/k_strip_config3.txt)"
+    return None, ("the kernel sources changed since the counters were read (" + now[:16] + " now, " + TRAFFIC_C3_SOURCES_SHA256[:16] +
+                  " then): re-measure as in profiles/k_strip_config3.txt")
 
 if __name__ == "__main__":
     main()

@@ -362,6 +362,25 @@ int fklcase_set_to_shapes(void* stream_, int w, int h, int planes, const uint8_t
     });
 }
 
+// setTo on a transposed tensor (ND::T3D) of `planes` images with `color_planes` channel planes each, filled with a
+// sentinel first: host_tensor receives color_planes * planes * h * w floats, as they lie in memory.
+int fklcase_set_to_transposed(void* stream_, int w, int h, int planes, int color_planes, float sentinel, float value, float* host_tensor) {
+    return guarded([&] {
+        Stream stream(stream_);
+        TensorT<float> t(uint(w), uint(h), uint(planes), uint(color_planes), MemType::DeviceAndPinned);
+        const size_t n = size_t(w) * size_t(h) * size_t(planes) * size_t(color_planes);
+        float* mirror = t.ptrPinned().data;
+        for (size_t i = 0; i < n; ++i) mirror[i] = sentinel;
+        t.upload(stream);
+        stream.sync();
+        setTo(value, t, stream);
+        for (size_t i = 0; i < n; ++i) mirror[i] = sentinel;      // setTo filled the mirror too: only the device copy is checked
+        t.download(stream);
+        stream.sync();
+        std::memcpy(host_tensor, t.ptrPinned().data, n * sizeof(float));
+    });
+}
+
 // Chains that are NOT in the ahead-of-time list: the library compiles them when it first sees them.
 int fklcase_uncompiled_pointwise_f32(void* stream_, const float* in, int w, int h, int pitch, float* out, int out_pitch) {
     return guarded([&] {

@@ -183,6 +183,14 @@ def set_and_loop_f32(n, init, add, iterations):
     return out
 
 
+def set_to_transposed(w, h, planes, color_planes, sentinel, value):
+    """setTo on a TensorT<float> that held `sentinel` everywhere; returns the device copy, (color_planes * planes, h, w) f32."""
+    out = np.zeros((color_planes * planes, h, w), np.float32)
+    _ok(cases().fklcase_set_to_transposed(_stream(), int(w), int(h), int(planes), int(color_planes), C.c_float(float(sentinel)),
+                                          C.c_float(float(value)), out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
 def set_to_shapes(w, h, planes, v3, vf):
     """setTo on a pitched (h,w) uchar3 image and a (planes,h,w) float tensor; returns (image rows incl. pitch, pitch, tensor)."""
     img = np.zeros(h * (w * 3 + 1024), np.uint8)

@@ -27,3 +27,11 @@ def test_set_to_pitched_image_and_tensor(device):
     px = img[:, : w * 3].reshape(h, w, 3)
     assert (px == np.array([7, 200, 33], np.uint8)).all()
     assert (ten == np.float32(-2.5)).all() and ten.shape == (planes, h, w)
+
+
+def test_set_to_fills_every_colour_plane_of_a_transposed_tensor(device):
+    """Documented difference: the reference's setTo on an ND::T3D Ptr goes through PerThreadWrite<T3D>, which addresses
+    colour plane 0 only and leaves the other colour planes as they were (FK/core/data/ptr_utils.h:24-45,
+    FK/core/data/rawptr.h:228-240); here every element of the Ptr takes the value, as for the other dimensionalities."""
+    got = cases.set_to_transposed(21, 5, 4, 3, sentinel=-99.0, value=6.25)
+    assert got.shape == (12, 5, 21) and (got == np.float32(6.25)).all()
