@@ -192,7 +192,15 @@ def main():
         add = np.stack([p.range_floats(3, -64.0, 64.0) for _ in range(100)])
         record("c4", 100 * 1920 * 1080, 2 * 100 * 1920 * 1080 * 3, lambda: cases.batch_muladd_sat(srcs, mul, add, outs),
                max(10, args.steps // 10), max(2, args.warmup // 10))
-        results["c4"]["note"] = "inputs: uniform random bytes made on the GPU (timing only; parity of this configuration is tests/test_gpu_parity.py)"
+        # this run's own check of what it timed: every plane against the same arithmetic done by torch on the GPU (one
+        # multiplication, one addition, round half to even, clamp: each rounded once, as the chain's operations are)
+        for i in range(100):
+            m, a = torch.from_numpy(mul[i]).to(dev), torch.from_numpy(add[i]).to(dev)
+            if not torch.equal(outs[i], torch.clamp(torch.round(srcs[i].to(torch.float32) * m + a), 0, 255).to(torch.uint8)):
+                print(f"bench.py: configuration 4, image {i}: the output differs from mul, add, round-half-even, clamp", file=sys.stderr)
+                sys.exit(3)
+        results["c4"]["note"] = ("inputs: uniform random bytes made on the GPU; all 100 outputs of this run checked bit for bit against the same "
+                                 "arithmetic in torch (the seeded inputs and the reference's digests: tests/test_gpu_parity.py)")
 
         del srcs, outs
 
