@@ -80,6 +80,22 @@ def test_yuv_resize(device, pf):
         assert out.cpu().numpy().tobytes() == ol.oracle_yuv_resize(pf, buf, w, h, dst, 0.5).tobytes(), dst
 
 
+def test_yuv_resize_to_a_large_image_runs_in_bands(device):
+    """A bilinear read that takes its taps one element at a time runs on the rows kernel, one element per thread; from 4 096
+    workgroups per plane up its launch takes the one-dimensional grid whose workgroups are renumbered into one band per XCD."""
+    import torch
+    from fusedkernellibrary_amd import last_launch
+    pf, w, h, dst = ol.PF_UYVY, 320, 180, (1030, 1021)
+    buf = frame(pf, w, h, 1234)
+    out = torch.zeros((dst[1], dst[0], 3), dtype=torch.float32, device=device)
+    cases.yuv_resize(pf, to_dev(buf, device), w, h, dst, 0.5, out)
+    torch.cuda.synchronize()
+    ll = last_launch()
+    blocks = ((dst[0] + 63) // 64) * ((dst[1] + 3) // 4)
+    assert blocks >= 4096 and ll["kernel"].startswith("rows") and ll["grid"] == [(blocks + 7) // 8 * 8, 1, 1], ll
+    assert out.cpu().numpy().tobytes() == ol.oracle_yuv_resize(pf, buf, w, h, dst, 0.5).tobytes()
+
+
 RESIZED = [ol.PF_NV21, ol.PF_UYVY, ol.PF_P010]
 
 

@@ -43,3 +43,30 @@ def test_warp_float(device, matrix, persp):
     torch.cuda.synchronize()
     want = ol.oracle_warp(img, 1, matrix, (60, 50), persp)
     assert out.cpu().numpy().tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("persp,dst", [(False, (2048, 2052)), (True, (2051, 2049)), (False, (1024, 3000))])
+def test_large_warps_run_their_workgroups_in_one_band_per_xcd(device, persp, dst):
+    """Launches of 4 096 workgroups per plane or more take a one-dimensional grid whose workgroups the kernel renumbers
+    (one contiguous band of the output per XCD); smaller ones keep the two-dimensional grid.  Same bits either way: the
+    affine chain is compiled ahead of time, the perspective one at run time, and the odd sizes leave partial blocks
+    at the right and bottom edges and idle workgroups at the end of the grid."""
+    import torch
+    from fusedkernellibrary_amd import last_launch
+    rng = np.random.RandomState(15)
+    img = rng.randint(0, 256, (300, 417, 3)).astype(np.uint8)
+    s = 0.19
+    matrix = ([[s * math.cos(TH), -s * math.sin(TH), 60.0], [s * math.sin(TH), s * math.cos(TH), -40.0], [0.00001, -0.00002, 1.0]] if persp
+              else [[s * math.cos(TH), -s * math.sin(TH), 60.0], [s * math.sin(TH), s * math.cos(TH), -40.0]])
+    src = torch.from_numpy(img).to(device)
+    out = torch.full((dst[1], dst[0], 3), -1.0, dtype=torch.float32, device=device)
+    cases.warp(src, matrix, persp, dst, out)
+    torch.cuda.synchronize()
+    ll = last_launch()
+    blocks = ((dst[0] + 255) // 256) * ((dst[1] + 3) // 4)
+    if blocks >= 4096:
+        assert ll["grid"] == [(blocks + 7) // 8 * 8, 1, 1], ll
+    else:
+        assert ll["grid"] == [(dst[0] + 255) // 256, (dst[1] + 3) // 4, 1], ll
+    want = ol.oracle_warp(img, 3, matrix, dst, persp)
+    assert out.cpu().numpy().tobytes() == want.tobytes()
