@@ -2016,6 +2016,20 @@ template <int BT, class Back> struct Border {
     FKD_DEV static int iabs(int v) { return v < 0 ? -v : v; }
     // n = extent along the axis (last index = n - 1)
     FKD_DEV static int fold(int i, int n) {
+        // Within one image size of the image the reference's formulas below come to a single reflection or a single period,
+        // and no division is needed (a pad, a crop that leans over an edge); anything further out takes the formulas as written.
+        if constexpr (BT >= 2) {
+            const int last = n - 1;
+            int near_value;
+            bool near;
+            if constexpr (BT == 2) { near_value = i < 0 ? -i - 1 : (i > last ? 2 * last - i + 1 : i); near = i >= -n && i <= 2 * last + 1; }
+            else if constexpr (BT == 3) { near_value = i < 0 ? i + n : (i >= n ? i - n : i); near = i >= -n && i < 2 * n; }
+            else { near_value = i < 0 ? -i : (i > last ? 2 * last - i : i); near = i >= -last && i <= 2 * last; }
+            if (near) return near_value;
+        }
+        return fold_as_written(i, n);
+    }
+    FKD_DEV static int fold_as_written(int i, int n) {
         const int last = n - 1;
         if constexpr (BT == 1) {
             const int hi = i < last ? i : last;
