@@ -386,7 +386,7 @@ def main():
 TRAFFIC_C3_BYTES = 52058000
 TRAFFIC_C3_SOURCES = ("fusedkernellibrary_amd/csrc/fkd_kernels.hpp", "fusedkernellibrary_amd/csrc/fkd_launch.hpp",
                       "include/fkd/ops.hpp", "include/fkd/types.hpp")
-TRAFFIC_C3_SOURCES_SHA256 = "9dbd5965dcd4e5016b6575c398e291308713d9dff6254e6323de5078da10cbff"
+TRAFFIC_C3_SOURCES_SHA256 = "fd9332be9cee3417c98746d31234ced16c6c83a09100db06b25623bd32fb79b2"
 
 
 def device_sources_sha256():

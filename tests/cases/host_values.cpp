@@ -68,6 +68,26 @@ int main() {
     CHECK(with_alpha.x == 1 && with_alpha.w == 255);
     const uchar3 denorm = SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{-0.5f, 0.5f, 1.5f});
     CHECK(denorm.x == 0 && denorm.y == 127 && denorm.z == 255);
+    // ---- BorderReader's index folding: the division-free form used within one image size of the image gives what the
+    // reference's formulas give (FK/algorithms/image_processing/border_reader.h:177-327), for every extent up to 70 and every
+    // index from four extents below the image to five above (the formulas as written take over beyond one extent) ----
+    {
+        using fkd::Border; using fkd::Read2D; using fkd::u8;
+        int differing = 0;
+        for (int n = 1; n <= 70; ++n)
+            for (int i = -4 * n - 5; i <= 5 * n + 5; ++i) {
+                differing += Border<1, Read2D<u8>>::fold(i, n) != Border<1, Read2D<u8>>::fold_as_written(i, n);
+                differing += Border<2, Read2D<u8>>::fold(i, n) != Border<2, Read2D<u8>>::fold_as_written(i, n);
+                differing += Border<3, Read2D<u8>>::fold(i, n) != Border<3, Read2D<u8>>::fold_as_written(i, n);
+                differing += Border<4, Read2D<u8>>::fold(i, n) != Border<4, Read2D<u8>>::fold_as_written(i, n);
+            }
+        CHECK(differing == 0);
+        // and the patterns themselves on a 4-wide axis: aaa|abcd|ddd, cba|abcd|dcb, bcd|abcd|abc, dcb|abcd|cba
+        CHECK((Border<1, Read2D<u8>>::fold(-2, 4) == 0 && Border<1, Read2D<u8>>::fold(5, 4) == 3));
+        CHECK((Border<2, Read2D<u8>>::fold(-1, 4) == 0 && Border<2, Read2D<u8>>::fold(-3, 4) == 2 && Border<2, Read2D<u8>>::fold(4, 4) == 3 && Border<2, Read2D<u8>>::fold(6, 4) == 1));
+        CHECK((Border<3, Read2D<u8>>::fold(-1, 4) == 3 && Border<3, Read2D<u8>>::fold(-3, 4) == 1 && Border<3, Read2D<u8>>::fold(4, 4) == 0 && Border<3, Read2D<u8>>::fold(6, 4) == 2));
+        CHECK((Border<4, Read2D<u8>>::fold(-1, 4) == 1 && Border<4, Read2D<u8>>::fold(-3, 4) == 3 && Border<4, Read2D<u8>>::fold(4, 4) == 2 && Border<4, Read2D<u8>>::fold(6, 4) == 0));
+    }
     std::printf(failures ? "host values: %d check(s) failed\n" : "host values: all checks passed\n", failures);
     return failures ? 1 : 0;
 }
