@@ -80,6 +80,8 @@ template <class WP, class Plane, class V> __device__ __forceinline__ void masked
 
 // ---- the geometry a launcher hands to kernels that renumber their workgroups -------------------------------------
 
+// (A run-time compiled kernel takes a TileGeom whichever form its launch has.  A launch of the strip form of the bilinear
+// kernel has no tiles: its TileGeom has tiles_x == 0 and carries in n_tiles what strip_first_late_workgroup() says about it.)
 struct TileGeom {
     u32 tiles_x, tiles_y, n_tiles;
     // floor(2^32 / tiles_x) + 1 when (t * magic) >> 32 == t / tiles_x for every tile number t of a plane, else 0: the
@@ -604,6 +606,23 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
 // block is made (Chain::finalize_write, bit 0 of Params::reserved); launchers take the tile form when the bit is clear.
 // Taps come through a buffer resource whose extent ends with the image, so windows that reach past the last row read
 // zeros in bytes nobody uses and no lane needs a narrower access; the row is part of the lane's offset.
+// Wave priorities of the strip form.  A SIMD serves its oldest wave first, so in a launch that fits the chip in one round
+// (every workgroup resident from the start: configuration 3's 1 792) the seven waves of a SIMD do not advance side by side:
+// the wave that was started last is held back at every stage and ends up walking its steps nearly alone, each step exposed
+// to the full latency of its taps (measured with per-wave time stamps: the first wave of a SIMD issues its last stores 3.6 us
+// after the launch's first wave entered, the seventh 7.5 us).  Such a launch therefore starts every wave at priority 3 and
+// lowers it as the wave advances (2 from step 3, 1 from step 5), which makes the waves of a SIMD advance together; and
+// workgroups that were started late (the dispatcher hands consecutive workgroup numbers round the compute units, so a
+// workgroup's number divided by the number of compute units says roughly how many were on its unit before it) keep each
+// level one step longer, which is what keeps the last wave of a SIMD from finishing alone.  Configuration 3: 8.15 -> 7.85 us.
+// A launch of several rounds is left alone: the fresh waves of a later round would outrank the last steps of the round
+// before (twice the rows: 14.1 -> 15.4 us with the priorities on).  Priorities change the order of issue, never a result.
+// The launcher decides and hands the kernel one number: the number of the first workgroup that counts as started late, or
+// 0 for a launch whose waves keep the default priority.
+constexpr unsigned kStripOneRoundWorkgroups = 2048, kComputeUnits = 256, kStripLateWorkgroup = 4;
+inline u32 strip_first_late_workgroup(unsigned long long workgroups) {
+    return workgroups <= kStripOneRoundWorkgroups ? kStripLateWorkgroup * kComputeUnits : 0u;
+}
 constexpr int kStripRows = kGatherBY * FKD_GATHER_YI, kStripStep = 32, kStripMaxWidth = 256;
 constexpr int kStripThreads = kStripRows * kStripStep, kStripMaxSteps = kStripMaxWidth / kStripStep;
 static_assert(kStripThreads == kGatherBX * kGatherBY, "the two forms of the bilinear kernel share their workgroup shape");
@@ -624,7 +643,7 @@ template <class Chain> constexpr bool strip_capable() {
 }
 
 template <class Chain>
-__device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
+__device__ __forceinline__ void strip_body(const typename Chain::Params& p, const u32 first_late_workgroup) {
     using Root = ResizeRoot<typename Chain::Read>;
     using RZ = typename Root::Resize;
     using Back = typename RZ::BackOp;
@@ -637,17 +656,31 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
     constexpr u32 kClamped = 0x80000000u, kOutsideX = 0x40000000u;
 
     const int z = int(blockIdx.z);
+    // every wave starts at the highest priority, before its arguments are there: a launch of more than one round drops
+    // it again below, once they say so
+    __builtin_amdgcn_s_setprio(3);
     const typename RZ::Params* rp;
     if constexpr (Root::batched) rp = &p.read.plane[z]; else rp = &p.read;
     typename RZ::Params q = *rp;
     typename Chain::OpParams ops = p.ops;
     typename WP::Params wpar = W::plane_params(p.write, z);
+    u32 dims[4] = {p.active_w, p.active_h, first_late_workgroup, gridDim.x};
     detail::pin_scalars(q);
     detail::pin_scalars(ops);
     detail::pin_scalars(wpar);
-    u32 dims[2] = {p.active_w, p.active_h};
-    asm volatile("" : "+s"(dims[0]), "+s"(dims[1]));
+    // (the grid's width with the rest: fetched where it is used, it would be a second trip to the kernel-argument segment)
+    asm volatile("" : "+s"(dims[0]), "+s"(dims[1]), "+s"(dims[2]), "+s"(dims[3]));
     const int aw = int(dims[0]), ah = int(dims[1]);
+    // the steps at which this wave's priority falls to 2 and to 1, as two scalars (wave uniform)
+    int falls[2] = {3, 5};
+    if (dims[2] == 0u) {
+        __builtin_amdgcn_s_setprio(0);
+        falls[0] = falls[1] = kStripMaxSteps;                           // never
+    } else if (blockIdx.z * dims[3] + blockIdx.x >= dims[2]) {
+        falls[0] = 4;
+        falls[1] = 6;
+    }
+    asm volatile("" : "+s"(falls[0]), "+s"(falls[1]));
     int ox = 0, oy = 0;
     if constexpr (RZ::kAR != IGNORE_AR) { ox = q.x1; oy = q.y1; }
     const int sw = Back::width(q.back), sh = Back::height(q.back);
@@ -739,6 +772,9 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
         constexpr bool STATIC = decltype(static_tag)::value != 0;
         constexpr bool CLAMP = decltype(clamp_tag)::value != 0;
         auto produce = [&](int k, const StepTaps& s) {
+            // (k is known where the steps are written out: one comparison in four of the steps)
+            if ((k == 3 || k == 4) && k == falls[0]) __builtin_amdgcn_s_setprio(2);
+            if ((k == 5 || k == 6) && k == falls[1]) __builtin_amdgcn_s_setprio(1);
             // (the words are copied out first: a bit cast applied directly to an element of the vector reads element 0)
             const u32 ax_bits = s.e.x, bx_bits = s.e.y;
             const f32 ax = __builtin_bit_cast(f32, ax_bits), bx = __builtin_bit_cast(f32, bx_bits);
@@ -794,8 +830,8 @@ __device__ __forceinline__ void strip_body(const typename Chain::Params& p) {
 }
 
 template <class Chain>
-__global__ __launch_bounds__(kStripThreads) void k_strip(const typename Chain::Params p) {
-    if constexpr (strip_capable<Chain>()) strip_body<Chain>(p);
+__global__ __launch_bounds__(kStripThreads) void k_strip(const typename Chain::Params p, const u32 first_late_workgroup) {
+    if constexpr (strip_capable<Chain>()) strip_body<Chain>(p, first_late_workgroup);
 }
 
 template <class Chain, int XI, int YI>
@@ -892,7 +928,7 @@ template <class Chain> __device__ __forceinline__ void jit_body(const typename C
     if constexpr (IsDivergent<Chain>::value) DivergentBody<Chain>::run(p);
     else if constexpr (is_gather_chain<Chain>()) {
         if constexpr (strip_capable<Chain>()) {
-            if (g.tiles_x == 0u) { strip_body<Chain>(p); return; }      // wave uniform: the launcher chose the strip form
+            if (g.tiles_x == 0u) { strip_body<Chain>(p, g.n_tiles); return; }      // wave uniform: the launcher chose the strip form
         }
         gather_body<Chain, FKD_GATHER_XI, FKD_GATHER_YI>(p, g);
     }

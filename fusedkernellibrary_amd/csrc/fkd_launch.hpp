@@ -72,7 +72,7 @@ hipError_t launch_gather(const typename Chain::Params& p, hipStream_t stream, La
             if (info) *info = LaunchInfo{"strip", {grid.x, 1, grid.z}, {block.x, block.y, 1}, unsigned(kStripMaxWidth * 16 + (kStripThreads / 64) * 4)};
             if (grid.x == 0 || grid.z == 0) return hipSuccess;
             if (grid.z > 65535u) return hipErrorInvalidConfiguration;
-            return launch_by_pointer(&k_strip<Chain>, grid, block, stream, p);
+            return launch_by_pointer(&k_strip<Chain>, grid, block, stream, p, strip_first_late_workgroup((unsigned long long)grid.x * grid.z));
         }
     }
     TileGeom g;

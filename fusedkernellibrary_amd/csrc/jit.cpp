@@ -43,6 +43,9 @@ struct TileGeom {
     unsigned tiles_x, tiles_y, n_tiles, tiles_x_magic;
 };
 constexpr unsigned kRowsBandBlocks = 4096;     // as fkd::kRowsBandBlocks
+// As fkd::strip_first_late_workgroup: a strip launch that fits the chip in one round (at most 2048 workgroups) runs with
+// wave priorities and treats workgroups from number 4 * 256 on as started late; 0 leaves the priorities alone.
+unsigned strip_first_late_workgroup(unsigned long long workgroups) { return workgroups <= 2048u ? 1024u : 0u; }
 // As fkd::division_magic: floor(2^32 / d) + 1 when it divides every number below `limit` exactly, else 0.
 unsigned division_magic(unsigned d, unsigned limit) {
     if (d == 0) return 0;
@@ -215,12 +218,14 @@ int jit_launch(const void* ctx, const void* blob, size_t bytes, void* stream, fk
     unsigned grid[3], block[3] = {64, 4, 1};
     const char* kind = m.gather ? "gather_jit" : "rows_jit";
     if (m.gather && m.strip_width != 0 && active[0] != 0 && active[0] <= m.strip_width && (active[3] & 1u) != 0 && strip_enabled()) {
-        // strip form: one workgroup per m.by * m.yi output rows of a plane; the all-zero TileGeom tells the kernel
+        // strip form: one workgroup per m.by * m.yi output rows of a plane; tiles_x == 0 tells the kernel, and n_tiles
+        // carries the launch's priority schedule
         kind = "strip_jit";
         grid[0] = (active[1] + m.by * m.yi - 1) / (m.by * m.yi);
         grid[1] = 1;
         grid[2] = active[2];
         block[1] = m.by;
+        g.n_tiles = strip_first_late_workgroup((unsigned long long)grid[0] * grid[2]);
     } else if (m.gather) {
         const unsigned tw = 64 * m.xi, th = m.by * m.yi;
         g.tiles_x = (active[0] + tw - 1) / tw;

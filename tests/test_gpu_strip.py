@@ -174,3 +174,44 @@ def test_configuration_3_takes_the_strip_form(device):
         tiles = _c3(src, c["rects"], c["dst"], c["sub"], c["div"], device)
         assert last_launch()["kernel"] == "gather"
     assert got.tobytes() == tiles.tobytes()
+
+
+@pytest.mark.parametrize("rows", [256, 257, 448])
+def test_wave_priorities_follow_the_size_of_the_launch(device, rows):
+    """A strip launch of up to 2 048 workgroups (64 planes of 256 rows) runs its waves at priorities that fall as they
+    advance, with workgroups from number 1 024 on one step behind; a larger one (257 rows: 2 112 workgroups, 448 rows:
+    two full rounds) leaves the priorities alone.  Either way the result is the tile form's and the oracle's."""
+    import torch
+    c = wl.config3()
+    dst = (224, rows)
+    src = torch.from_numpy(c["src"]).to(device)
+    got = _c3(src, c["rects"], dst, c["sub"], c["div"], device)
+    ll = last_launch()
+    assert ll["kernel"] == "strip" and ll["grid"] == [(rows + 7) // 8, 1, 64]
+    with strip_switched(False):
+        tiles = _c3(src, c["rects"], dst, c["sub"], c["div"], device)
+        assert last_launch()["kernel"] == "gather"
+    assert got.tobytes() == tiles.tobytes()
+    assert got.tobytes() == ol.oracle_crop_resize_norm_split(c["src"], c["rects"], dst, c["sub"], c["div"]).tobytes()
+
+
+@pytest.mark.parametrize("rows", [16384, 16392])
+def test_wave_priorities_in_a_kernel_compiled_on_first_use(device, rows):
+    """One tall plane through the run-time compiled strip form: 2 048 workgroups (priorities on, the second half of the
+    workgroups counted as started late) and 2 049 (priorities off)."""
+    import torch
+    rng = np.random.RandomState(77)
+    w, h, cn = 160, 120, 4
+    img = rng.randint(0, 256, (h, w, cn)).astype(np.uint8)
+    src = torch.from_numpy(img).to(device)
+    dst, rect = (40, rows), (3, 2, 150, 117)
+    want = np.zeros((cn, dst[1], dst[0]), np.float32)
+    ol.execute([ol.read_2d(img, cn, crop=rect, resize=dst, ar=ol.IGNORE_AR)], [ol.op(ol.MUL, (0.5, 0.5, 0.5, 0.5))],
+               [ol.write(ol.TENSOR_SPLIT, want, cn, dst[0], dst[1], 1, cn)])
+    out = torch.full((cn, dst[1], dst[0]), -7.0, dtype=torch.float32, device=device)
+    cases.uncompiled_resize_split(1, src, rect, dst, 0.5, out)
+    torch.cuda.synchronize()
+    ll = last_launch()
+    assert ll["kernel"] == "strip_jit" and ll["grid"] == [(rows + 7) // 8, 1, 1]
+    assert out.cpu().numpy().tobytes() == want.tobytes()
+
