@@ -386,7 +386,7 @@ def main():
 TRAFFIC_C3_BYTES = 52066000
 TRAFFIC_C3_SOURCES = ("fusedkernellibrary_amd/csrc/fkd_kernels.hpp", "fusedkernellibrary_amd/csrc/fkd_launch.hpp",
                       "include/fkd/ops.hpp", "include/fkd/types.hpp")
-TRAFFIC_C3_SOURCES_SHA256 = "cd57a7dff842e9e13477de191519945032a110961e4bf83c7158b8cb303dbfe6"
+TRAFFIC_C3_SOURCES_SHA256 = "cfabe52f7411cdd9e6f736bdd19850672750c01d1842f4d718a51575ba54e545"
 
 
 def device_sources_sha256():

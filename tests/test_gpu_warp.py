@@ -45,6 +45,24 @@ def test_warp_float(device, matrix, persp):
     assert out.cpu().numpy().tobytes() == want.tobytes()
 
 
+def test_lanes_outside_the_source_ignore_what_their_stand_in_pixel_holds(device):
+    """A lane whose source point lies outside fetches pixel (0, 0) instead and drops it.  A float image may hold anything
+    there: the result is +0 all the same (integer images get there through weights of zero, float images must not)."""
+    import torch
+    img = (np.random.RandomState(16).rand(40, 48).astype(np.float32) * 10 - 5)
+    img[0, 0] = np.nan
+    img[0, 1] = np.inf
+    matrix = [[1, 0, 5], [0, 1, -3]]                       # rows 0-2 and the last five columns map outside; column 0 and 1 are never read
+    src = torch.from_numpy(img).to(device)
+    out = torch.full((40, 48), -1.0, dtype=torch.float32, device=device)
+    cases.warp(src, matrix, False, (48, 40), out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    want = ol.oracle_warp(img, 1, matrix, (48, 40), False)
+    assert np.isfinite(want).all() and (want[:3] == 0).all() and (want[:, 43:] == 0).all()
+    assert got.tobytes() == want.tobytes()
+
+
 @pytest.mark.parametrize("persp,dst", [(False, (2048, 2052)), (True, (2051, 2049)), (False, (1024, 3000))])
 def test_large_warps_run_their_workgroups_in_one_band_per_xcd(device, persp, dst):
     """Launches of 4 096 workgroups per plane or more take a one-dimensional grid whose workgroups the kernel renumbers
