@@ -386,7 +386,7 @@ def main():
 TRAFFIC_C3_BYTES = 52066000
 TRAFFIC_C3_SOURCES = ("fusedkernellibrary_amd/csrc/fkd_kernels.hpp", "fusedkernellibrary_amd/csrc/fkd_launch.hpp",
                       "include/fkd/ops.hpp", "include/fkd/types.hpp")
-TRAFFIC_C3_SOURCES_SHA256 = "cfabe52f7411cdd9e6f736bdd19850672750c01d1842f4d718a51575ba54e545"
+TRAFFIC_C3_SOURCES_SHA256 = "930697e25be5fa7204918c162c1474628745d51d3766a881ccb9ba5bcef06928"
 
 
 def device_sources_sha256():

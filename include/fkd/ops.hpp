@@ -2015,16 +2015,20 @@ template <int BT, class Back> struct Border {
     FKD_DEV static int height(const Params& p) { return Back::height(p.back); }
     FKD_DEV static int iabs(int v) { return v < 0 ? -v : v; }
     // n = extent along the axis (last index = n - 1)
+    // Within one image size of the image the reference's formulas below come to a single reflection or a single period,
+    // and no division is needed (a pad, a crop that leans over an edge): fold_near gives that value and clears `near` for
+    // an index further out, which takes the formulas as written.
+    FKD_DEV static int fold_near(int i, int n, bool& near) {
+        const int last = n - 1;
+        if constexpr (BT == 2) { near = near && i >= -n && i <= 2 * last + 1; return i < 0 ? -i - 1 : (i > last ? 2 * last - i + 1 : i); }
+        else if constexpr (BT == 3) { near = near && i >= -n && i < 2 * n; return i < 0 ? i + n : (i >= n ? i - n : i); }
+        else if constexpr (BT == 4) { near = near && i >= -last && i <= 2 * last; return i < 0 ? -i : (i > last ? 2 * last - i : i); }
+        else { return i < last ? (i > 0 ? i : 0) : last; }          // REPLICATE: the formula as written has no division
+    }
     FKD_DEV static int fold(int i, int n) {
-        // Within one image size of the image the reference's formulas below come to a single reflection or a single period,
-        // and no division is needed (a pad, a crop that leans over an edge); anything further out takes the formulas as written.
         if constexpr (BT >= 2) {
-            const int last = n - 1;
-            int near_value;
-            bool near;
-            if constexpr (BT == 2) { near_value = i < 0 ? -i - 1 : (i > last ? 2 * last - i + 1 : i); near = i >= -n && i <= 2 * last + 1; }
-            else if constexpr (BT == 3) { near_value = i < 0 ? i + n : (i >= n ? i - n : i); near = i >= -n && i < 2 * n; }
-            else { near_value = i < 0 ? -i : (i > last ? 2 * last - i : i); near = i >= -last && i <= 2 * last; }
+            bool near = true;
+            const int near_value = fold_near(i, n, near);
             if (near) return near_value;
         }
         return fold_as_written(i, n);
@@ -2068,6 +2072,34 @@ template <int BT, class Back> struct Border {
         } else {
             if (run_inside) { Back::template exec_row<V, kLaneMode>(x, fold(y, h), z, p.back, out); return; }
         }
+#if defined(FKD_DEVICE_CODE)
+        // A lane at the left or right edge: its elements come from wherever the border sends them, each as one access of
+        // whole dwords (an element of three bytes as one dword, where the byte behind it is still inside the image's
+        // allocation: everywhere but on the image's last rows), all of them requested before the first is taken apart.
+        // Row and columns are folded without a branch first; a lane that has one of them further out than an image size
+        // (no pad does) goes element by element.
+        if constexpr (BT != 0 && requires(typename Back::TapRow r) { Back::template tap_load<true>(r, 0, p.back); Back::tap_last(r); }) {
+            bool near = true;
+            const int fy = fold_near(y, h, near);
+            int fx[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) fx[i] = fold_near(x + i, w, near);
+            if (near) {
+                const auto row = Back::tap_row(0, fy, z, p.back);
+                typename Back::TapBits bits[V];
+                if (Back::tap_last(row)) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) bits[i] = Back::template tap_load<false>(row, fx[i], p.back);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) bits[i] = Back::template tap_load<true>(row, fx[i], p.back);
+                }
+#pragma unroll
+                for (int i = 0; i < V; ++i) out[i].v = Back::finish(Back::tap_value(bits[i]), p.back);
+                return;
+            }
+        }
+#endif
 #pragma unroll
         for (int i = 0; i < V; ++i) out[i].v = exec(x + i, y, z, p);
     }
