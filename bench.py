@@ -385,8 +385,8 @@ def main():
 # than a stale one.
 TRAFFIC_C3_BYTES = 52066000
 TRAFFIC_C3_SOURCES = ("fusedkernellibrary_amd/csrc/fkd_kernels.hpp", "fusedkernellibrary_amd/csrc/fkd_launch.hpp",
-                      "include/fkd/ops.hpp", "include/fkd/types.hpp")
-TRAFFIC_C3_SOURCES_SHA256 = "930697e25be5fa7204918c162c1474628745d51d3766a881ccb9ba5bcef06928"
+                      "include/fkd/ops.hpp", "include/fkd/types.hpp", "include/fkd/launch_info.hpp")
+TRAFFIC_C3_SOURCES_SHA256 = "ab66b4478c3be640393a47f96a0c8c6950e17c6b135baa9b819977413fdb49e2"
 
 
 def device_sources_sha256():

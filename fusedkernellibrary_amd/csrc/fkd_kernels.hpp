@@ -78,22 +78,8 @@ template <class WP, class Plane, class V> __device__ __forceinline__ void masked
     if constexpr (requires { WP::kLaneMasked; }) WP::put_masked(plane, row_off, lane_off, v);
 }
 
-// ---- the geometry a launcher hands to kernels that renumber their workgroups -------------------------------------
-
-// (A run-time compiled kernel takes a TileGeom whichever form its launch has.  A launch of the strip form of the bilinear
-// kernel has no tiles: its TileGeom has tiles_x == 0 and carries in n_tiles what strip_first_late_workgroup() says about it.)
-struct TileGeom {
-    u32 tiles_x, tiles_y, n_tiles;
-    // floor(2^32 / tiles_x) + 1 when (t * magic) >> 32 == t / tiles_x for every tile number t of a plane, else 0: the
-    // division then costs two scalar multiplications instead of a float reciprocal on the vector unit.
-    u32 tiles_x_magic;
-};
-// The magic for dividing numbers below `limit` by d, or 0 when there is none.
-inline u32 division_magic(u32 d, u32 limit) {
-    if (d == 0) return 0;
-    const unsigned long long m = (1ull << 32) / d + 1;        // m * d - 2^32 is in (0, d]; exact while n * d < 2^32
-    return (m < (1ull << 32) && (unsigned long long)limit * d < (1ull << 32)) ? u32(m) : 0u;
-}
+// (The geometry a launcher hands to kernels that renumber their workgroups -- TileGeom, division_magic, the limits that
+// choose a form of grid -- is in fkd/launch_info.hpp, which the launchers of run-time compiled kernels share.)
 
 // ---- rows kernel ---------------------------------------------------------------------------------------
 
@@ -153,9 +139,8 @@ template <class Chain> constexpr bool rows_in_bands() {
 // workgroups in plain row-major order a warp fetched its source 2.5 to 3.2 times, once into nearly every L2; in bands it
 // is fetched once (rocprofv3 FETCH_SIZE), and a 3840 x 2160 warp takes 25.1 instead of 30.8 us.  Launches of fewer than
 // kRowsBandBlocks blocks per plane keep the two-dimensional grid: their source comes out of the last-level cache either
-// way, and the 1080p warp measured 5 % slower in bands (9.27 against 8.83 us).
-inline constexpr u32 rows_band_chunk(u32 blocks) { return (blocks + 7u) / 8u; }
-constexpr u32 kRowsBandBlocks = 4096;
+// way, and the 1080p warp measured 5 % slower in bands (9.27 against 8.83 us).  (rows_band_chunk and kRowsBandBlocks:
+// fkd/launch_info.hpp.)
 
 // `kernarg_offset`: where p sits inside the kernel-argument segment (0 when the chain's parameter block is the
 // kernel's first argument); long chains fetch their operations' parameters from there.  BANDS: the launch has the bands
@@ -619,10 +604,7 @@ __device__ __forceinline__ void gather_body(const typename Chain::Params& p, con
 // before (twice the rows: 14.1 -> 15.4 us with the priorities on).  Priorities change the order of issue, never a result.
 // The launcher decides and hands the kernel one number: the number of the first workgroup that counts as started late, or
 // 0 for a launch whose waves keep the default priority.
-constexpr unsigned kStripOneRoundWorkgroups = 2048, kComputeUnits = 256, kStripLateWorkgroup = 4;
-inline u32 strip_first_late_workgroup(unsigned long long workgroups) {
-    return workgroups <= kStripOneRoundWorkgroups ? kStripLateWorkgroup * kComputeUnits : 0u;
-}
+// (strip_first_late_workgroup, fkd/launch_info.hpp)
 constexpr int kStripRows = kGatherBY * FKD_GATHER_YI, kStripStep = 32, kStripMaxWidth = 256;
 constexpr int kStripThreads = kStripRows * kStripStep, kStripMaxSteps = kStripMaxWidth / kStripStep;
 static_assert(kStripThreads == kGatherBX * kGatherBY, "the two forms of the bilinear kernel share their workgroup shape");
@@ -906,15 +888,7 @@ template <class D> __global__ __launch_bounds__(kRowsBX * kRowsBY) void k_diverg
 
 // The one kernel of a chain compiled at run time, and what its launcher needs to know about it.  A launcher that
 // only has the parameter block as bytes reads the active grid from its first three words.
-struct JitMeta {
-    u32 gather;          // 1: gather kernel geometry, 0: rows kernel geometry
-    u32 params_bytes;    // sizeof(Chain::Params)
-    u32 v, rows;         // rows kernel: elements per thread along x, rows per thread
-    u32 xi, yi, by;      // gather kernel: pixels per lane along x, rows per wave, waves per workgroup
-    u32 max_planes;      // most planes (grid z) a launch may have, 0: no limit of the kernel's own
-    u32 strip_width;     // gather kernel: outputs up to this width are launched in strip form (TileGeom all zero), 0: never
-    u32 bands;           // rows kernel: 1 when launches of kRowsBandBlocks blocks per plane or more take the bands form of grid
-};
+// (JitMeta: fkd/launch_info.hpp)
 template <class Chain> constexpr JitMeta jit_meta() {
     if constexpr (IsDivergent<Chain>::value)
         return JitMeta{0u, u32(sizeof(typename Chain::Params)), u32(RowsConfig<Chain>::V), u32(RowsConfig<Chain>::ROWS), 0u, 0u, 0u, u32(Chain::kMaxPlanes), 0u, 0u};

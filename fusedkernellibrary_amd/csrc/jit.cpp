@@ -35,23 +35,12 @@
 namespace fklhip {
 namespace {
 
-// Mirrors of fkd::JitMeta and fkd::TileGeom (csrc/fkd_kernels.hpp): ten and four 32-bit words.
-struct JitMeta {
-    unsigned gather, params_bytes, v, rows, xi, yi, by, max_planes, strip_width, bands;
-};
-struct TileGeom {
-    unsigned tiles_x, tiles_y, n_tiles, tiles_x_magic;
-};
-constexpr unsigned kRowsBandBlocks = 4096;     // as fkd::kRowsBandBlocks
-// As fkd::strip_first_late_workgroup: a strip launch that fits the chip in one round (at most 2048 workgroups) runs with
-// wave priorities and treats workgroups from number 4 * 256 on as started late; 0 leaves the priorities alone.
-unsigned strip_first_late_workgroup(unsigned long long workgroups) { return workgroups <= 2048u ? 1024u : 0u; }
-// As fkd::division_magic: floor(2^32 / d) + 1 when it divides every number below `limit` exactly, else 0.
-unsigned division_magic(unsigned d, unsigned limit) {
-    if (d == 0) return 0;
-    const unsigned long long m = (1ull << 32) / d + 1;
-    return (m < (1ull << 32) && (unsigned long long)limit * d < (1ull << 32)) ? unsigned(m) : 0u;
-}
+// The launch geometry and the description of a compiled kernel are the kernels' own (fkd/launch_info.hpp).
+using fkd::JitMeta;
+using fkd::TileGeom;
+using fkd::division_magic;
+using fkd::kRowsBandBlocks;
+using fkd::strip_first_late_workgroup;
 
 struct JitKernel {
     std::string signature;
