@@ -44,12 +44,19 @@ template <class DPP, class StreamT> struct Chains {
         default: return 2;
         }
     }
-    // elem: 0 uchar3 images (value = 3 bytes), 1 float images (value = 1 float)
+    // elem: 0 uchar3 images (value = 3 bytes), 1 float images (value = 1 float), 2 uchar4, 3 ushort3, 4 uchar, 5 float3
     static int pad(StreamT& s, MemType mem, int elem, int border_type, const void* src, int w, int h, int pitch, int left, int top,
                    int out_w, int out_h, const float* value, void* out, int out_pitch) {
         if (elem == 0) return pad_t<uchar3>(s, mem, border_type, src, w, h, pitch, left, top, out_w, out_h,
                                             make_<uchar3>(uchar(value[0]), uchar(value[1]), uchar(value[2])), out, out_pitch);
         if (elem == 1) return pad_t<float>(s, mem, border_type, src, w, h, pitch, left, top, out_w, out_h, value[0], out, out_pitch);
+        if (elem == 2) return pad_t<uchar4>(s, mem, border_type, src, w, h, pitch, left, top, out_w, out_h,
+                                            make_<uchar4>(uchar(value[0]), uchar(value[1]), uchar(value[2]), uchar(value[3])), out, out_pitch);
+        if (elem == 3) return pad_t<ushort3>(s, mem, border_type, src, w, h, pitch, left, top, out_w, out_h,
+                                             make_<ushort3>(ushort(value[0]), ushort(value[1]), ushort(value[2])), out, out_pitch);
+        if (elem == 4) return pad_t<uchar>(s, mem, border_type, src, w, h, pitch, left, top, out_w, out_h, uchar(value[0]), out, out_pitch);
+        if (elem == 5) return pad_t<float3>(s, mem, border_type, src, w, h, pitch, left, top, out_w, out_h,
+                                            make_<float3>(value[0], value[1], value[2]), out, out_pitch);
         return 2;
     }
 };

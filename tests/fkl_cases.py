@@ -334,11 +334,14 @@ def dual(which, a_bytes, b_bytes, width, height, out_bytes):
                              _p(out_bytes), _pitch(out_bytes)))
 
 
-def pad(src, border_type, left, top, out, value=(0, 0, 0)):
-    """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out."""
+def pad(src, border_type, left, top, out, value=(0, 0, 0), kind=None):
+    """src (H,W,3) u8 or (H,W) f32 cuda -> BorderReader<border_type> -> Crop starting `left`/`top` pixels before the origin -> out.
+    `kind`: the element number of border_chains.h for other pixel types (uint16 images travel as int16 tensors)."""
     v = np.zeros(4, np.float32)
     v[: len(value)] = value
-    _ok(cases().fklcase_pad(_stream(), 0 if src.element_size() == 1 else 1, int(border_type), _p(src), src.shape[1], src.shape[0], _pitch(src),
+    if kind is None:
+        kind = 0 if src.element_size() == 1 else 1
+    _ok(cases().fklcase_pad(_stream(), int(kind), int(border_type), _p(src), src.shape[1], src.shape[0], _pitch(src),
                             int(left), int(top), out.shape[1], out.shape[0], v.ctypes.data_as(C.c_void_p), _p(out), _pitch(out)))
 
 

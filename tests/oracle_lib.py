@@ -822,9 +822,14 @@ def ref_circular_transposed(batch, oldest_first, images, fill):
 BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
 
 
+def pad_kind(dtype, cn):
+    """The element number of tests/cases/border_chains.h for images of `cn` channels of `dtype`."""
+    return {("uint8", 3): 0, ("float32", 1): 1, ("uint8", 4): 2, ("uint16", 3): 3, ("uint8", 1): 4, ("float32", 3): 5}[(np.dtype(dtype).name, cn)]
+
+
 def oracle_pad(src, border_type, left, top, out_w, out_h, value=(0, 0, 0)):
-    """src (H,W,3) uint8 or (H,W) float32; the output grid starts `left`/`top` pixels before the image origin."""
-    cn = 3 if src.ndim == 3 else 1
+    """src (H,W,cn) or (H,W) of uint8, uint16 or float32; the output grid starts `left`/`top` pixels before the image origin."""
+    cn = src.shape[2] if src.ndim == 3 else 1
     out = np.zeros((out_h, out_w, cn) if cn > 1 else (out_h, out_w), src.dtype)
     r = read_2d(src, cn, crop=(-left, -top, out_w, out_h))
     r.border = 1 + border_type
@@ -835,11 +840,11 @@ def oracle_pad(src, border_type, left, top, out_w, out_h, value=(0, 0, 0)):
 
 
 def ref_pad(src, border_type, left, top, out_w, out_h, value=(0, 0, 0)):
-    cn = 3 if src.ndim == 3 else 1
+    cn = src.shape[2] if src.ndim == 3 else 1
     out = np.zeros((out_h, out_w, cn) if cn > 1 else (out_h, out_w), src.dtype)
     v = np.zeros(4, np.float32)
     v[: len(value)] = value
-    rc = ref().fklref_pad(0 if src.dtype == np.uint8 else 1, int(border_type), C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0],
+    rc = ref().fklref_pad(pad_kind(src.dtype, cn), int(border_type), C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0],
                           int(left), int(top), int(out_w), int(out_h), _f32p(v), C.c_void_p(_ptr(out)), out.strides[0])
     assert rc == 0, rc
     return out

@@ -34,3 +34,25 @@ def test_pad_float(device, bt):
         cases.pad(src, bt, left, top, out, value=(-1.5,))
         torch.cuda.synchronize()
         assert out.cpu().numpy().tobytes() == ol.oracle_pad(img, bt, left, top, ow, oh, value=(-1.5,)).tobytes(), (left, top, ow, oh)
+
+
+
+@pytest.mark.parametrize("dtype,cn", [(np.uint8, 4), (np.uint16, 3), (np.uint8, 1), (np.float32, 3)])
+@pytest.mark.parametrize("bt", [ol.BORDER_CONSTANT, ol.BORDER_REPLICATE, ol.BORDER_WRAP, ol.BORDER_REFLECT_101])
+def test_pad_other_pixel_types(device, bt, dtype, cn):
+    """Pixels of 4, 6, 1 and 12 bytes: a lane on the left or right edge fetches each pixel as one access of whole dwords where
+    the bytes behind the pixel are still inside the image (6-byte pixels: two bytes behind), element by element on the
+    image's last rows; the second pad reaches further out than an image size, where indices are folded with divisions."""
+    import torch
+    rng = np.random.default_rng(23)
+    shape = (45, 67, cn) if cn > 1 else (45, 67)
+    img = (rng.random(shape, dtype=np.float32) * 100 - 50) if dtype == np.float32 else rng.integers(0, 1000 if dtype == np.uint16 else 256, shape).astype(dtype)
+    src = torch.from_numpy(img.view(np.int16) if dtype == np.uint16 else img).to(device)
+    h, w = img.shape[:2]
+    value = (9, 8, 7, 6)[:cn]
+    for (left, top, ow, oh) in ((6, 5, w + 13, h + 9), (3 * w + 2, 2 * h + 1, 5 * w, 4 * h)):
+        out = torch.zeros((oh, ow, cn) if cn > 1 else (oh, ow), dtype=src.dtype, device=device)
+        cases.pad(src, bt, left, top, out, value=value, kind=ol.pad_kind(dtype, cn))
+        torch.cuda.synchronize()
+        want = ol.oracle_pad(img, bt, left, top, ow, oh, value=value)
+        assert out.cpu().numpy().tobytes() == want.tobytes(), (left, top, ow, oh)

@@ -14,7 +14,9 @@ NUMPY_MODE = {ol.BORDER_CONSTANT: "constant", ol.BORDER_REPLICATE: "edge", ol.BO
 
 def images():
     r = np.random.default_rng(11)
-    return [r.integers(0, 256, (9, 14, 3), dtype=np.uint8), (r.random((7, 5), dtype=np.float32) * 50 - 25).astype(np.float32)]
+    return [r.integers(0, 256, (9, 14, 3), dtype=np.uint8), (r.random((7, 5), dtype=np.float32) * 50 - 25).astype(np.float32),
+            r.integers(0, 256, (6, 11, 4), dtype=np.uint8), r.integers(0, 1000, (8, 7, 3)).astype(np.uint16),
+            r.integers(0, 256, (5, 9), dtype=np.uint8), (r.random((6, 8, 3), dtype=np.float32) * 50 - 25).astype(np.float32)]
 
 
 @pytest.mark.parametrize("bt", sorted(NUMPY_MODE))
@@ -25,7 +27,7 @@ def test_padding_within_one_image_size_is_numpy_pad(bt):
             pads = ((top, bottom), (left, right)) + (((0, 0),) if img.ndim == 3 else ())
             kw = {"constant_values": 7} if bt == ol.BORDER_CONSTANT else {}
             want = np.pad(img, pads, mode=NUMPY_MODE[bt], **kw)
-            got = ol.oracle_pad(img, bt, left, top, w + left + right, h + top + bottom, value=(7, 7, 7))
+            got = ol.oracle_pad(img, bt, left, top, w + left + right, h + top + bottom, value=(7, 7, 7, 7))
             assert got.tobytes() == want.tobytes(), (bt, left, top, right, bottom)
 
 
@@ -41,6 +43,6 @@ def test_padding_matches_reference_backend(bt):
     for img in images():
         h, w = img.shape[:2]
         for (left, top, ow, oh) in ((3, 2, w + 7, h + 3), (2 * w + 3, 3 * h + 1, 5 * w + 2, 7 * h), (-1, -2, 4, 3), (w, h, 3 * w, 3 * h)):
-            a = ol.oracle_pad(img, bt, left, top, ow, oh, value=(9, 8, 7))
-            b = ol.ref_pad(img, bt, left, top, ow, oh, value=(9, 8, 7))
+            a = ol.oracle_pad(img, bt, left, top, ow, oh, value=(9, 8, 7, 6))
+            b = ol.ref_pad(img, bt, left, top, ow, oh, value=(9, 8, 7, 6))
             assert a.tobytes() == b.tobytes(), (bt, left, top, ow, oh)
