@@ -159,6 +159,22 @@ int warp_u8x3(const uint8_t* src, int w, int h, int pitch, const float* m, int d
     return 0;
 }
 
+template <WarpType WT, class T, class O>
+int warp_any(const void* src, int w, int h, int pitch, const float* m, int dw, int dh, float* out) {
+    CpuStream stream;
+    const auto in = wrap2d<T>(src, w, h, pitch);
+    Ptr2D<O> o(reinterpret_cast<O*>(out), uint(dw), uint(dh), uint(dw) * uint(sizeof(O)), MemType::Host, 0);
+    WarpingParameters<WT> params{};
+    constexpr int rows = WT == WarpType::Affine ? 2 : 3;
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < 3; ++c) params.transformMatrix.data[r][c] = m[r * 3 + c];
+    params.dstSize = Size(dw, dh);
+    executeOperations<CpuDPP>(stream, PerThreadRead<ND::_2D, T>::build(in.ptr()).then(Warping<WT>::build(params)),
+                              PerThreadWrite<ND::_2D, O>::build(o.ptr()));
+    stream.sync();
+    return 0;
+}
+
 // Benchmark configuration 4: B independent uchar3 images, per-image Mul and Add fused into each plane's
 // read, SaturateCast, B separate outputs in one launch.
 template <size_t B>
@@ -256,6 +272,18 @@ int fklref_batch_default_cast_mul_b4(const uint8_t* const* srcs, int w, int h, i
 int fklref_warp_u8x3(const uint8_t* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh, float* out) {
     return perspective ? warp_u8x3<WarpType::Perspective>(src, w, h, pitch, m, dw, dh, out)
                        : warp_u8x3<WarpType::Affine>(src, w, h, pitch, m, dw, dh, out);
+}
+// The same for other pixel types: kind 2 uchar4 -> float4, 3 ushort3 -> float3, 4 uchar -> float (tight float output).
+int fklref_warp_kind(int kind, const void* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh, float* out) {
+    auto run = [&](auto in_tag, auto out_tag) {
+        using T = decltype(in_tag); using O = decltype(out_tag);
+        return perspective ? warp_any<WarpType::Perspective, T, O>(src, w, h, pitch, m, dw, dh, out)
+                           : warp_any<WarpType::Affine, T, O>(src, w, h, pitch, m, dw, dh, out);
+    };
+    if (kind == 2) return run(uchar4{}, float4{});
+    if (kind == 3) return run(ushort3{}, float3{});
+    if (kind == 4) return run(uchar{}, float{});
+    return 2;
 }
 
 // Deinterlace of a uchar3 image into a float3 image: mode 1 BLEND, 2 INTER_LINEAR keeping even lines, 3 keeping odd.

@@ -496,6 +496,24 @@ int fklcase_warp_f32(void* stream, const float* src, int w, int h, int pitch, co
     });
 }
 
+// Other pixel types (compiled on first use): kind 2 uchar4 -> float4, 3 ushort3 -> float3, 4 uchar -> float.
+int fklcase_warp_kind(void* stream, int kind, const void* src, int w, int h, int pitch, const float* m, int perspective, int dw, int dh,
+                      float* out, int out_pitch) {
+    int rc = 0;
+    const int g = guarded([&] {
+        auto run = [&](auto in_tag, auto out_tag) {
+            using T = decltype(in_tag); using O = decltype(out_tag);
+            if (perspective) warp_image<WarpType::Perspective, T, O>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
+            else warp_image<WarpType::Affine, T, O>(stream, src, w, h, pitch, m, dw, dh, out, out_pitch);
+        };
+        if (kind == 2) run(uchar4{}, float4{});
+        else if (kind == 3) run(ushort3{}, float3{});
+        else if (kind == 4) run(uchar{}, float{});
+        else rc = 2;
+    });
+    return g ? g : rc;
+}
+
 int fklcase_deinterlace_u8x3(void* stream, const uint8_t* src, int w, int h, int pitch, int mode, float* out, int out_pitch) {
     return guarded([&] { deinterlace_image<uchar3, float3>(stream, src, w, h, pitch, mode, out, out_pitch); });
 }

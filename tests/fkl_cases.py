@@ -235,10 +235,15 @@ def uncompiled_float4_resize(src, dst, out):
                                                  _p(out), out.stride(0) * 4))
 
 
-def warp(src, matrix, perspective, dst, out):
-    """src (H,W,3) u8 or (H,W) f32 cuda; matrix 2x3 (affine) or 3x3 (perspective); out (dh,dw,3) / (dh,dw) f32 cuda."""
+def warp(src, matrix, perspective, dst, out, kind=None):
+    """src (H,W,3) u8 or (H,W) f32 cuda; matrix 2x3 (affine) or 3x3 (perspective); out (dh,dw,3) / (dh,dw) f32 cuda.
+    `kind`: 2 (H,W,4) u8, 3 (H,W,3) u16 travelling as int16, 4 (H,W) u8 -- chains compiled on first use."""
     m = np.zeros(9, np.float32)
     m[: (9 if perspective else 6)] = np.asarray(matrix, np.float32).ravel()
+    if kind is not None:
+        _ok(cases().fklcase_warp_kind(_stream(), int(kind), _p(src), src.shape[1], src.shape[0], src.stride(0) * src.element_size(),
+                                      m.ctypes.data_as(C.c_void_p), int(bool(perspective)), int(dst[0]), int(dst[1]), _p(out), out.stride(0) * 4))
+        return
     is_u8 = src.element_size() == 1
     fn = cases().fklcase_warp_u8x3 if is_u8 else cases().fklcase_warp_f32
     esz = 1 if is_u8 else 4

@@ -369,6 +369,24 @@ def ref_warp_u8x3(src, matrix, dst, perspective):
     return out
 
 
+def warp_kind(dtype, cn):
+    """The pixel-type number of fklref_warp_kind / fklcase_warp_kind."""
+    return {("uint8", 4): 2, ("uint16", 3): 3, ("uint8", 1): 4}[(np.dtype(dtype).name, cn)]
+
+
+def ref_warp(src, matrix, dst, perspective):
+    """As ref_warp_u8x3 for (H,W,4) uint8, (H,W,3) uint16 and (H,W) uint8 images."""
+    cn = src.shape[2] if src.ndim == 3 else 1
+    dw, dh = dst
+    out = np.zeros((dh, dw, cn) if cn > 1 else (dh, dw), np.float32)
+    m = np.zeros(9, np.float32)
+    m[: (9 if perspective else 6)] = np.asarray(matrix, np.float32).ravel()
+    rc = ref().fklref_warp_kind(warp_kind(src.dtype, cn), C.c_void_p(_ptr(src)), src.shape[1], src.shape[0], src.strides[0], _f32p(m),
+                                int(bool(perspective)), dw, dh, C.c_void_p(_ptr(out)))
+    assert rc == 0
+    return out
+
+
 DEINTERLACE_BLEND, DEINTERLACE_LINEAR_EVEN, DEINTERLACE_LINEAR_ODD = 1, 2, 3
 
 

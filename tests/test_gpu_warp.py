@@ -45,6 +45,24 @@ def test_warp_float(device, matrix, persp):
     assert out.cpu().numpy().tobytes() == want.tobytes()
 
 
+@pytest.mark.parametrize("dtype,cn", [(np.uint8, 4), (np.uint16, 3), (np.uint8, 1)])
+@pytest.mark.parametrize("matrix,persp", [(AFFINE, False), (SHIFT_OUT, False), (PERSPECTIVE, True)])
+def test_warp_other_pixel_types(device, matrix, persp, dtype, cn):
+    """Pixels of 4, 6 and 1 bytes (chains compiled on first use): the tap windows, the duplicate of the edge tap and the
+    zero weights of lanes outside are per element size."""
+    import torch
+    rng = np.random.RandomState(25)
+    shape = (90, 131, cn) if cn > 1 else (90, 131)
+    img = rng.randint(0, 1000 if dtype == np.uint16 else 256, shape).astype(dtype)
+    src = torch.from_numpy(img.view(np.int16) if dtype == np.uint16 else img).to(device)
+    for dst in ((100, 70), (131, 90), (9, 5)):
+        out = torch.full((dst[1], dst[0], cn) if cn > 1 else (dst[1], dst[0]), -1.0, dtype=torch.float32, device=device)
+        cases.warp(src, matrix, persp, dst, out, kind=ol.warp_kind(dtype, cn))
+        torch.cuda.synchronize()
+        want = ol.oracle_warp(img, cn, matrix, dst, persp)
+        assert out.cpu().numpy().tobytes() == want.tobytes(), dst
+
+
 def test_lanes_outside_the_source_ignore_what_their_stand_in_pixel_holds(device):
     """A lane whose source point lies outside fetches pixel (0, 0) instead and drops it.  A float image may hold anything
     there: the result is +0 all the same (integer images get there through weights of zero, float images must not)."""

@@ -392,6 +392,22 @@ def test_warp_matches_reference_backend():
         assert a.tobytes() == b.tobytes()
 
 
+@pytest.mark.skipif(not ol.have_ref(), reason="reference CPU backend not built (needs the reference tree)")
+@pytest.mark.parametrize("dtype,cn", [(np.uint8, 4), (np.uint16, 3), (np.uint8, 1)])
+def test_warp_of_other_pixel_types_matches_reference_backend(dtype, cn):
+    import math
+    rng = np.random.RandomState(9)
+    shape = (50, 71, cn) if cn > 1 else (50, 71)
+    src = rng.randint(0, 1000 if dtype == np.uint16 else 256, shape).astype(dtype)
+    th = math.radians(-11)
+    affine = [[0.8 * math.cos(th), -0.8 * math.sin(th), -6.5], [0.8 * math.sin(th), 0.8 * math.cos(th), 9.25]]
+    persp = [[1.1, 0.05, -3.0], [0.02, 0.9, 4.0], [0.0008, -0.0005, 1.0]]
+    for matrix, p, dst in ((affine, False, (90, 60)), (persp, True, (80, 64)), ([[1, 0, 40], [0, 1, 0]], False, (71, 50))):
+        a = ol.oracle_warp(src, cn, matrix, dst, p)
+        b = ol.ref_warp(src, matrix, dst, p)
+        assert a.tobytes() == b.tobytes()
+
+
 def test_warp_closed_forms():
     """Identity warp returns float(source); an integer shift returns the shifted source and zeros outside."""
     rng = np.random.RandomState(8)
