@@ -386,7 +386,7 @@ def main():
 TRAFFIC_C3_BYTES = 52066000
 TRAFFIC_C3_SOURCES = ("fusedkernellibrary_amd/csrc/fkd_kernels.hpp", "fusedkernellibrary_amd/csrc/fkd_launch.hpp",
                       "include/fkd/ops.hpp", "include/fkd/types.hpp", "include/fkd/launch_info.hpp")
-TRAFFIC_C3_SOURCES_SHA256 = "ab66b4478c3be640393a47f96a0c8c6950e17c6b135baa9b819977413fdb49e2"
+TRAFFIC_C3_SOURCES_SHA256 = "89f542a2e77568a8a23247e74374aaaafbd2c26b093af28469f2c0811798663c"
 
 
 def device_sources_sha256():
